@@ -1,0 +1,196 @@
+// extern "C" surface of librpa_hip.so: argument checking, kernel selection, launches.
+#include <atomic>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "rpa_common.h"
+
+namespace rpa {
+int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_t*, void*, int, int, int64_t, int,
+                          int64_t, int);
+int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
+                          const int32_t*, const int32_t*, int, int, int, int, int, int, int, int);
+}  // namespace rpa
+
+namespace {
+
+thread_local char g_err[512] = "";
+std::atomic<int> g_decode_chunk{512};
+std::atomic<int> g_max_splits{32};
+std::atomic<int> g_force_generic{0};
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(int err, const char* what) {
+  if (err == 0) return 0;
+  return fail(err, "%s: %s", what, hipGetErrorString((hipError_t)err));
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// Split-K partial storage per split: outputs [T][Hq][D] f32, then (max, sum) [T][Hq][2] f32.
+size_t part_o_bytes(int T, int Hq, int D) { return align256((size_t)T * Hq * D * 4); }
+size_t part_ml_bytes(int T, int Hq) { return align256((size_t)T * Hq * 2 * 4); }
+
+int static_splits(int M, int page_size) {
+  const int chunk = g_decode_chunk.load();
+  long span = (long)M * page_size;
+  long n = (span + chunk - 1) / chunk;
+  const int cap = g_max_splits.load();
+  if (n > cap) n = cap;
+  if (n < 1) n = 1;
+  return (int)n;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* rpa_version(void) { return "0.1.0"; }
+
+const char* rpa_last_error(void) { return g_err; }
+
+int rpa_set_tunable(const char* name, int value) {
+  if (!name) return -1;
+  if (!strcmp(name, "decode_chunk")) {
+    if (value < 64) value = 64;
+    value = (value + 63) & ~63;
+    return g_decode_chunk.exchange(value);
+  }
+  if (!strcmp(name, "max_splits")) {
+    if (value < 1) value = 1;
+    if (value > rpa::kMaxSplitsCap) value = rpa::kMaxSplitsCap;
+    return g_max_splits.exchange(value);
+  }
+  if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
+  return -1;
+}
+
+int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32_t* slice_indices,
+                            const int32_t* num_slices, void* kv_pages, int T, int N, int64_t num_positions,
+                            int page_size, int64_t row_bytes, int page_shard_index) {
+  if (T < 0 || N < 0 || num_positions < 0 || page_size <= 0 || row_bytes <= 0 || page_shard_index < 0)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_slices: bad size (T=%d N=%d positions=%lld page_size=%d row_bytes=%lld shard=%d)",
+                T, N, (long long)num_positions, page_size, (long long)row_bytes, page_shard_index);
+  if (T == 0 || N == 0 || num_positions == 0) return RPA_OK;  // nothing to move (the reference returns the cache unchanged)
+  if (!new_kv || !slice_indices || !num_slices || !kv_pages)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_slices: null pointer");
+  return hip_fail(rpa::launch_scatter_slices((hipStream_t)stream, new_kv, slice_indices, num_slices, kv_pages, T, N,
+                                             num_positions, page_size, row_bytes, page_shard_index),
+                  "rpa_page_scatter_slices launch");
+}
+
+int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
+                            const int32_t* context_lens, const int32_t* block_tables,
+                            const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M, int P,
+                            int page_size, int Hkv, int D, int C, int elem_bytes) {
+  if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hkv <= 0 || D <= 0 || C < 2 * Hkv ||
+      (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4))
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged: bad size (T=%d S=%d M=%d P=%d page_size=%d Hkv=%d D=%d C=%d elem=%d)",
+                T, S, M, P, page_size, Hkv, D, C, elem_bytes);
+  if (T == 0) return RPA_OK;
+  if (!key || !value || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged: null pointer");
+  return hip_fail(rpa::launch_scatter_ragged((hipStream_t)stream, key, value, kv_pages, context_lens, block_tables,
+                                             query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C, elem_bytes),
+                  "rpa_page_scatter_ragged launch");
+}
+
+size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int q_dtype,
+                                     int kv_dtype) {
+  (void)S; (void)Hkv; (void)q_dtype; (void)kv_dtype;
+  if (T <= 0 || M <= 0 || page_size <= 0 || Hq <= 0 || D <= 0) return 256;
+  const int splits = static_splits(M, page_size);
+  return (size_t)splits * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) + 256;
+}
+
+int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages, const float* kv_scales,
+                               const int32_t* context_lens, const int32_t* block_tables,
+                               const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
+                               size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv,
+                               int D, int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
+                               float logits_soft_cap) {
+  if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: bad size (T=%d S=%d M=%d P=%d page_size=%d Hq=%d Hkv=%d D=%d)",
+                T, S, M, P, page_size, Hq, Hkv, D);
+  if (Hq % Hkv != 0) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  if (C < 2 * Hkv) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: C=%d combined heads < 2*Hkv=%d", C, 2 * Hkv);
+  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: q_dtype %d (want f32 or bf16)", q_dtype);
+  if (kv_dtype < RPA_F32 || kv_dtype > RPA_INT8) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: kv_dtype %d", kv_dtype);
+  if (D > 256 || D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: head_dim %d (want a multiple of 4, <= 256)", D);
+  if ((kv_dtype == RPA_FP8_E4M3 || kv_dtype == RPA_INT8) && !kv_scales)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: 8-bit KV pages need kv_scales");
+  if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: softmax_scale is not finite");
+  if (T == 0) return RPA_OK;
+  if (!q || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs || !out)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: null pointer");
+
+  rpa::AttnParams p;
+  memset(&p, 0, sizeof(p));
+  p.q = q; p.kv_pages = kv_pages; p.kv_scales = kv_scales;
+  p.context_lens = context_lens; p.block_tables = block_tables; p.qsl = query_start_loc; p.num_seqs = num_seqs;
+  p.out = out;
+  p.T = T; p.S = S; p.M = M; p.P = P; p.page_size = page_size; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv; p.D = D; p.C = C;
+  p.token_stride = (int64_t)C * D * rpa::elem_bytes(kv_dtype);
+  p.page_stride = p.token_stride * page_size;
+  p.q_dtype = q_dtype; p.kv_dtype = kv_dtype;
+  p.scale = softmax_scale;
+  p.scale_log2 = softmax_scale * 1.4426950408889634f;
+  p.window = sliding_window > 0 ? sliding_window : 0;
+  p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
+  p.chunk_target = g_decode_chunk.load();
+  p.max_splits = 1;
+  p.mfma_path = (!g_force_generic.load() && rpa::decode_supported(p)) ? 1 : 0;
+
+  hipStream_t s = (hipStream_t)stream;
+  if (p.mfma_path) {
+    const size_t po = part_o_bytes(T, Hq, D), pml = part_ml_bytes(T, Hq);
+    int splits = static_splits(M, page_size);
+    const size_t usable = workspace_bytes > 256 ? workspace_bytes - 256 : 0;
+    if (!workspace || usable < po + pml)
+      return fail(RPA_ERR_WORKSPACE, "rpa_ragged_paged_attention: workspace %zu bytes < %zu needed for one split", workspace_bytes, po + pml + 256);
+    if ((size_t)splits * (po + pml) > usable) splits = (int)(usable / (po + pml));
+    p.max_splits = splits;
+    char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    p.part_o = (float*)base;
+    p.part_ml = (float*)(base + (size_t)splits * po);
+    int err = rpa::launch_attn_decode(s, p);
+    if (err) return hip_fail(err, "decode kernel launch");
+    // Rows too large for the decode kernel: MFMA prefill kernel where it applies, fp32 kernel otherwise.
+    if (rpa::prefill_supported(p)) err = rpa::launch_attn_prefill(s, p);
+    else err = rpa::launch_attn_generic(s, p);
+    if (err) return hip_fail(err, "prefill kernel launch");
+  } else {
+    int err = rpa::launch_attn_generic(s, p);
+    if (err) return hip_fail(err, "fp32 kernel launch");
+  }
+  return hip_fail(rpa::launch_attn_merge(s, p), "merge kernel launch");
+}
+
+int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void* key, const void* value,
+                                  void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
+                                  const int32_t* query_start_loc, const int32_t* distribution, void* out,
+                                  void* workspace, size_t workspace_bytes, int T, int S, int M, int P, int page_size,
+                                  int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype, float softmax_scale,
+                                  int sliding_window, float logits_soft_cap) {
+  if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16)
+    return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention_v3: quantised pages are read-only (kv_dtype %d)", kv_dtype);
+  if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention_v3: null distribution");
+  const int32_t* n_live = distribution + 2;
+  int err = rpa_page_scatter_ragged(stream, key, value, kv_pages, context_lens, block_tables, query_start_loc, n_live,
+                                    T, S, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
+  if (err) return err;
+  return rpa_ragged_paged_attention(stream, q, kv_pages, nullptr, context_lens, block_tables, query_start_loc, n_live,
+                                    out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
+                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+}
+
+}  // extern "C"

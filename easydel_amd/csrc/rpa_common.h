@@ -1,0 +1,121 @@
+// Shared device-side definitions for the gfx950 ragged-paged-attention kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/rpa_hip.h"
+
+namespace rpa {
+
+constexpr int kWave = 64;
+constexpr int kRowBlock = 16;      // MFMA M/N extent: rows (token, group-head pairs) per wave
+constexpr int kMaxSplitsCap = 64;  // hard upper bound on split-K partials per sequence
+
+// Everything a kernel needs, passed by value.
+struct AttnParams {
+  const void* q;
+  const void* kv_pages;
+  const float* kv_scales;  // [P][C] or null
+  const int32_t* context_lens;
+  const int32_t* block_tables;
+  const int32_t* qsl;
+  const int32_t* num_seqs;
+  void* out;
+  float* part_o;   // [max_splits][T][Hq][D]
+  float* part_ml;  // [max_splits][T][Hq][2]  (running max in log2 units, running sum)
+  int T, S, M, P, page_size, Hq, Hkv, group, D, C;
+  int64_t token_stride;  // bytes between consecutive tokens of a page = C*D*elem
+  int64_t page_stride;   // bytes between pages
+  int q_dtype, kv_dtype;
+  float scale;       // softmax scale
+  float scale_log2;  // softmax scale * log2(e)
+  int window;        // <= 0: none
+  float softcap;     // <= 0: none
+  int max_splits;    // >= 1
+  int chunk_target;  // tokens, multiple of 64
+  int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
+};
+
+// Per-sequence work plan.  Every kernel derives it from device metadata with this one function,
+// so producer (attention) and consumer (merge) always agree on who wrote what.
+struct SeqPlan {
+  int q0, q_len, ctx;
+  int lo, hi;       // key range any row of the sequence may see, lo rounded down to 64 tokens
+  int chunk;        // tokens per split
+  int n_chunks;     // number of splits that hold data
+  bool live;        // has queries and keys
+  bool small_rows;  // q_len * group <= 16: served by the split-K decode kernel
+};
+
+__device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
+  SeqPlan s;
+  const int n_live = p.num_seqs[0];
+  s.q0 = p.qsl[i];
+  s.q_len = p.qsl[i + 1] - s.q0;
+  s.ctx = p.context_lens[i];
+  if (s.ctx > p.M * p.page_size) s.ctx = p.M * p.page_size;  // never index past the block-table row
+  s.live = (i < n_live) && (s.q_len > 0) && (s.ctx > 0);
+  s.hi = s.ctx;
+  s.lo = 0;
+  if (p.window > 0) {
+    int first = s.ctx - s.q_len - p.window + 1;  // lowest key visible to the first query row
+    s.lo = first > 0 ? (first & ~63) : 0;
+  }
+  s.small_rows = (s.q_len * p.group <= kRowBlock);
+  int span = s.hi - s.lo;
+  if (span < 1) span = 1;
+  int per = (span + p.max_splits - 1) / p.max_splits;
+  per = (per + 63) & ~63;
+  s.chunk = per > p.chunk_target ? per : p.chunk_target;
+  s.n_chunks = (span + s.chunk - 1) / s.chunk;
+  return s;
+}
+
+// Largest i in [0, n) with qsl[i] <= t (qsl non-decreasing); callers guarantee qsl[0] <= t < qsl[n].
+__device__ __forceinline__ int find_seq(const int32_t* qsl, int n, int t) {
+  int lo = 0, hi = n;  // invariant: qsl[lo] <= t < qsl[hi]
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (qsl[mid] <= t) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {  // round to nearest even, NaN kept quiet
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+
+__device__ __forceinline__ float fp8_e4m3_to_float(uint8_t c) {
+  auto v = __builtin_amdgcn_cvt_pk_f32_fp8((int)c, false);
+  return v[0];
+}
+
+template <int DT> struct ElemBytes;
+template <> struct ElemBytes<RPA_F32> { static constexpr int v = 4; };
+template <> struct ElemBytes<RPA_BF16> { static constexpr int v = 2; };
+template <> struct ElemBytes<RPA_FP8_E4M3> { static constexpr int v = 1; };
+template <> struct ElemBytes<RPA_INT8> { static constexpr int v = 1; };
+
+inline int elem_bytes(int dt) { return dt == RPA_F32 ? 4 : dt == RPA_BF16 ? 2 : 1; }
+
+template <int DT>
+__device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
+  if constexpr (DT == RPA_F32) return ((const float*)base)[idx];
+  else if constexpr (DT == RPA_BF16) return bf16_bits_to_float(((const uint16_t*)base)[idx]);
+  else if constexpr (DT == RPA_FP8_E4M3) return fp8_e4m3_to_float(((const uint8_t*)base)[idx]);
+  else return (float)((const int8_t*)base)[idx];
+}
+
+// Launchers (one per translation unit); all return a hipError_t as int.
+int launch_attn_generic(hipStream_t stream, const AttnParams& p);
+int launch_attn_decode(hipStream_t stream, const AttnParams& p);
+int launch_attn_prefill(hipStream_t stream, const AttnParams& p);
+int launch_attn_merge(hipStream_t stream, const AttnParams& p);
+bool decode_supported(const AttnParams& p);
+bool prefill_supported(const AttnParams& p);
+
+}  // namespace rpa

@@ -1,0 +1,73 @@
+// MFMA building blocks shared by the decode and prefill kernels (gfx950, wave64).
+//
+// Operand layouts of the two instructions used, for lane l with i = l & 15, g = l >> 4:
+//   v_mfma_f32_16x16x32_bf16 : A[row i][k = 8g..8g+7], B[k = 8g..8g+7][col i], C[row 4g+j][col i] (j = 0..3)
+//   v_mfma_f32_16x16x16_bf16 : A[row i][k = 4g..4g+3], B[k = 4g..4g+3][col i], C[row 4g+j][col i]
+// The contraction index k may be permuted freely as long as A and B use the same permutation.
+#pragma once
+#include "rpa_common.h"
+
+namespace rpa {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// Two floats -> packed bf16 pair (lo = a, hi = b), round to nearest even.
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  f32x2 v = {a, b};
+  bf16x2 r = __builtin_convertvector(v, bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// Four 8-bit codes in one dword -> four floats.
+template <int KVT>
+__device__ __forceinline__ void decode4(uint32_t w, float* f) {
+  if constexpr (KVT == RPA_FP8_E4M3) {
+    auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = hi[0]; f[3] = hi[1];
+  } else {
+    f[0] = (float)(int8_t)(w & 0xff);
+    f[1] = (float)(int8_t)((w >> 8) & 0xff);
+    f[2] = (float)(int8_t)((w >> 16) & 0xff);
+    f[3] = (float)(int8_t)(w >> 24);
+  }
+}
+
+// Eight 8-bit codes (two dwords) -> one bf16x8 MFMA operand (exact: both code sets fit bf16).
+template <int KVT>
+__device__ __forceinline__ bf16x8 codes8_to_bf16x8(uint32_t w0, uint32_t w1) {
+  float f[8];
+  decode4<KVT>(w0, f);
+  decode4<KVT>(w1, f + 4);
+  u32x4 r = {pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7])};
+  return __builtin_bit_cast(bf16x8, r);
+}
+
+// XOR swizzle of 16-byte chunks inside an LDS row of ROW_BYTES so that 16 consecutive token rows
+// read at the same logical chunk land on distinct bank groups.
+template <int ROW_BYTES>
+__device__ __forceinline__ int swz_key(int tok) {
+  constexpr int NCH = ROW_BYTES / 16;
+  if constexpr (NCH >= 16) return tok & 15;
+  else if constexpr (NCH == 8) return ((tok >> 1) ^ ((tok & 1) << 2)) & 7;
+  else if constexpr (NCH == 4) return (tok >> 2) & 3;
+  else return 0;
+}
+
+__device__ __forceinline__ float xor16_max(float v) { return fmaxf(v, __shfl_xor(v, 16)); }
+__device__ __forceinline__ float xor32_max(float v) { return fmaxf(v, __shfl_xor(v, 32)); }
+
+// tanh through the hardware exp2: tanh(x) = 1 - 2 / (exp(2x) + 1).  Good to ~1e-6 relative, far inside
+// the bf16 tolerance of the MFMA kernels (the fp32 kernel uses tanhf).
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);  // exp(2x)
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+
+}  // namespace rpa

@@ -1,0 +1,132 @@
+// Page scatter kernels: bit-exact copies of new K/V token rows into the paged cache.
+#include "rpa_common.h"
+
+namespace rpa {
+
+// Copy `bytes` from src to dst with the whole block; 16-byte vectors when both are aligned.
+__device__ __forceinline__ void block_copy(char* dst, const char* src, int64_t bytes) {
+  const bool aligned = ((((uintptr_t)dst) | ((uintptr_t)src) | (uintptr_t)bytes) & 15) == 0;
+  if (aligned) {
+    const int64_t n = bytes >> 4;
+    for (int64_t k = threadIdx.x; k < n; k += blockDim.x) ((uint4*)dst)[k] = ((const uint4*)src)[k];
+  } else {
+    for (int64_t k = threadIdx.x; k < bytes; k += blockDim.x) dst[k] = src[k];
+  }
+}
+
+// Slice form.  One block per slice column.  A column's packed-token offset is the sum of the
+// effective lengths of the columns before it (inactive and non-local columns count as zero),
+// which the block recomputes with a strided sum: N is at most a few thousand.
+__global__ __launch_bounds__(256) void scatter_slices_kernel(const char* __restrict__ new_kv,
+                                                             const int32_t* __restrict__ si,
+                                                             const int32_t* __restrict__ num_slices,
+                                                             char* __restrict__ pages, int T, int N,
+                                                             int64_t num_positions, int page_size,
+                                                             int64_t row_bytes, int shard) {
+  const int c = blockIdx.x;
+  const int n_valid = num_slices[0];
+  if (c >= n_valid) return;
+  int64_t local_pages = num_positions / page_size;
+  if (local_pages < 1) local_pages = 1;
+  const int64_t page_base = (int64_t)shard * local_pages;
+
+  auto floordiv = [](int64_t a, int64_t b) { int64_t q = a / b; return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q; };
+  auto eff_len = [&](int col) -> int {
+    if (col >= n_valid) return 0;
+    const int64_t lp = floordiv(si[col], page_size) - page_base;
+    if (lp < 0 || lp >= local_pages) return 0;
+    const int ln = si[2 * N + col];
+    return ln > 0 ? ln : 0;
+  };
+
+  __shared__ int red[256];
+  int partial = 0;
+  for (int col = threadIdx.x; col < c; col += blockDim.x) partial += eff_len(col);
+  red[threadIdx.x] = partial;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+    __syncthreads();
+  }
+  const int packed0 = red[0];
+  const int ln = eff_len(c);
+  if (ln == 0) return;
+
+  const int64_t g = si[c];
+  const int64_t gp = floordiv(g, page_size);
+  const int64_t dst0 = (gp - page_base) * page_size + (g - gp * page_size);
+  const int64_t src0 = si[N + c];
+  for (int off = 0; off < ln; ++off) {
+    if (packed0 + off >= T) break;  // beyond the packed prefix the reference can address
+    const int64_t src = src0 + off;
+    int64_t dst = dst0 + off;
+    if (src < 0 || src >= T) continue;
+    if (dst < 0) dst += num_positions;
+    if (dst < 0 || dst >= num_positions) continue;
+    block_copy(pages + dst * row_bytes, new_kv + src * row_bytes, row_bytes);
+  }
+}
+
+// Ragged form.  One block per query token: find its sequence, then its slot in the sequence's pages.
+__global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restrict__ key,
+                                                             const char* __restrict__ value,
+                                                             char* __restrict__ pages,
+                                                             const int32_t* __restrict__ context_lens,
+                                                             const int32_t* __restrict__ block_tables,
+                                                             const int32_t* __restrict__ qsl,
+                                                             const int32_t* __restrict__ num_seqs, int M, int P,
+                                                             int page_size, int Hkv, int head_bytes,
+                                                             int64_t token_stride, int64_t page_stride) {
+  const int t = blockIdx.x;
+  const int n_live = num_seqs[0];
+  if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
+  const int i = find_seq(qsl, n_live, t);
+  const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
+  const int pos = context_lens[i] - q_len + (t - q0);
+  if (pos < 0) return;
+  const int page_idx = pos / page_size;
+  if (page_idx >= M) return;
+  const int page = block_tables[(int64_t)i * M + page_idx];
+  if (page < 0 || page >= P) return;
+  char* row = pages + (int64_t)page * page_stride + (int64_t)(pos % page_size) * token_stride;
+  const char* ksrc = key + (int64_t)t * Hkv * head_bytes;
+  const char* vsrc = value + (int64_t)t * Hkv * head_bytes;
+  if ((head_bytes & 15) == 0 && ((((uintptr_t)row) | ((uintptr_t)ksrc) | ((uintptr_t)vsrc)) & 15) == 0) {
+    const int vec_per_head = head_bytes >> 4;
+    const int n = 2 * Hkv * vec_per_head;
+    for (int k = threadIdx.x; k < n; k += blockDim.x) {
+      const int ch = k / vec_per_head, w = k - ch * vec_per_head;  // combined head, vector within head
+      const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
+      ((uint4*)(row + (int64_t)ch * head_bytes))[w] = ((const uint4*)src)[w];
+    }
+  } else {
+    const int n = 2 * Hkv * head_bytes;
+    for (int k = threadIdx.x; k < n; k += blockDim.x) {
+      const int ch = k / head_bytes, w = k - ch * head_bytes;
+      const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
+      row[(int64_t)ch * head_bytes + w] = src[w];
+    }
+  }
+}
+
+int launch_scatter_slices(hipStream_t stream, const void* new_kv, const int32_t* si, const int32_t* num_slices,
+                          void* pages, int T, int N, int64_t num_positions, int page_size, int64_t row_bytes,
+                          int shard) {
+  hipLaunchKernelGGL(scatter_slices_kernel, dim3(N), dim3(256), 0, stream, (const char*)new_kv, si, num_slices,
+                     (char*)pages, T, N, num_positions, page_size, row_bytes, shard);
+  return (int)hipGetLastError();
+}
+
+int launch_scatter_ragged(hipStream_t stream, const void* key, const void* value, void* pages,
+                          const int32_t* context_lens, const int32_t* block_tables, const int32_t* qsl,
+                          const int32_t* num_seqs, int T, int M, int P, int page_size, int Hkv, int D, int C,
+                          int elem_bytes) {
+  const int head_bytes = D * elem_bytes;
+  const int64_t token_stride = (int64_t)C * head_bytes;
+  hipLaunchKernelGGL(scatter_ragged_kernel, dim3(T), dim3(256), 0, stream, (const char*)key, (const char*)value,
+                     (char*)pages, context_lens, block_tables, qsl, num_seqs, M, P, page_size, Hkv, head_bytes,
+                     token_stride, token_stride * page_size);
+  return (int)hipGetLastError();
+}
+
+}  // namespace rpa

@@ -1,0 +1,180 @@
+"""Tensor-level entry points: thin, checked wrappers over the C ABI.
+
+PyTorch appears here only as the owner of device memory and streams (``data_ptr()`` and the
+current HIP stream); all arithmetic happens in librpa_hip.so.  Every function raises if the
+library is missing, if a tensor is not on a GPU, or if the C ABI reports an error.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+_DTYPE_TAG = {
+    torch.float32: _lib.RPA_F32,
+    torch.bfloat16: _lib.RPA_BF16,
+    torch.float8_e4m3fn: _lib.RPA_FP8_E4M3,
+    torch.int8: _lib.RPA_INT8,
+}
+
+_workspaces: dict[tuple, torch.Tensor] = {}
+
+
+def dtype_tag(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_TAG[dtype]
+    except KeyError:
+        raise NotImplementedError(f"dtype {dtype} is not supported by the ROCm ragged-page kernels") from None
+
+
+def _dev(t: torch.Tensor, name: str) -> int:
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor holding device memory, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} is on {t.device}; the ROCm ragged-page kernels need GPU memory (no CPU fallback)")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    return t.data_ptr()
+
+
+def _i32(t: torch.Tensor, name: str) -> int:
+    if t.dtype != torch.int32:
+        raise TypeError(f"{name} must be int32, got {t.dtype}")
+    return _dev(t, name)
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def page_geometry(kv_pages: torch.Tensor, head_dim: int) -> tuple[int, int, int]:
+    """(P, page_size, C) of a v2 ``[P, pg, 2*Hkv, D]`` or v3 ``[P, pg, groups, packing, Dp]`` page buffer.
+
+    Both have token rows of ``C`` combined heads of ``head_dim`` elements, K at even and V at odd
+    combined heads; the v3 shape for ``head_dim == 64`` packs K_h|V_h into one 128-wide row, which
+    is the same bytes.  A padded head (``Dp > head_dim`` otherwise) is not supported.
+    """
+    if kv_pages.ndim not in (4, 5):
+        raise ValueError(f"kv_pages must be 4-D (v2) or 5-D (v3), got shape {tuple(kv_pages.shape)}")
+    stored = kv_pages.shape[-1]
+    if stored != head_dim and not (head_dim == 64 and stored == 128):
+        raise NotImplementedError(f"padded head storage (stored {stored}, head_dim {head_dim}) is not supported")
+    per_token = math.prod(kv_pages.shape[2:])
+    return kv_pages.shape[0], kv_pages.shape[1], per_token // head_dim
+
+
+def workspace_bytes(T, S, M, page_size, Hq, Hkv, D, q_dtype: torch.dtype, kv_dtype: torch.dtype) -> int:
+    return int(_lib.load().rpa_attention_workspace_bytes(T, S, M, page_size, Hq, Hkv, D, dtype_tag(q_dtype), dtype_tag(kv_dtype)))
+
+
+def _workspace(device, nbytes: int) -> torch.Tensor:
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def page_scatter_slices(new_kv, slice_indices, num_slices, kv_cache_pages, *, page_size: int, page_shard_index: int = 0):
+    """In-place v2 scatter: ``kv_cache_pages [N, C, D]`` (flat positions) <- ``new_kv [T, C, D]`` by slices."""
+    lib = _lib.load()
+    if new_kv.dtype != kv_cache_pages.dtype:
+        raise TypeError(f"new_kv dtype {new_kv.dtype} != cache dtype {kv_cache_pages.dtype}")
+    if slice_indices.ndim != 2 or slice_indices.shape[0] != 3:
+        raise ValueError(f"slice_indices must be [3, N], got {tuple(slice_indices.shape)}")
+    if tuple(new_kv.shape[1:]) != tuple(kv_cache_pages.shape[1:]):
+        raise ValueError(f"token row shapes differ: {tuple(new_kv.shape[1:])} vs {tuple(kv_cache_pages.shape[1:])}")
+    T, N, n_pos = new_kv.shape[0], slice_indices.shape[1], kv_cache_pages.shape[0]
+    if T == 0 or N == 0 or n_pos == 0:
+        return kv_cache_pages
+    row_bytes = math.prod(new_kv.shape[1:]) * new_kv.element_size()
+    _lib.check(lib.rpa_page_scatter_slices(
+        _stream(kv_cache_pages), _dev(new_kv, "new_kv"), _i32(slice_indices, "slice_indices"),
+        _i32(num_slices, "num_slices"), _dev(kv_cache_pages, "kv_cache_pages"), T, N, n_pos, int(page_size), row_bytes,
+        int(page_shard_index)))
+    return kv_cache_pages
+
+
+def page_scatter_ragged(key, value, kv_pages, context_lens, block_tables, query_start_loc, num_seqs):
+    """In-place v3 write: tokens of sequence i land at positions ``[ctx_i - q_len_i, ctx_i)`` of its pages."""
+    lib = _lib.load()
+    if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
+        raise TypeError(f"key/value dtype {key.dtype}/{value.dtype} must equal the cache dtype {kv_pages.dtype}")
+    T, Hkv, D = key.shape
+    P, pg, C = page_geometry(kv_pages, D)
+    S = context_lens.shape[0]
+    M = block_tables.numel() // S
+    if T == 0:
+        return kv_pages
+    _lib.check(lib.rpa_page_scatter_ragged(
+        _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+        _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, key.element_size()))
+    return kv_pages
+
+
+def _attn_common(query, kv_pages, context_lens, block_tables, num_kv_heads, softmax_scale, sliding_window, logits_soft_cap):
+    T, Hq, D = query.shape
+    P, pg, C = page_geometry(kv_pages, D)
+    S = context_lens.shape[0]
+    if block_tables.numel() % S:
+        raise ValueError("block_tables size is not a multiple of the number of sequence rows")
+    M = block_tables.numel() // S
+    Hkv = int(num_kv_heads) if num_kv_heads is not None else C // 2
+    scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    window = int(sliding_window) if sliding_window else 0
+    cap = float(logits_soft_cap) if logits_soft_cap else 0.0
+    return T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap
+
+
+def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *,
+                           softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_scales=None,
+                           num_kv_heads=None, out=None):
+    """Read-only ragged paged attention; returns ``[T, Hq, D]`` in the query dtype."""
+    lib = _lib.load()
+    T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+        query, kv_pages, context_lens, block_tables, num_kv_heads, softmax_scale, sliding_window, logits_soft_cap)
+    if out is None:
+        out = torch.empty_like(query)
+    if T == 0:
+        return out
+    qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    scales_ptr = None
+    if kv_scales is not None:
+        if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
+            raise ValueError(f"kv_scales must be float32 [P={P}, C={C}]")
+        scales_ptr = _dev(kv_scales, "kv_scales")
+    _lib.check(lib.rpa_ragged_paged_attention(
+        _stream(query), _dev(query, "query"), _dev(kv_pages, "kv_pages"), scales_ptr,
+        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+        _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap))
+    return out
+
+
+def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_tables, query_start_loc, distribution, *,
+                              softmax_scale=None, sliding_window=None, logits_soft_cap=None, num_kv_heads=None, out=None):
+    """Fused scatter + attention; updates ``kv_pages`` in place and returns ``(out, kv_pages)``."""
+    lib = _lib.load()
+    if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
+        raise TypeError(f"key/value dtype {key.dtype}/{value.dtype} must equal the cache dtype {kv_pages.dtype}")
+    T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+        query, kv_pages, context_lens, block_tables, key.shape[1] if num_kv_heads is None else num_kv_heads,
+        softmax_scale, sliding_window, logits_soft_cap)
+    if out is None:
+        out = torch.empty_like(query)
+    if T == 0:
+        return out, kv_pages
+    qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    _lib.check(lib.rpa_ragged_paged_attention_v3(
+        _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+        _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap))
+    return out, kv_pages

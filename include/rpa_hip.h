@@ -1,0 +1,152 @@
+/*
+ * rpa_hip.h -- C ABI of the MI355X (gfx950) ragged-paged-attention library.
+ *
+ * One shared library, librpa_hip.so, exports the entry points below.  Every pointer marked
+ * "device" is a HIP device pointer; metadata arrays are int32.  No entry point synchronises
+ * the device, allocates device memory, or reads device data back to the host: work is
+ * enqueued on `stream` with launch grids sized from the static bounds (T, S, M) and blocks
+ * that exit early on padded rows, so the calls are legal inside a compiled serving step.
+ *
+ * Return value: 0 on success; a positive value is a hipError_t from a failed launch; a
+ * negative value is one of the RPA_ERR_* codes.  rpa_last_error() returns a thread-local,
+ * human-readable description of the most recent failure on the calling thread.
+ *
+ * KV page layout (all entry points): kv_pages[P][page_size][C][D] elements, where combined
+ * head 2h holds K of KV head h and 2h+1 holds V (reference: easydel/caching/ragged_page/
+ * cache.py:719-726 for the v2 shape, :711-718 for the v3 shape, :954-973 for the K-even /
+ * V-odd interleave).  The reference's v3 storage [P][page][groups][packing][Dp] has the same
+ * bytes as [P][page][C = groups*packing][Dp]; for head_dim 64 it stores K_h|V_h in one
+ * 128-wide row, which is again the same bytes as C = 2*Hkv rows of 64.  C >= 2*Hkv.
+ */
+#ifndef RPA_HIP_H_
+#define RPA_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element formats of q / out (F32, BF16) and of KV pages (all four). */
+typedef enum rpa_dtype {
+  RPA_F32 = 0,
+  RPA_BF16 = 1,
+  RPA_FP8_E4M3 = 2, /* OCP e4m3fn codes, value = code * kv_scales[page][combined head] */
+  RPA_INT8 = 3      /* signed 8-bit codes, value = code * kv_scales[page][combined head] */
+} rpa_dtype;
+
+#define RPA_OK 0
+#define RPA_ERR_INVALID_ARGUMENT (-1) /* null pointer, non-positive size, inconsistent heads */
+#define RPA_ERR_UNSUPPORTED (-2)      /* dtype / head_dim combination no kernel covers */
+#define RPA_ERR_WORKSPACE (-3)        /* workspace smaller than rpa_attention_workspace_bytes() */
+
+typedef void* rpa_stream_t; /* a hipStream_t; NULL is the default stream */
+
+/* Library version, "major.minor.patch". */
+const char* rpa_version(void);
+
+/* Description of the last failure seen by the calling thread ("" if none). */
+const char* rpa_last_error(void);
+
+/*
+ * Page scatter, slice form.  Replaces kv_cache_update_jax
+ * (easydel/caching/ragged_page/utils.py:302-387, with the shard localisation of :66-123),
+ * which RaggedPagesCacheView.concatenate_to_cache calls for v2 caches (cache.py:853-930).
+ *
+ *   new_kv        device, [T][row_bytes]      token rows (K/V interleaved on the combined head axis)
+ *   slice_indices device, int32 [3][N]        row 0 = destination flat cache position (global page
+ *                                              space), row 1 = source token, row 2 = length
+ *   num_slices    device, int32 [1]           number of valid columns
+ *   kv_pages      device, [num_positions][row_bytes], updated in place
+ *   page_shard_index                          which contiguous block of num_positions/page_size
+ *                                              pages this buffer holds (0 when unsharded)
+ * Bit-exact copy of whole token rows.  Columns >= num_slices[0], non-local slices, packed
+ * tokens beyond T, sources outside [0,T) and destinations outside the buffer are dropped,
+ * exactly as the reference's mode="drop" scatter does.
+ */
+int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32_t* slice_indices,
+                            const int32_t* num_slices, void* kv_pages, int T, int N,
+                            int64_t num_positions, int page_size, int64_t row_bytes,
+                            int page_shard_index);
+
+/*
+ * Page scatter, ragged form: the write half of the fused v3 operation
+ * (ejkernel.modules.ragged_page_attention_v3 as called at
+ * easydel/operations/kernels/ragged_page_attention.py:732-746).  Sequence i < num_seqs[0]
+ * writes key/value[qsl[i] .. qsl[i+1]) to token positions [ctx_i - q_len_i, ctx_i) of the pages
+ * block_tables[i][*]; K of head h goes to combined head 2h, V to 2h+1.
+ *
+ *   key, value    device, [T][Hkv][D] in the cache element type (elem_bytes each)
+ *   kv_pages      device, [P][page_size][C][D], updated in place
+ *   block_tables  device, int32 [S][M] (the flattened [S*M] form is the same bytes)
+ *   num_seqs      device, int32 [1]: number of live rows (pass distribution + 2 for v3 metadata)
+ * Bit-exact.  Positions < 0 and padded tokens (t >= qsl[num_seqs]) are skipped.
+ */
+int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
+                            const int32_t* context_lens, const int32_t* block_tables,
+                            const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M,
+                            int P, int page_size, int Hkv, int D, int C, int elem_bytes);
+
+/*
+ * Bytes of scratch rpa_ragged_paged_attention needs for these static bounds (split-K
+ * partial outputs and their running max / sum).  The caller owns the buffer (under XLA it
+ * is an extra result of the custom call), 256-byte aligned.
+ */
+size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D,
+                                     int q_dtype, int kv_dtype);
+
+/*
+ * Ragged paged attention (read-only over the pages).  Replaces
+ * ejkernel.modules.ragged_page_attention_v2 as called at
+ * easydel/operations/kernels/ragged_page_attention.py:281-313, and the attention half of
+ * ragged_page_attention_v3 (:684-695, :732-746).
+ *
+ *   q             device, [T][Hq][D]          q_dtype in {RPA_F32, RPA_BF16}
+ *   kv_pages      device, [P][page_size][C][D] kv_dtype
+ *   kv_scales     device, float [P][C] or NULL; required for RPA_FP8_E4M3 / RPA_INT8 pages
+ *   context_lens  device, int32 [S]           tokens in the cache per sequence, new ones included
+ *   block_tables  device, int32 [S][M]
+ *   query_start_loc device, int32 [S+1]
+ *   num_seqs      device, int32 [1]           live rows
+ *   out           device, [T][Hq][D] q_dtype; rows of padded tokens are written as zeros
+ *   workspace     device, workspace_bytes >= rpa_attention_workspace_bytes(...)
+ *   softmax_scale                            multiplies q.k before the soft cap
+ *   sliding_window                           <= 0: none; W: key j visible iff pos-W < j <= pos
+ *   logits_soft_cap                          <= 0: none; cap: s = cap*tanh(s/cap)
+ * Query row r of sequence i sits at position ctx_i - q_len_i + r and attends causally.
+ */
+int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages,
+                               const float* kv_scales, const int32_t* context_lens,
+                               const int32_t* block_tables, const int32_t* query_start_loc,
+                               const int32_t* num_seqs, void* out, void* workspace, size_t workspace_bytes,
+                               int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
+                               int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
+                               float logits_soft_cap);
+
+/*
+ * Fused v3 form: rpa_page_scatter_ragged followed by rpa_ragged_paged_attention on the
+ * same stream, pages updated in place (the reference returns (out, kv_pages) and the
+ * caller stores the pages back, ragged_page_attention.py:747).  key/value must already be
+ * in the cache element type (the reference casts them first, :570-580); quantised pages
+ * are read-only here, so kv_dtype must be RPA_F32 or RPA_BF16.
+ */
+int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void* key, const void* value,
+                                  void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
+                                  const int32_t* query_start_loc, const int32_t* distribution, void* out,
+                                  void* workspace, size_t workspace_bytes, int T, int S, int M, int P,
+                                  int page_size, int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype,
+                                  float softmax_scale, int sliding_window, float logits_soft_cap);
+
+/*
+ * Tuning knobs (process-wide, read at call time).  Returns the previous value.
+ *   "decode_chunk"   target tokens per split-K chunk of the decode kernel (multiple of 64)
+ *   "max_splits"     upper bound on split-K partials per sequence (1..64)
+ *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
+ */
+int rpa_set_tunable(const char* name, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RPA_HIP_H_ */

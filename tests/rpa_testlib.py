@@ -1,0 +1,185 @@
+"""Shared helpers for the parity tests: seeded ragged batches in numpy, torch plumbing, comparisons."""
+
+from __future__ import annotations
+
+import math
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from oracle import rpa_oracle as orc  # noqa: E402
+
+F32, BF16, FP8, INT8 = orc.F32, orc.BF16, orc.FP8_E4M3, orc.INT8
+
+
+class Batch:
+    """A ragged batch: raw storage bits for the device plus decoded float64 values for the oracle."""
+
+
+def make_batch(seed, ctx_lens, q_lens, *, Hq, Hkv, D, page_size, num_pages=None, q_dtype=BF16, kv_dtype=BF16,
+               pad_rows=0, pad_tokens=0, max_pages=None, shared_prefix_pages=0, fill="normal"):
+    rng = np.random.default_rng(seed)
+    ctx_lens = np.asarray(ctx_lens, dtype=np.int32)
+    q_lens = np.asarray(q_lens, dtype=np.int32)
+    n = len(ctx_lens)
+    S = n + pad_rows
+    pages_needed = [-(-int(c) // page_size) for c in ctx_lens]
+    M = max_pages or max(max(pages_needed), 1)
+    P = num_pages or (sum(pages_needed) + 8)
+    C = 2 * Hkv
+    b = Batch()
+    b.Hq, b.Hkv, b.D, b.page_size, b.P, b.M, b.S, b.C = Hq, Hkv, D, page_size, P, M, S, C
+    b.q_dtype, b.kv_dtype = q_dtype, kv_dtype
+    b.n = n
+
+    # block tables: joint draw without replacement from pages 1..P-1 (page 0 is the null page)
+    perm = rng.permutation(np.arange(1, P))
+    bt = np.zeros((S, M), dtype=np.int32)
+    k = 0
+    for i, need in enumerate(pages_needed):
+        bt[i, :need] = perm[k:k + need]
+        k += need
+    if shared_prefix_pages and n >= 2:  # prefix caching: several sequences share physical pages
+        for i in range(1, n):
+            m = min(shared_prefix_pages, pages_needed[0], pages_needed[i] - 1)
+            if m > 0:
+                bt[i, :m] = bt[0, :m]
+    b.block_tables = bt
+    ctx_full = np.zeros(S, dtype=np.int32)
+    ctx_full[:n] = ctx_lens
+    b.context_lens = ctx_full
+    qsl = np.zeros(S + 1, dtype=np.int32)
+    qsl[1:n + 1] = np.cumsum(q_lens)
+    qsl[n + 1:] = qsl[n]  # flat extension, as the reference's batch preparer pads it
+    b.query_start_loc = qsl
+    b.num_seqs = np.array([n], dtype=np.int32)
+    T = int(qsl[n]) + pad_tokens
+    b.T = T
+    b.q_lens = q_lens
+
+    # queries
+    qf = rng.standard_normal((T, Hq, D), dtype=np.float32)
+    if q_dtype == BF16:
+        b.q_raw = orc.f32_to_bf16_bits(qf)
+        b.q_val = orc.bf16_bits_to_f32(b.q_raw).astype(np.float64)
+    else:
+        b.q_raw = qf
+        b.q_val = qf.astype(np.float64)
+
+    # pool
+    shape = (P, page_size, C, D)
+    if fill == "normal":
+        vals = rng.standard_normal(shape, dtype=np.float32)
+    else:
+        vals = np.full(shape, np.float32(fill), dtype=np.float32)
+    b.kv_scales = None
+    if kv_dtype == F32:
+        b.kv_raw = vals
+        b.kv_val = vals.astype(np.float64)
+    elif kv_dtype == BF16:
+        b.kv_raw = orc.f32_to_bf16_bits(vals)
+        b.kv_val = orc.bf16_bits_to_f32(b.kv_raw).astype(np.float64)
+    elif kv_dtype == FP8:
+        scales = rng.uniform(0.5, 2.0, size=(P, C)).astype(np.float32)
+        b.kv_raw = orc.f32_to_e4m3fn_bits(vals)  # codes ~ N(0,1); true values are codes * scale
+        b.kv_val = orc.e4m3fn_bits_to_f32(b.kv_raw).astype(np.float64)
+        b.kv_scales = scales
+    elif kv_dtype == INT8:
+        true_vals = vals * rng.uniform(0.5, 2.0, size=(P, 1, C, 1)).astype(np.float32)
+        amax = np.abs(true_vals).max(axis=(1, 3))
+        scales = (amax / 127.0).astype(np.float32)
+        codes = np.clip(np.rint(true_vals / scales[:, None, :, None]), -127, 127).astype(np.int8)
+        b.kv_raw = codes
+        b.kv_val = codes.astype(np.float64)
+        b.kv_scales = scales
+    else:
+        raise ValueError(kv_dtype)
+    return b
+
+
+def oracle_out(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_val=None):
+    return orc.ragged_paged_attention_ref(
+        b.q_val, b.kv_val if kv_val is None else kv_val, b.context_lens, b.block_tables, b.query_start_loc, b.num_seqs,
+        softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
+        kv_scales=b.kv_scales, num_kv_heads=b.Hkv)
+
+
+# ---- torch plumbing (imported lazily so the CPU-only tests need no GPU) ---------------------------
+
+
+def to_torch(raw: np.ndarray, tag: int, device):
+    import torch
+
+    if tag == BF16:
+        return torch.from_numpy(np.ascontiguousarray(raw).view(np.int16)).to(device).view(torch.bfloat16)
+    if tag == FP8:
+        return torch.from_numpy(np.ascontiguousarray(raw)).to(device).view(torch.float8_e4m3fn)
+    return torch.from_numpy(np.ascontiguousarray(raw)).to(device)
+
+
+def from_torch(t, tag: int) -> np.ndarray:
+    """Device tensor -> float64 numpy values."""
+    import torch
+
+    if tag == BF16:
+        return orc.bf16_bits_to_f32(t.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
+    if tag == FP8:
+        return orc.e4m3fn_bits_to_f32(t.view(torch.uint8).cpu().numpy()).astype(np.float64)
+    return t.cpu().numpy().astype(np.float64)
+
+
+def device_batch(b, device="cuda:0"):
+    import torch
+
+    d = {
+        "query": to_torch(b.q_raw, b.q_dtype, device),
+        "kv_pages": to_torch(b.kv_raw, b.kv_dtype, device),
+        "context_lens": torch.from_numpy(b.context_lens).to(device),
+        "block_tables": torch.from_numpy(b.block_tables).to(device),
+        "query_start_loc": torch.from_numpy(b.query_start_loc).to(device),
+        "num_seqs": torch.from_numpy(b.num_seqs).to(device),
+        "kv_scales": None if b.kv_scales is None else torch.from_numpy(b.kv_scales).to(device),
+    }
+    return d
+
+
+def run_gpu_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, device="cuda:0"):
+    from easydel_amd import kernels
+
+    d = device_batch(b, device)
+    out = kernels.ragged_paged_attention(
+        d["query"], d["kv_pages"], d["context_lens"], d["block_tables"], d["query_start_loc"], d["num_seqs"],
+        softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
+        kv_scales=d["kv_scales"], num_kv_heads=b.Hkv)
+    import torch
+
+    torch.cuda.synchronize()
+    return from_torch(out, b.q_dtype)
+
+
+def valid_rows(b) -> slice:
+    return slice(0, int(b.query_start_loc[b.n]))
+
+
+# Tolerances stated by the task: fp32 1e-5 max-abs; bf16 and dequantised 8-bit KV 2e-2 max-abs, 5e-3 mean-abs.
+TOL_F32_MAX = 1e-5
+TOL_BF16_MAX = 2e-2
+TOL_BF16_MEAN = 5e-3
+
+
+def assert_close(got, want, b, what=""):
+    rows = valid_rows(b)
+    g, w = got[rows], want[rows]
+    assert np.isfinite(g).all(), f"{what}: non-finite output"
+    err = np.abs(g - w)
+    if b.q_dtype == F32:
+        assert err.max() <= TOL_F32_MAX, f"{what}: fp32 max-abs {err.max():.3e} > {TOL_F32_MAX}"
+    else:
+        assert err.max() <= TOL_BF16_MAX, f"{what}: max-abs {err.max():.3e} > {TOL_BF16_MAX}"
+        assert err.mean() <= TOL_BF16_MEAN, f"{what}: mean-abs {err.mean():.3e} > {TOL_BF16_MEAN}"
+    return float(err.max()), float(err.mean())

@@ -1,0 +1,159 @@
+"""GPU parity: HIP ragged paged attention (through the C ABI) against the float64 oracle."""
+
+import numpy as np
+import pytest
+
+import rpa_testlib as tl
+from rpa_testlib import BF16, F32, FP8, INT8
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(b, what, **kw):
+    got = tl.run_gpu_attention(b, **kw)
+    want = tl.oracle_out(b, **kw)
+    mx, mean = tl.assert_close(got, want, b, what)
+    print(f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    return got
+
+
+def test_config1_fp32_mixed_batch(gpu):
+    # BASELINE config 1: 4 sequences, ctx [17,64,130,255], q_lens [1,1,8,33], Hq 8, Hkv 2, D 64, page 16, 128 pages
+    b = tl.make_batch(0, [17, 64, 130, 255], [1, 1, 8, 33], Hq=8, Hkv=2, D=64, page_size=16, num_pages=128,
+                      q_dtype=F32, kv_dtype=F32)
+    assert list(b.query_start_loc[:5]) == [0, 1, 2, 10, 43]
+    _check(b, "C1 fp32", softmax_scale=1.0 / 8.0)
+
+
+@pytest.mark.parametrize("D,page_size,Hq,Hkv", [(128, 64, 32, 8), (64, 16, 8, 2), (256, 128, 16, 8), (128, 16, 8, 1),
+                                                 (128, 32, 24, 6), (64, 64, 32, 8)])
+def test_bf16_decode(gpu, D, page_size, Hq, Hkv):
+    rng = np.random.default_rng(D + page_size)
+    ctx = rng.integers(1, 1600, size=12).tolist() + [1, 15, 16, 17, 512, 513, 1024]
+    b = tl.make_batch(1, ctx, [1] * len(ctx), Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, max_pages=-(-1600 // page_size))
+    _check(b, f"bf16 decode D{D} pg{page_size} Hq{Hq}/Hkv{Hkv}")
+
+
+@pytest.mark.parametrize("kv_dtype", [FP8, INT8])
+@pytest.mark.parametrize("D,page_size,Hq,Hkv", [(128, 64, 40, 8), (64, 16, 8, 2), (256, 32, 16, 8)])
+def test_quantised_kv_decode(gpu, kv_dtype, D, page_size, Hq, Hkv):
+    rng = np.random.default_rng(7)
+    ctx = rng.integers(1, 1400, size=10).tolist() + [1, 31, 32, 33, 700]
+    b = tl.make_batch(2, ctx, [1] * len(ctx), Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype,
+                      max_pages=-(-1400 // page_size))
+    _check(b, f"kv{kv_dtype} decode D{D} pg{page_size}")
+
+
+def test_small_multi_token_rows(gpu):
+    # speculative-style rows: q_len * group <= 16 stays on the split-K decode kernel with per-row causal limits
+    ctx = [5, 64, 300, 1100, 777, 4, 2]
+    q_lens = [4, 2, 3, 4, 1, 4, 2]
+    b = tl.make_batch(3, ctx, q_lens, Hq=32, Hkv=8, D=128, page_size=64, max_pages=20)
+    _check(b, "bf16 multi-token small rows")
+
+
+@pytest.mark.parametrize("window", [1, 64, 100, 1000])
+def test_sliding_window_decode(gpu, window):
+    ctx = [1, window, window + 1, window + 2, 900, 1500, 65, 129]
+    b = tl.make_batch(4, ctx, [1] * len(ctx), Hq=16, Hkv=4, D=128, page_size=64, max_pages=24)
+    _check(b, f"bf16 window {window}", sliding_window=window)
+
+
+def test_window_with_null_pages_left_of_window(gpu):
+    # pages entirely left of the window are freed by the scheduler and their table entries become the null page
+    # (page 0); poison page 0 with NaN bit patterns: it must never be read as data
+    W, pg = 256, 64
+    ctx = [1000, 1500, 700, 300]
+    b = tl.make_batch(5, ctx, [1] * 4, Hq=16, Hkv=4, D=128, page_size=pg, max_pages=24)
+    want = tl.oracle_out(b, sliding_window=W)
+    for i, c in enumerate(ctx):
+        first_needed = max(c - 1 - W + 1, 0) // pg
+        b.block_tables[i, :first_needed] = 0
+    b.kv_raw[0] = 0x7FC0  # bf16 NaN
+    got = tl.run_gpu_attention(b, sliding_window=W)
+    tl.assert_close(got, want, b, "window + null pages")
+
+
+@pytest.mark.parametrize("cap", [50.0, 5.0])
+def test_logit_soft_cap(gpu, cap):
+    ctx = [3, 200, 1000, 64]
+    b = tl.make_batch(6, ctx, [1, 1, 1, 1], Hq=16, Hkv=8, D=256, page_size=128, max_pages=8)
+    _check(b, f"bf16 softcap {cap}", logits_soft_cap=cap, softmax_scale=1.0 / 16.0)
+    bf = tl.make_batch(6, ctx, [1, 2, 5, 64], Hq=4, Hkv=2, D=64, page_size=16, q_dtype=F32, kv_dtype=F32)
+    _check(bf, f"fp32 softcap {cap}", logits_soft_cap=cap)
+
+
+def test_padding_rows_tokens_and_zero_length_rows(gpu):
+    # padded sequence rows, padded tokens past qsl[num_seqs], and a live row index with q_len == 0
+    ctx = [100, 0, 257, 64]
+    q_lens = [1, 0, 1, 1]
+    b = tl.make_batch(8, ctx, q_lens, Hq=32, Hkv=8, D=128, page_size=64, pad_rows=5, pad_tokens=7, max_pages=8)
+    got = _check(b, "padding")
+    assert np.all(got[int(b.query_start_loc[b.n]):] == 0.0), "padded token rows must be written as zeros"
+
+
+def test_shared_prefix_pages(gpu):
+    # prefix caching: the same physical pages appear in several block-table rows
+    ctx = [640, 700, 1000, 650]
+    b = tl.make_batch(9, ctx, [1] * 4, Hq=32, Hkv=8, D=128, page_size=64, shared_prefix_pages=9, max_pages=16)
+    _check(b, "shared prefix")
+
+
+def test_physical_page_permutation_is_bit_invariant(gpu):
+    ctx = [333, 1200, 64, 2000]
+    b = tl.make_batch(10, ctx, [1] * 4, Hq=32, Hkv=8, D=128, page_size=64, max_pages=32)
+    got1 = tl.run_gpu_attention(b)
+    rng = np.random.default_rng(0)
+    perm = np.concatenate([[0], 1 + rng.permutation(b.P - 1)])  # new physical id of each page; null page stays
+    kv2 = np.empty_like(b.kv_raw)
+    kv2[perm] = b.kv_raw
+    b.kv_raw = kv2
+    b.block_tables = perm[b.block_tables].astype(np.int32)
+    got2 = tl.run_gpu_attention(b)
+    assert np.array_equal(got1[tl.valid_rows(b)], got2[tl.valid_rows(b)])
+
+
+@pytest.mark.parametrize("q_dtype,kv_dtype", [(BF16, BF16), (F32, BF16), (BF16, F32), (BF16, FP8)])
+def test_mixed_prefill_decode_batch(gpu, q_dtype, kv_dtype):
+    ctx = [17, 64, 130, 255, 500, 33, 1]
+    q_lens = [1, 1, 8, 33, 100, 33, 1]
+    b = tl.make_batch(11, ctx, q_lens, Hq=8, Hkv=2, D=64, page_size=16, q_dtype=q_dtype, kv_dtype=kv_dtype)
+    _check(b, f"mixed q{q_dtype} kv{kv_dtype}")
+
+
+def test_mixed_batch_llama_shape(gpu):
+    ctx = [1500, 900, 300, 40, 2048]
+    q_lens = [1, 1, 256, 40, 130]
+    b = tl.make_batch(12, ctx, q_lens, Hq=32, Hkv=8, D=128, page_size=64, max_pages=32)
+    _check(b, "mixed llama-shaped")
+    _check(b, "mixed llama-shaped window", sliding_window=200)
+
+
+def test_generic_kernel_agrees_with_mfma_kernel(gpu):
+    from easydel_amd import _lib
+
+    ctx = [1500, 900, 300, 40, 2048, 1]
+    b = tl.make_batch(13, ctx, [1] * 6, Hq=32, Hkv=8, D=128, page_size=64, max_pages=32)
+    fast = tl.run_gpu_attention(b)
+    prev = _lib.set_tunable("force_generic", 1)
+    try:
+        slow = tl.run_gpu_attention(b)
+    finally:
+        _lib.set_tunable("force_generic", prev)
+    want = tl.oracle_out(b)
+    tl.assert_close(slow, want, b, "generic")
+    assert np.abs(fast - slow)[tl.valid_rows(b)].max() <= tl.TOL_BF16_MAX
+
+
+@pytest.mark.parametrize("chunk,splits", [(64, 64), (128, 2), (512, 1), (256, 5)])
+def test_split_k_settings_do_not_change_results(gpu, chunk, splits):
+    from easydel_amd import _lib
+
+    ctx = [1, 63, 64, 65, 1000, 1999, 128]
+    b = tl.make_batch(14, ctx, [1] * len(ctx), Hq=32, Hkv=8, D=128, page_size=64, max_pages=32)
+    p1, p2 = _lib.set_tunable("decode_chunk", chunk), _lib.set_tunable("max_splits", splits)
+    try:
+        _check(b, f"chunk {chunk} splits {splits}")
+    finally:
+        _lib.set_tunable("decode_chunk", p1)
+        _lib.set_tunable("max_splits", p2)
