@@ -1,0 +1,233 @@
+#!/usr/bin/env python3
+"""Benchmark of the ragged-paged-attention hot path on one MI355X.
+
+A step is one attention-layer call of the serving path on one ragged batch: the page scatter
+that writes the new K/V rows, then the attention over the paged cache (the fused v3 entry
+point of the C ABI).  The default workload is the Llama-3-8B-shaped pure decode batch
+(256 sequences, 512-8192 tokens of context, bf16, 64-token pages, 40 000-page pool).
+
+Prints one JSON line.  ``value`` = query tokens per second of one layer call with every
+input resident in HBM; ``roofline`` describes the dominant kernel (decode attention), timed
+with events on the launch stream in isolation; ``cpu_baseline`` times the C restatement of
+the same operation (oracle/rpa_oracle_c.c) on the host cores over a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c4-fp8", "c4-int8"])
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
+    ap.add_argument("--decode-chunk", type=int, default=0)
+    ap.add_argument("--max-splits", type=int, default=0)
+    return ap.parse_args()
+
+
+def build_workload(name, seed):
+    from easydel_amd import workloads
+
+    if name == "c2":
+        return workloads.config2_llama_decode(seed)
+    if name == "c4-fp8":
+        return workloads.config4_quantised_decode(seed, "fp8")
+    return workloads.config4_quantised_decode(seed, "int8")
+
+
+def cpu_baseline(w, tens, sample_seqs):
+    """Time the C restatement on the host for a subset of the batch's sequences (same pages, same queries)."""
+    import torch
+    from oracle import c_oracle
+
+    tag = {"f32": 0, "bf16": 1, "fp8": 2, "int8": 3}
+    threads = c_oracle.max_threads()
+    idx = np.arange(min(sample_seqs, w.S))
+    ctx = w.context_lens[idx]
+    need = -(-ctx.astype(np.int64) // w.page_size)
+    # compact host pool: the live pages of the sample, renumbered from 1
+    ids = np.concatenate([w.block_tables[i, :n] for i, n in zip(idx, need)])
+    bt = np.zeros((len(idx), w.max_pages_per_seq), dtype=np.int32)
+    k = 1
+    for r, n in enumerate(need):
+        bt[r, :n] = np.arange(k, k + n)
+        k += int(n)
+    dev_ids = torch.from_numpy(np.concatenate([[0], ids]).astype(np.int64)).to(tens["kv_pages"].device)
+    pool = tens["kv_pages"][dev_ids]
+    raw_dtype = {1: torch.uint8, 2: torch.int16, 4: torch.float32}[pool.element_size()]
+    pool_np = pool.view(raw_dtype).cpu().numpy()
+    scales_np = None if tens["kv_scales"] is None else tens["kv_scales"][dev_ids].cpu().numpy()
+    qsl = np.concatenate([[0], np.cumsum(w.q_lens[idx])]).astype(np.int32)
+    q0 = w.query_start_loc
+    rows = np.concatenate([np.arange(q0[i], q0[i + 1]) for i in idx])
+    q = tens["query"][torch.from_numpy(rows).to(tens["query"].device)]
+    q_np = q.view(torch.int16 if q.element_size() == 2 else torch.float32).cpu().numpy()
+
+    def run():
+        return c_oracle.attention(q_np, tag[w.q_dtype], pool_np, tag[w.kv_dtype], scales_np, ctx, bt, qsl, [len(idx)],
+                                  Hkv=w.Hkv, softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
+                                  logits_soft_cap=w.logits_soft_cap, num_threads=threads)
+
+    run()  # warm-up (page faults, thread pool)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        out = run()
+        reps += 1
+        if time.perf_counter() - t0 > 5.0 or reps >= 5:
+            break
+    dt = (time.perf_counter() - t0) / reps
+    tokens = int(w.q_lens[idx].sum())
+    return {
+        "value": tokens / dt,
+        "unit": "tokens/s (one attention-layer call)",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"first {len(idx)} of {w.S} sequences of the same batch ({int(ctx.sum())} cached tokens), "
+                  f"C restatement with OpenMP, {reps} timed calls of {dt * 1e3:.1f} ms",
+    }, out, rows
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    from easydel_amd import _lib, kernels, workloads
+
+    _lib.load()
+    if args.decode_chunk:
+        _lib.set_tunable("decode_chunk", args.decode_chunk)
+    if args.max_splits:
+        _lib.set_tunable("max_splits", args.max_splits)
+
+    dev = torch.device("cuda:0")
+    w = build_workload(args.workload, args.seed)
+    tens = workloads.device_tensors(w, dev, seed=args.seed)
+    quant = w.kv_dtype in ("fp8", "int8")
+    out = torch.empty_like(tens["query"])
+
+    def step():
+        if quant:  # quantised pages are read-only for this path
+            kernels.ragged_paged_attention(tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"],
+                                           tens["query_start_loc"], tens["num_seqs"], softmax_scale=w.softmax_scale,
+                                           sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap,
+                                           kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv, out=out)
+        else:
+            kernels.ragged_paged_attention_v3(tens["query"], tens["key"], tens["value"], tens["kv_pages"],
+                                              tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
+                                              tens["distribution"], softmax_scale=w.softmax_scale,
+                                              sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # dominant kernel in isolation: only the decode launch, events on the launch stream
+    prev = _lib.set_tunable("stages", 1)
+    stream = torch.cuda.current_stream(dev)
+    att = lambda: kernels.ragged_paged_attention(  # noqa: E731
+        tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
+        tens["num_seqs"], softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
+        logits_soft_cap=w.logits_soft_cap, kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv, out=out)
+    for _ in range(3):
+        att()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record(stream)
+        att()
+        b.record(stream)
+    torch.cuda.synchronize()
+    _lib.set_tunable("stages", prev)
+    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    att_bytes = w.attention_bytes()
+    achieved = att_bytes / (kernel_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "decode tokens/s + attn HBM TB/s (% of 8 TB/s), Llama-3-8B-shaped, 1 GPU",
+        "value": w.T / (ms_per_step * 1e-3),
+        "unit": "tokens/s (one attention-layer call: page scatter + ragged paged attention)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": {"bf16": "bf16", "fp8": "bf16 x fp8-e4m3 KV", "int8": "bf16 x int8 KV"}[w.kv_dtype],
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "sequences": w.S,
+            "query_tokens": w.T,
+            "q_heads": w.Hq,
+            "kv_heads": w.Hkv,
+            "head_dim": w.D,
+            "page_size": w.page_size,
+            "pool_pages": w.num_pages,
+            "context_tokens_total": int(w.context_lens.sum()),
+            "context_range": [int(w.context_lens.min()), int(w.context_lens.max())],
+            "seed": args.seed,
+        },
+        "attention_only_model_tokens_per_s_32_layers": w.T / (ms_per_step * 1e-3) / 32.0,
+        "attn_hbm_tb_s": achieved / 1e3,
+        "attn_hbm_pct_of_8tb_s": 100.0 * achieved / HBM_PEAK_GBS,
+        "step_hbm_tb_s": (att_bytes + w.scatter_bytes()) / (ms_per_step * 1e-3) / 1e12,
+        "roofline": {
+            "kernel": "attn_decode_kernel",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": att_bytes,
+            "kernel_ms": kernel_ms,
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        # size the sample for roughly 10-30 s of host work: ~0.35 GFLOP-equivalents per cached token-head here
+        sample = args.cpu_sample_seqs or max(8, min(w.S, 32))
+        base, cpu_out, rows = cpu_baseline(w, tens, sample)
+        step()
+        torch.cuda.synchronize()
+        gpu_rows = out[torch.from_numpy(rows).to(dev)].float().cpu().numpy()
+        base["max_abs_diff_vs_gpu_on_sample"] = float(np.abs(gpu_rows - cpu_out).max())
+        result["cpu_baseline"] = base
+    else:
+        result["cpu_baseline"] = None
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -20,6 +20,7 @@ thread_local char g_err[512] = "";
 std::atomic<int> g_decode_chunk{512};
 std::atomic<int> g_max_splits{32};
 std::atomic<int> g_force_generic{0};
+std::atomic<int> g_stages{7};  // bit 0: decode kernel, bit 1: prefill / large-row kernel, bit 2: merge
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -71,6 +72,7 @@ int rpa_set_tunable(const char* name, int value) {
     return g_max_splits.exchange(value);
   }
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
+  if (!strcmp(name, "stages")) return g_stages.exchange(value & 7);
   return -1;
 }
 
@@ -151,6 +153,7 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   p.mfma_path = (!g_force_generic.load() && rpa::decode_supported(p)) ? 1 : 0;
 
   hipStream_t s = (hipStream_t)stream;
+  const int stages = g_stages.load();
   if (p.mfma_path) {
     const size_t po = part_o_bytes(T, Hq, D), pml = part_ml_bytes(T, Hq);
     int splits = static_splits(M, page_size);
@@ -162,16 +165,17 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     p.part_o = (float*)base;
     p.part_ml = (float*)(base + (size_t)splits * po);
-    int err = rpa::launch_attn_decode(s, p);
+    int err = 0;
+    if (stages & 1) err = rpa::launch_attn_decode(s, p);
     if (err) return hip_fail(err, "decode kernel launch");
     // Rows too large for the decode kernel: MFMA prefill kernel where it applies, fp32 kernel otherwise.
-    if (rpa::prefill_supported(p)) err = rpa::launch_attn_prefill(s, p);
-    else err = rpa::launch_attn_generic(s, p);
+    if (stages & 2) err = rpa::prefill_supported(p) ? rpa::launch_attn_prefill(s, p) : rpa::launch_attn_generic(s, p);
     if (err) return hip_fail(err, "prefill kernel launch");
   } else {
-    int err = rpa::launch_attn_generic(s, p);
+    int err = (stages & 2) ? rpa::launch_attn_generic(s, p) : 0;
     if (err) return hip_fail(err, "fp32 kernel launch");
   }
+  if (!(stages & 4)) return RPA_OK;
   return hip_fail(rpa::launch_attn_merge(s, p), "merge kernel launch");
 }
 

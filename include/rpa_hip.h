@@ -143,6 +143,8 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
  *   "decode_chunk"   target tokens per split-K chunk of the decode kernel (multiple of 64)
  *   "max_splits"     upper bound on split-K partials per sequence (1..64)
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
+ *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
+ *                    1 = decode kernel, 2 = prefill / large-row kernel, 4 = merge (default 7)
  */
 int rpa_set_tunable(const char* name, int value);
 

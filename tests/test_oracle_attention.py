@@ -1,0 +1,175 @@
+"""Pins the attention oracle by mathematics: the reference holds no golden vector for the attention
+output (its only test of the call replaces the kernel with a stub), so each convention is fixed by a
+closed form, a reduction to textbook softmax attention (scipy), or an invariant chosen so that a
+plausible mistake (wrong sign or index, transposed operand, off-by-one window, swapped K/V) fails."""
+
+import numpy as np
+import pytest
+from scipy.special import softmax
+
+import rpa_testlib as tl
+from rpa_testlib import F32, orc
+
+
+def _dense_pages(k, v, page_size, table):
+    """Lay [ctx, Hkv, D] K/V out into pages following `table`; returns pages [P, pg, 2Hkv, D]."""
+    ctx, hkv, d = k.shape
+    P = int(max(table)) + 1
+    pages = np.full((P, page_size, 2 * hkv, d), 1e6)  # poison: anything read past ctx shows up
+    for j in range(ctx):
+        pages[table[j // page_size], j % page_size, 0::2] = k[j]
+        pages[table[j // page_size], j % page_size, 1::2] = v[j]
+    return pages
+
+
+def test_full_prefill_single_page_is_textbook_causal_attention():
+    rng = np.random.default_rng(0)
+    n, hq, hkv, d = 12, 4, 2, 8
+    q = rng.standard_normal((n, hq, d)); k = rng.standard_normal((n, hkv, d)); v = rng.standard_normal((n, hkv, d))
+    pages = _dense_pages(k, v, 16, [3])
+    got = orc.ragged_paged_attention_ref(q, pages, [n], np.array([[3]]), [0, n], [1], softmax_scale=0.3)
+    for h in range(hq):
+        s = 0.3 * q[:, h] @ k[:, h // 2].T
+        s = np.where(np.tril(np.ones((n, n), bool)), s, -np.inf)
+        np.testing.assert_allclose(got[:, h], softmax(s, axis=1) @ v[:, h // 2], rtol=1e-12, atol=1e-12)
+
+
+def test_ctx_one_returns_the_value_row_and_default_scale():
+    rng = np.random.default_rng(1)
+    q = rng.standard_normal((1, 4, 8)); k = rng.standard_normal((1, 2, 8)); v = rng.standard_normal((1, 2, 8))
+    got = orc.ragged_paged_attention_ref(q, _dense_pages(k, v, 4, [2]), [1], np.array([[2]]), [0, 1], [1])
+    np.testing.assert_allclose(got[0, :2], np.broadcast_to(v[0, 0], (2, 8)))
+    np.testing.assert_allclose(got[0, 2:], np.broadcast_to(v[0, 1], (2, 8)))
+    # default scale is D**-0.5: two keys, scores differ by q.(k1-k0)/sqrt(D)
+    q = rng.standard_normal((1, 1, 16)); k = rng.standard_normal((2, 1, 16)); v = np.stack([np.zeros((1, 16)), np.ones((1, 16))])
+    got = orc.ragged_paged_attention_ref(q, _dense_pages(k, v, 4, [1]), [2], np.array([[1]]), [0, 1], [1])
+    w1 = 1.0 / (1.0 + np.exp(-(q[0, 0] @ (k[1, 0] - k[0, 0])) / 4.0))
+    np.testing.assert_allclose(got[0, 0], np.full(16, w1), rtol=1e-12)
+
+
+def test_equal_keys_give_the_mean_of_visible_values():
+    rng = np.random.default_rng(2)
+    ctx, pg = 37, 8
+    k = np.broadcast_to(rng.standard_normal((1, 1, 8)), (ctx, 1, 8)); v = rng.standard_normal((ctx, 1, 8))
+    table = rng.permutation(np.arange(1, 9))[:5]
+    q = rng.standard_normal((3, 2, 8))
+    got = orc.ragged_paged_attention_ref(q, _dense_pages(k, v, pg, table), [ctx], table[None], [0, 3], [1])
+    for r in range(3):  # query row r sits at position ctx - 3 + r and sees keys 0..pos
+        np.testing.assert_allclose(got[r, 0], v[: ctx - 3 + r + 1, 0].mean(axis=0), rtol=1e-12)
+    gotw = orc.ragged_paged_attention_ref(q, _dense_pages(k, v, pg, table), [ctx], table[None], [0, 3], [1], sliding_window=5)
+    for r in range(3):  # W keys including self
+        pos = ctx - 3 + r
+        np.testing.assert_allclose(gotw[r, 1], v[pos - 4: pos + 1, 0].mean(axis=0), rtol=1e-12)
+
+
+def test_window_off_by_one_is_w_keys_including_self():
+    # ctx = W + 1: the decode row must ignore key 0 (a W+1-key window would include it)
+    W = 6
+    k = np.zeros((W + 1, 1, 4)); v = np.zeros((W + 1, 1, 4)); v[0] = 1000.0
+    q = np.ones((1, 1, 4))
+    pages = _dense_pages(k, v, 4, [1, 2])
+    got = orc.ragged_paged_attention_ref(q, pages, [W + 1], np.array([[1, 2]]), [0, 1], [1], sliding_window=W)
+    np.testing.assert_allclose(got, 0.0)
+    got = orc.ragged_paged_attention_ref(q, pages, [W + 1], np.array([[1, 2]]), [0, 1], [1], sliding_window=W + 1)
+    np.testing.assert_allclose(got, 1000.0 / (W + 1))
+
+
+def test_window_at_least_ctx_equals_no_window_and_huge_cap_equals_no_cap():
+    b = tl.make_batch(3, [17, 64, 130], [1, 5, 30], Hq=4, Hkv=2, D=16, page_size=16, q_dtype=F32, kv_dtype=F32)
+    base = tl.oracle_out(b)
+    np.testing.assert_allclose(tl.oracle_out(b, sliding_window=130), base, rtol=1e-12)
+    np.testing.assert_allclose(tl.oracle_out(b, logits_soft_cap=1e9), base, rtol=1e-9, atol=1e-12)
+    assert np.abs(tl.oracle_out(b, sliding_window=8) - base).max() > 1e-3
+    assert np.abs(tl.oracle_out(b, logits_soft_cap=0.5) - base).max() > 1e-3
+
+
+def test_soft_cap_is_applied_to_scaled_scores_before_softmax():
+    # two keys; with cap c the logit difference is c*(tanh(s1/c) - tanh(s0/c)), s = scale * q.k
+    q = np.array([[[2.0, 0.0]]]); k = np.array([[[1.0, 0.0]], [[-3.0, 0.0]]]); v = np.array([[[1.0, 0.0]], [[0.0, 1.0]]])
+    pages = _dense_pages(k, v, 2, [1])
+    got = orc.ragged_paged_attention_ref(q, pages, [2], np.array([[1]]), [0, 1], [1], softmax_scale=0.5, logits_soft_cap=2.0)
+    s = 2.0 * np.tanh(0.5 * np.array([2.0, -6.0]) / 2.0)
+    w = np.exp(s) / np.exp(s).sum()
+    np.testing.assert_allclose(got[0, 0], w, rtol=1e-12)
+
+
+def test_gqa_mapping_is_contiguous_groups():
+    # query head h reads KV head h // group: make KV head 1's values distinctive
+    rng = np.random.default_rng(4)
+    k = rng.standard_normal((5, 2, 4)); v = np.zeros((5, 2, 4)); v[:, 1] = 7.0
+    q = rng.standard_normal((1, 6, 4))
+    got = orc.ragged_paged_attention_ref(q, _dense_pages(k, v, 8, [1]), [5], np.array([[1]]), [0, 1], [1])
+    np.testing.assert_allclose(got[0, :3], 0.0, atol=1e-12)
+    np.testing.assert_allclose(got[0, 3:], 7.0, rtol=1e-12)
+
+
+def test_k_even_v_odd_interleave():
+    # swap K and V in storage: result must change to the swapped-roles attention
+    rng = np.random.default_rng(5)
+    k = rng.standard_normal((6, 1, 4)); v = rng.standard_normal((6, 1, 4)); q = rng.standard_normal((1, 1, 4))
+    a = orc.ragged_paged_attention_ref(q, _dense_pages(k, v, 8, [1]), [6], np.array([[1]]), [0, 1], [1], softmax_scale=1.0)
+    np.testing.assert_allclose(a[0, 0], softmax(q[0, 0] @ k[:, 0].T) @ v[:, 0], rtol=1e-12)
+    b = orc.ragged_paged_attention_ref(q, _dense_pages(v, k, 8, [1]), [6], np.array([[1]]), [0, 1], [1], softmax_scale=1.0)
+    np.testing.assert_allclose(b[0, 0], softmax(q[0, 0] @ v[:, 0].T) @ k[:, 0], rtol=1e-12)
+
+
+def test_chunked_prefill_and_decode_equal_rows_of_full_prefill():
+    rng = np.random.default_rng(6)
+    n, pg = 50, 8
+    k = rng.standard_normal((n, 2, 8)); v = rng.standard_normal((n, 2, 8)); q = rng.standard_normal((n, 4, 8))
+    table = rng.permutation(np.arange(1, 12))[:7]
+    pages = _dense_pages(k, v, pg, table)
+    full = orc.ragged_paged_attention_ref(q, pages, [n], table[None], [0, n], [1])
+    # chunk: rows 20..34 with context 35; decode: row 49 with context 50
+    chunk = orc.ragged_paged_attention_ref(q[20:35], pages, [35], table[None], [0, 15], [1])
+    np.testing.assert_allclose(chunk, full[20:35], rtol=1e-12)
+    dec = orc.ragged_paged_attention_ref(q[49:50], pages, [50], table[None], [0, 1], [1])
+    np.testing.assert_allclose(dec, full[49:50], rtol=1e-12)
+
+
+def test_page_permutation_invariance_and_padding_rows():
+    b = tl.make_batch(7, [17, 64, 130, 255], [1, 1, 8, 33], Hq=8, Hkv=2, D=64, page_size=16, num_pages=128,
+                      q_dtype=F32, kv_dtype=F32, pad_rows=3, pad_tokens=5)
+    base = tl.oracle_out(b)
+    assert np.all(base[43:] == 0)
+    rng = np.random.default_rng(0)
+    perm = np.concatenate([[0], 1 + rng.permutation(b.P - 1)])
+    kv2 = np.empty_like(b.kv_val); kv2[perm] = b.kv_val
+    got = orc.ragged_paged_attention_ref(b.q_val, kv2, b.context_lens, perm[b.block_tables], b.query_start_loc, b.num_seqs)
+    np.testing.assert_array_equal(got, base)
+    # flattened block tables (the v3 call passes pages_tables.reshape(-1)) give the same result
+    got = orc.ragged_paged_attention_ref(b.q_val, b.kv_val, b.context_lens, b.block_tables.reshape(-1), b.query_start_loc, b.num_seqs)
+    np.testing.assert_array_equal(got, base)
+
+
+def test_quantised_pages_equal_host_dequantised_pages():
+    for kv_dtype in (tl.FP8, tl.INT8):
+        b = tl.make_batch(8, [40, 100], [1, 7], Hq=4, Hkv=2, D=16, page_size=16, q_dtype=F32, kv_dtype=kv_dtype)
+        deq = b.kv_val * b.kv_scales.astype(np.float64)[:, None, :, None]
+        want = orc.ragged_paged_attention_ref(b.q_val, deq, b.context_lens, b.block_tables, b.query_start_loc, b.num_seqs)
+        np.testing.assert_allclose(tl.oracle_out(b), want, rtol=1e-12, atol=1e-14)
+
+
+def test_brute_force_scalar_loops_match():
+    # tiny case, written as scalar loops with no shared code
+    import math
+    rng = np.random.default_rng(9)
+    b = tl.make_batch(9, [5, 9], [2, 3], Hq=2, Hkv=1, D=4, page_size=4, q_dtype=F32, kv_dtype=F32)
+    got = tl.oracle_out(b, softmax_scale=0.7, sliding_window=4, logits_soft_cap=3.0)
+    for i, (ctx, ql) in enumerate([(5, 2), (9, 3)]):
+        for r in range(ql):
+            t = int(b.query_start_loc[i]) + r
+            pos = ctx - ql + r
+            for h in range(2):
+                ws, acc = [], np.zeros(4)
+                for j in range(ctx):
+                    if j > pos or j <= pos - 4:
+                        continue
+                    page = b.block_tables[i, j // 4]
+                    kk = b.kv_val[page, j % 4, 0]; vv = b.kv_val[page, j % 4, 1]
+                    s = 0.7 * sum(b.q_val[t, h, d] * kk[d] for d in range(4))
+                    ws.append((math.exp(3.0 * math.tanh(s / 3.0)), vv))
+                z = sum(w for w, _ in ws)
+                for w, vv in ws:
+                    acc += w / z * vv
+                np.testing.assert_allclose(got[t, h], acc, rtol=1e-12)
