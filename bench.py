@@ -38,16 +38,21 @@ def parse_args():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
-    ap.add_argument("--decode-chunk", type=int, default=0)
+    ap.add_argument("--decode-wgs", type=int, default=0)
     ap.add_argument("--max-splits", type=int, default=0)
+    ap.add_argument("--sequential-pages", action="store_true", help="experiment: block tables in pool order")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy, so a counter run shows what a known-size kernel reads")
+    ap.add_argument("--decode-wpb", type=int, default=0)
+    ap.add_argument("--decode-occ", type=int, default=0)
     return ap.parse_args()
 
 
-def build_workload(name, seed):
+def build_workload(name, seed, sequential=False):
     from easydel_amd import workloads
 
     if name == "c2":
-        return workloads.config2_llama_decode(seed)
+        return workloads.config2_llama_decode(seed, shuffle_pages=not sequential)
     if name == "c4-fp8":
         return workloads.config4_quantised_decode(seed, "fp8")
     return workloads.config4_quantised_decode(seed, "int8")
@@ -92,7 +97,7 @@ def cpu_baseline(w, tens, sample_seqs):
     while True:
         out = run()
         reps += 1
-        if time.perf_counter() - t0 > 5.0 or reps >= 5:
+        if time.perf_counter() - t0 > 10.0:
             break
     dt = (time.perf_counter() - t0) / reps
     tokens = int(w.q_lens[idx].sum())
@@ -119,13 +124,17 @@ def main():
     from easydel_amd import _lib, kernels, workloads
 
     _lib.load()
-    if args.decode_chunk:
-        _lib.set_tunable("decode_chunk", args.decode_chunk)
+    if args.decode_wgs:
+        _lib.set_tunable("decode_wgs", args.decode_wgs)
     if args.max_splits:
         _lib.set_tunable("max_splits", args.max_splits)
+    if args.decode_wpb:
+        _lib.set_tunable("decode_wpb", args.decode_wpb)
+    if args.decode_occ:
+        _lib.set_tunable("decode_occ", args.decode_occ)
 
     dev = torch.device("cuda:0")
-    w = build_workload(args.workload, args.seed)
+    w = build_workload(args.workload, args.seed, args.sequential_pages)
     tens = workloads.device_tensors(w, dev, seed=args.seed)
     quant = w.kv_dtype in ("fp8", "int8")
     out = torch.empty_like(tens["query"])
@@ -141,6 +150,14 @@ def main():
                                               tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
                                               tens["distribution"], softmax_scale=w.softmax_scale,
                                               sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap, out=out)
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)  # elementwise copy kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -215,8 +232,8 @@ def main():
     }
 
     if not args.no_cpu_baseline:
-        # size the sample for roughly 10-30 s of host work: ~0.35 GFLOP-equivalents per cached token-head here
-        sample = args.cpu_sample_seqs or max(8, min(w.S, 32))
+        # the whole batch fits the host here; it is re-run for about 10 s
+        sample = args.cpu_sample_seqs or w.S
         base, cpu_out, rows = cpu_baseline(w, tens, sample)
         step()
         torch.cuda.synchronize()

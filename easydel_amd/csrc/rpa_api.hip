@@ -17,9 +17,11 @@ int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const in
 namespace {
 
 thread_local char g_err[512] = "";
-std::atomic<int> g_decode_chunk{512};
-std::atomic<int> g_max_splits{32};
+std::atomic<int> g_max_splits{0};   // 0 = sized from the shapes
+std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are resident at once
 std::atomic<int> g_force_generic{0};
+std::atomic<int> g_decode_wpb{0};
+std::atomic<int> g_decode_occ{0};
 std::atomic<int> g_stages{7};  // bit 0: decode kernel, bit 1: prefill / large-row kernel, bit 2: merge
 
 int fail(int code, const char* fmt, ...) {
@@ -41,15 +43,21 @@ size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 size_t part_o_bytes(int T, int Hq, int D) { return align256((size_t)T * Hq * D * 4); }
 size_t part_ml_bytes(int T, int Hq) { return align256((size_t)T * Hq * 2 * 4); }
 
-int static_splits(int M, int page_size) {
-  const int chunk = g_decode_chunk.load();
-  long span = (long)M * page_size;
-  long n = (span + chunk - 1) / chunk;
-  const int cap = g_max_splits.load();
-  if (n > cap) n = cap;
-  if (n < 1) n = 1;
-  return (int)n;
+// Partial slots per sequence the workspace is sized for: enough to spread one maximal sequence over
+// 256-token pieces, capped so the partial buffers stay within ~256 MiB, never fewer than 2.
+int static_splits(int T, int M, int page_size, int Hq, int D) {
+  const int forced = g_max_splits.load();
+  if (forced > 0) return forced < 2 ? 2 : forced;
+  long want = ((long)M * page_size + 255) / 256 + 1;
+  const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
+  long cap = (long)(((size_t)256 << 20) / per);
+  if (cap > rpa::kMaxSplitsCap) cap = rpa::kMaxSplitsCap;
+  if (want > cap) want = cap;
+  if (want < 2) want = 2;
+  return (int)want;
 }
+
+size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + S + 1 + rpa::kMaxDecodeWgs) * 4); }
 
 }  // namespace
 
@@ -61,17 +69,15 @@ const char* rpa_last_error(void) { return g_err; }
 
 int rpa_set_tunable(const char* name, int value) {
   if (!name) return -1;
-  if (!strcmp(name, "decode_chunk")) {
-    if (value < 64) value = 64;
-    value = (value + 63) & ~63;
-    return g_decode_chunk.exchange(value);
-  }
   if (!strcmp(name, "max_splits")) {
-    if (value < 1) value = 1;
+    if (value < 0) value = 0;
     if (value > rpa::kMaxSplitsCap) value = rpa::kMaxSplitsCap;
     return g_max_splits.exchange(value);
   }
+  if (!strcmp(name, "decode_wgs")) return g_decode_wgs.exchange(value < 0 ? 0 : value);
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
+  if (!strcmp(name, "decode_wpb")) return g_decode_wpb.exchange(value);
+  if (!strcmp(name, "decode_occ")) return g_decode_occ.exchange(value);
   if (!strcmp(name, "stages")) return g_stages.exchange(value & 7);
   return -1;
 }
@@ -108,10 +114,10 @@ int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* va
 
 size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int q_dtype,
                                      int kv_dtype) {
-  (void)S; (void)Hkv; (void)q_dtype; (void)kv_dtype;
-  if (T <= 0 || M <= 0 || page_size <= 0 || Hq <= 0 || D <= 0) return 256;
-  const int splits = static_splits(M, page_size);
-  return (size_t)splits * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) + 256;
+  (void)Hkv; (void)q_dtype; (void)kv_dtype;
+  if (T <= 0 || S <= 0 || M <= 0 || page_size <= 0 || Hq <= 0 || D <= 0) return 256;
+  const int splits = static_splits(T, M, page_size, Hq, D);
+  return (size_t)splits * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) + plan_bytes(S) + 256;
 }
 
 int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages, const float* kv_scales,
@@ -148,23 +154,27 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.window = sliding_window > 0 ? sliding_window : 0;
   p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
-  p.chunk_target = g_decode_chunk.load();
-  p.max_splits = 1;
+  p.decode_wgs = g_decode_wgs.load();
+  p.decode_wpb = g_decode_wpb.load();
+  p.decode_occ = g_decode_occ.load();
+  p.max_splits = 2;
   p.mfma_path = (!g_force_generic.load() && rpa::decode_supported(p)) ? 1 : 0;
 
   hipStream_t s = (hipStream_t)stream;
   const int stages = g_stages.load();
   if (p.mfma_path) {
-    const size_t po = part_o_bytes(T, Hq, D), pml = part_ml_bytes(T, Hq);
-    int splits = static_splits(M, page_size);
-    const size_t usable = workspace_bytes > 256 ? workspace_bytes - 256 : 0;
-    if (!workspace || usable < po + pml)
-      return fail(RPA_ERR_WORKSPACE, "rpa_ragged_paged_attention: workspace %zu bytes < %zu needed for one split", workspace_bytes, po + pml + 256);
+    const size_t po = part_o_bytes(T, Hq, D), pml = part_ml_bytes(T, Hq), pb = plan_bytes(S);
+    int splits = static_splits(T, M, page_size, Hq, D);
+    const size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
+    if (!workspace || usable < 2 * (po + pml))
+      return fail(RPA_ERR_WORKSPACE, "rpa_ragged_paged_attention: workspace %zu bytes < %zu needed for two partial slots",
+                  workspace_bytes, 2 * (po + pml) + pb + 256);
     if ((size_t)splits * (po + pml) > usable) splits = (int)(usable / (po + pml));
     p.max_splits = splits;
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
-    p.part_o = (float*)base;
-    p.part_ml = (float*)(base + (size_t)splits * po);
+    p.plan = (int32_t*)base;
+    p.part_o = (float*)(base + pb);
+    p.part_ml = (float*)(base + pb + (size_t)splits * po);
     int err = 0;
     if (stages & 1) err = rpa::launch_attn_decode(s, p);
     if (err) return hip_fail(err, "decode kernel launch");

@@ -1,9 +1,13 @@
-// Split-K decode attention on MFMA: one wavefront per (sequence, KV head, key chunk).
+// Split-K decode attention on MFMA, persistent and evenly split: one wavefront per KV head.
 //
 // Serves sequences whose query rows for one KV head (q_len * group) fit one 16-row MFMA block:
-// plain decode (q_len = 1) and short speculative / multi-token rows.  A workgroup holds WPB
-// waves working on WPB adjacent KV heads of the same (sequence, chunk), so together they sweep
-// whole token rows of a page; each wave streams its own K_h|V_h spans (contiguous in the
+// plain decode (q_len = 1) and short speculative / multi-token rows.  The keys of all such
+// sequences are laid end to end (a small plan kernel computes the prefix sums on the device); each
+// of the resident workgroups takes one equal span of that stream, whatever sequence boundaries fall
+// inside it, so every CU streams the same number of bytes and no launch-time shape depends on the
+// batch.  A sequence cut by a span boundary leaves partial results that the merge kernel combines.
+// A workgroup holds WPB waves working on WPB adjacent KV heads of the same keys, so together they
+// sweep whole token rows of a page; each wave streams its own K_h|V_h spans (contiguous in the
 // [page][token][2*Hkv][D] layout) with 128-bit loads into registers one tile ahead, stages them
 // in a wave-private swizzled LDS tile, and reads them back in MFMA operand order:
 //     S^T[token][row] = K[token][:] . Q[row][:]          v_mfma_f32_16x16x32_bf16, k = head dim
@@ -17,8 +21,39 @@
 
 namespace rpa {
 
-template <int D, int KVT, int TT, int WPB>
-__global__ __launch_bounds__(64 * WPB) void attn_decode_kernel(AttnParams p) {
+// Per-workgroup piece of the flattened key stream: a token range of one sequence.
+struct Piece {
+  int i, q0, q_len, ctx;
+  int t_begin, t_end;  // keys [t_begin, t_end) of sequence i
+  int slot;            // which partial slot of the sequence this piece fills
+  int single;          // the sequence lies in one piece: write the final output directly
+  int flat_end;        // flat position where the piece ends
+};
+
+// Finds the sequence that holds flat position `pos` (searching upwards from i) and cuts the piece
+// [pos, min(span_end, end of that sequence)) out of it.  pos < span_end <= W.
+__device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* __restrict__ P, int i, int pos,
+                                            int span_end, int Q) {
+  int p1 = P[i + 1];
+  while (p1 <= pos) {  // sequences without decode-class work have zero length
+    ++i;
+    p1 = P[i + 1];
+  }
+  const int p0 = P[i];
+  const SeqPlan sp = seq_plan(p, i);
+  Piece pc;
+  pc.i = i; pc.q0 = sp.q0; pc.q_len = sp.q_len; pc.ctx = sp.ctx;
+  pc.flat_end = min(span_end, p1);
+  pc.t_begin = sp.lo + (pos - p0);
+  pc.t_end = min(sp.hi, sp.lo + (pc.flat_end - p0));
+  const int j_first = p0 / Q;
+  pc.slot = pos / Q - j_first;
+  pc.single = (j_first == (p1 - 1) / Q);
+  return pc;
+}
+
+template <int D, int KVT, int TT, int WPB, int OCC>
+__global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
   constexpr int HB = 2 * RK;           // K_h | V_h span of one token
@@ -36,34 +71,69 @@ __global__ __launch_bounds__(64 * WPB) void attn_decode_kernel(AttnParams p) {
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int i = blockIdx.x;
-  const int c = blockIdx.y;
-  const int h = blockIdx.z * WPB + wave;
+  const int h = blockIdx.y * WPB + wave;
   if (h >= p.Hkv) return;
-  const SeqPlan sp = seq_plan(p, i);
-  if (!sp.live || !sp.small_rows || c >= sp.n_chunks) return;
+
+  // ---- this workgroup's span of the flattened key stream --------------------------------------
+  const int32_t* __restrict__ plan = p.plan;
+  const int W = plan[0], Q = plan[1];
+  const int32_t* __restrict__ P = plan + kPlanHeader;
+  if ((int64_t)blockIdx.x * Q >= W) return;
+  const int span_begin = blockIdx.x * Q;
+  const int span_end = min(W, span_begin + Q);
 
   const int G = p.group;
-  const int rows = sp.q_len * G;
-  const int t_begin = sp.lo + c * sp.chunk;
-  const int t_end = min(sp.hi, t_begin + sp.chunk);
-  const int n_tiles = (t_end - t_begin + TT - 1) / TT;
-
   const int n = lane & 15;   // query row (column of S^T / O^T)
   const int g4 = lane >> 4;  // token group / k group
+  const int pg = p.page_size;
+
+  // ---- tile addressing (independent of the piece) ---------------------------------------------
+  unsigned char* lds_k = lds_all + wave * (TT * HB);
+  unsigned char* lds_v = lds_k + TT * RK;
+  const int sub = lane / LPT;
+  const int c32 = lane % LPT;
+  const bool is_v = c32 >= NCH;
+  const int cc = is_v ? c32 - NCH : c32;
+  const char* pages = (const char*)p.kv_pages;
+  const int64_t lane_goff = (int64_t)h * HB + c32 * 16 + (int64_t)sub * p.token_stride;
+
+  u32x4 stage[NLD];
+  auto page_of = [&](int seq, int tok) -> int {
+    int pgid = p.block_tables[(int64_t)seq * p.M + tok / pg];
+    pgid = __builtin_amdgcn_readfirstlane(pgid);
+    return min(max(pgid, 0), p.P - 1);
+  };
+  auto issue = [&](int tb, int page) {
+    const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride + lane_goff;
+#pragma unroll
+    for (int u = 0; u < NLD; ++u) stage[u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
+  };
+
+  const bool has_cap = p.softcap > 0.f;
+  const float cap_out = p.softcap * 1.4426950408889634f;
+  const float cap_in = has_cap ? p.scale / p.softcap : 0.f;
+
+  Piece cur = make_piece(p, P, plan[kPlanHeader + p.S + 1 + blockIdx.x], span_begin, span_end, Q);
+  int page_cur = page_of(cur.i, cur.t_begin);
+  issue(cur.t_begin, page_cur);  // first tile in flight before anything else is set up
+
+  for (;;) {
+  const int rows = cur.q_len * G;
+  const int t_begin = cur.t_begin;
+  const int n_tiles = (cur.t_end - t_begin + TT - 1) / TT;
 
   // ---- per-lane row limits -------------------------------------------------------------
   const int r_tok = (n < rows) ? n / G : 0;           // padded rows shadow row 0 and are never stored
   const int r_head = (n < rows) ? n - r_tok * G : 0;
-  const int pos = sp.ctx - sp.q_len + r_tok;
-  const int row_hi = min(pos + 1, sp.ctx);            // exclusive
+  const int pos = cur.ctx - cur.q_len + r_tok;
+  const int row_hi = min(pos + 1, cur.ctx);            // exclusive
   const int row_lo = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
-  const int vis_lo = (p.window > 0) ? max(sp.ctx - sp.q_len - p.window + 1, 0) : 0;  // lowest key any row sees
+  const int vis_lo = (p.window > 0) ? max(cur.ctx - cur.q_len - p.window + 1, 0) : 0;  // lowest key any row sees
 
   // ---- Q as B operands -----------------------------------------------------------------
   bf16x8 qf[NKK];
   {
-    const char* qrow = (const char*)p.q + ((int64_t)(sp.q0 + r_tok) * p.Hq + (h * G + r_head)) * D * 2;
+    const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok) * p.Hq + (h * G + r_head)) * D * 2;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
       // bf16 pages: step kk covers dims 32kk + 8g4 + e.  8-bit pages: a 16-byte K chunk holds 16
@@ -75,48 +145,29 @@ __global__ __launch_bounds__(64 * WPB) void attn_decode_kernel(AttnParams p) {
     }
   }
 
-  // ---- tile addressing -----------------------------------------------------------------
-  unsigned char* lds_k = lds_all + wave * (TT * HB);
-  unsigned char* lds_v = lds_k + TT * RK;
-  const int sub = lane / LPT;
-  const int c32 = lane % LPT;
-  const bool is_v = c32 >= NCH;
-  const int cc = is_v ? c32 - NCH : c32;
-  const int32_t* bt = p.block_tables + (int64_t)i * p.M;
-  const char* pages = (const char*)p.kv_pages;
-  const int64_t lane_goff = (int64_t)h * HB + c32 * 16 + (int64_t)sub * p.token_stride;
-  const int pg = p.page_size;
-
-  u32x4 stage[NLD];
-  auto page_of = [&](int tok) -> int {
-    int pgid = bt[tok / pg];
-    pgid = __builtin_amdgcn_readfirstlane(pgid);
-    return min(max(pgid, 0), p.P - 1);
-  };
-  auto issue = [&](int tile, int page) {
-    const int tb = t_begin + tile * TT;
-    const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride + lane_goff;
-#pragma unroll
-    for (int u = 0; u < NLD; ++u) stage[u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
-  };
+  // ---- the piece after this one (its first tile is prefetched during this piece's last tile) ---
+  const bool has_next = cur.flat_end < span_end;
+  Piece nxt = cur;
+  int page_nxt = 0;
+  if (has_next) {
+    nxt = make_piece(p, P, cur.i + 1, cur.flat_end, span_end, Q);
+    page_nxt = page_of(nxt.i, nxt.t_begin);
+  }
 
   float m_run = -INFINITY, l_run = 0.f;
   f32x4 o_acc[DPL];
 #pragma unroll
   for (int rt = 0; rt < DPL; ++rt) o_acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  int page_cur = page_of(t_begin);
-  issue(0, page_cur);
-
   for (int tile = 0; tile < n_tiles; ++tile) {
     const int tb = t_begin + tile * TT;
     // ---- registers -> LDS (zero rows past the context end or left of every row's window, so stale
     //      or null-page bytes cannot reach P.V as 0 * NaN)
-    if (tb + TT > sp.ctx || tb < vis_lo) {
+    if (tb + TT > cur.ctx || tb < vis_lo) {
 #pragma unroll
       for (int u = 0; u < NLD; ++u) {
         const int tok = tb + u * TPI + sub;
-        if (tok >= sp.ctx || tok < vis_lo) stage[u] = (u32x4){0u, 0u, 0u, 0u};
+        if (tok >= cur.ctx || tok < vis_lo) stage[u] = (u32x4){0u, 0u, 0u, 0u};
       }
     }
 #pragma unroll
@@ -133,8 +184,11 @@ __global__ __launch_bounds__(64 * WPB) void attn_decode_kernel(AttnParams p) {
     }
     // ---- prefetch the next tile into registers ---------------------------------------------
     if (tile + 1 < n_tiles) {
-      page_cur = page_of(tb + TT);
-      issue(tile + 1, page_cur);
+      page_cur = page_of(cur.i, tb + TT);
+      issue(tb + TT, page_cur);
+    } else if (has_next) {
+      page_cur = page_nxt;
+      issue(nxt.t_begin, page_nxt);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -164,15 +218,20 @@ __global__ __launch_bounds__(64 * WPB) void attn_decode_kernel(AttnParams p) {
     }
 
     // ---- online softmax (log2 domain) -------------------------------------------------------
+    if (has_cap) {
+#pragma unroll
+      for (int st = 0; st < NS; ++st)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s_acc[st][j] = fast_tanh(s_acc[st][j] * (cap_in * k_scale));
+    }
+    const float sc_mul = has_cap ? cap_out : p.scale_log2 * k_scale;
     float mx = -INFINITY;
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int tok = tb + st * 16 + 4 * g4 + j;
-        float s = s_acc[st][j];
-        if (p.softcap > 0.f) s = p.softcap * 1.4426950408889634f * fast_tanh(s * (p.scale * k_scale / p.softcap));
-        else s *= p.scale_log2 * k_scale;
+        float s = s_acc[st][j] * sc_mul;
         s = (tok >= row_lo && tok < row_hi) ? s : -INFINITY;
         s_acc[st][j] = s;
         mx = fmaxf(mx, s);
@@ -269,51 +328,136 @@ __global__ __launch_bounds__(64 * WPB) void attn_decode_kernel(AttnParams p) {
   // ---- epilogue: lane (n, g4) holds dims [4*DPL*g4, 4*DPL*(g4+1)) of row n, ordered j*DPL + rt ----
   float l_tot = l_run + __shfl_xor(l_run, 16);
   l_tot += __shfl_xor(l_tot, 32);
-  if (n >= rows) return;
-  const int tok_out = sp.q0 + r_tok;
-  const int head_out = h * G + r_head;
-  const int d_base = 4 * DPL * g4;
-  if (sp.n_chunks == 1) {
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D + d_base;
+  if (n < rows) {
+    const int tok_out = cur.q0 + r_tok;
+    const int head_out = h * G + r_head;
+    const int d_base = 4 * DPL * g4;
+    if (cur.single) {
+      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+      uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D + d_base;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < 4; ++j) {
 #pragma unroll
-      for (int rt = 0; rt < DPL; rt += 2) {
-        *(uint32_t*)(orow + j * DPL + rt) = pack_bf16(o_acc[rt][j] * inv, o_acc[rt + 1][j] * inv);
+        for (int rt = 0; rt < DPL; rt += 2) {
+          *(uint32_t*)(orow + j * DPL + rt) = pack_bf16(o_acc[rt][j] * inv, o_acc[rt + 1][j] * inv);
+        }
+      }
+    } else {
+      const int64_t slot = ((int64_t)cur.slot * p.T + tok_out) * p.Hq + head_out;
+      float* prow = p.part_o + slot * D + d_base;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int rt = 0; rt < DPL; ++rt) prow[j * DPL + rt] = o_acc[rt][j];
+      }
+      if (g4 == 0) {
+        p.part_ml[slot * 2 + 0] = m_run;
+        p.part_ml[slot * 2 + 1] = l_tot;
       }
     }
-  } else {
-    const int64_t slot = ((int64_t)c * p.T + tok_out) * p.Hq + head_out;
-    float* prow = p.part_o + slot * D + d_base;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int rt = 0; rt < DPL; ++rt) prow[j * DPL + rt] = o_acc[rt][j];
+  }
+  if (!has_next) break;
+  cur = nxt;
+  }  // pieces
+}
+
+// One block: exclusive prefix sum of the 64-token-rounded key spans of the decode-class sequences
+// (the flattened key stream), the per-workgroup span length Q, and each workgroup's first sequence.
+__global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
+  __shared__ int part[1024];
+  __shared__ int s_Q;
+  int32_t* plan = p.plan;
+  int32_t* P = plan + kPlanHeader;
+  const int S = p.S, tid = threadIdx.x;
+  const int per = (S + 1023) / 1024;
+  const int i0 = min(S, tid * per), i1 = min(S, i0 + per);
+  auto span_of = [&](int i) -> int {
+    const SeqPlan sp = seq_plan(p, i);
+    if (!sp.live || !sp.small_rows) return 0;
+    return (sp.hi - sp.lo + 63) & ~63;
+  };
+  int sum = 0;
+  for (int i = i0; i < i1; ++i) sum += span_of(i);
+  part[tid] = sum;
+  __syncthreads();
+  for (int off = 1; off < 1024; off <<= 1) {  // inclusive Hillis-Steele scan
+    const int v = (tid >= off) ? part[tid - off] : 0;
+    __syncthreads();
+    part[tid] += v;
+    __syncthreads();
+  }
+  int run = part[tid] - sum;
+  for (int i = i0; i < i1; ++i) {
+    P[i] = run;
+    run += span_of(i);
+  }
+  const int W = part[1023];
+  if (tid == 0) {
+    P[S] = W;
+    // span per workgroup: even split, but never so small that a sequence needs more than max_splits pieces
+    int q = ((W + p.n_wg - 1) / p.n_wg + 63) & ~63;
+    const int q_min = (((p.M * p.page_size + 64) + (p.max_splits - 2)) / (p.max_splits - 1) + 63) & ~63;
+    q = max(max(q, q_min), 256);
+    plan[0] = W;
+    plan[1] = q;
+    s_Q = q;
+  }
+  __threadfence_block();
+  __syncthreads();
+  // first sequence of every workgroup: the last i with P[i] <= j*Q (the kernel then skips empty ones)
+  const int Q = s_Q;
+  for (int j = tid; j < p.n_wg; j += 1024) {
+    const int64_t target = (int64_t)j * Q;
+    int lo = 0, hi = S;  // invariant: P[lo] <= target (P[0] = 0); answer in [lo, hi)
+    if (target >= W) { plan[kPlanHeader + S + 1 + j] = 0; continue; }
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (P[mid] <= target) lo = mid; else hi = mid;
     }
-    if (g4 == 0) {
-      p.part_ml[slot * 2 + 0] = m_run;
-      p.part_ml[slot * 2 + 1] = l_tot;
-    }
+    plan[kPlanHeader + S + 1 + j] = lo;
   }
 }
 
-template <int D, int KVT, int TT, int WPB>
-static int launch_one(hipStream_t stream, const AttnParams& p) {
-  dim3 grid(p.S, p.max_splits, (p.Hkv + WPB - 1) / WPB), block(64 * WPB);
-  hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB>), grid, block, 0, stream, p);
+template <int D, int KVT, int TT, int WPB, int OCC>
+static int launch_one(hipStream_t stream, AttnParams p) {
+  // persistent grid: as many workgroups as are resident at once, per KV-head group
+  static int resident = 0;
+  if (resident == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, OCC>, 64 * WPB, 0) != hipSuccess)
+      return (int)hipGetLastError();
+    resident = max(1, cus * max(1, per_cu));
+  }
+  const int head_groups = (p.Hkv + WPB - 1) / WPB;
+  int n_wg = resident / head_groups;
+  if (p.decode_wgs > 0) n_wg = p.decode_wgs;
+  n_wg = max(1, min(n_wg, kMaxDecodeWgs));
+  p.n_wg = n_wg;
+  hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(1024), 0, stream, p);
+  hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, OCC>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();
+}
+
+template <int D, int KVT, int TT, int WPB>
+static int launch_occ(hipStream_t stream, const AttnParams& p) {
+  // waves per SIMD the register allocator must leave room for; 0 = compiler's choice
+  if (p.decode_occ == 4) return launch_one<D, KVT, TT, WPB, 4>(stream, p);
+  if (p.decode_occ == 3) return launch_one<D, KVT, TT, WPB, 3>(stream, p);
+  return launch_one<D, KVT, TT, WPB, 1>(stream, p);
 }
 
 template <int D, int KVT, int TT>
 static int launch_wpb(hipStream_t stream, const AttnParams& p) {
   constexpr int tile_bytes = TT * 2 * D * ElemBytes<KVT>::v;
+  const int want = p.decode_wpb > 0 ? p.decode_wpb : 8;
   if constexpr (tile_bytes * 8 <= 65536) {
-    if (p.Hkv >= 8) return launch_one<D, KVT, TT, 8>(stream, p);
+    if (p.Hkv >= 8 && want >= 8) return launch_occ<D, KVT, TT, 8>(stream, p);
   }
-  if (p.Hkv >= 4) return launch_one<D, KVT, TT, 4>(stream, p);
-  if (p.Hkv >= 2) return launch_one<D, KVT, TT, 2>(stream, p);
-  return launch_one<D, KVT, TT, 1>(stream, p);
+  if (p.Hkv >= 4 && want >= 4) return launch_occ<D, KVT, TT, 4>(stream, p);
+  if (p.Hkv >= 2 && want >= 2) return launch_occ<D, KVT, TT, 2>(stream, p);
+  return launch_occ<D, KVT, TT, 1>(stream, p);
 }
 
 template <int KVT>

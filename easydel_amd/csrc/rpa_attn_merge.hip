@@ -1,59 +1,85 @@
 // Split-K merge: combines the decode kernel's per-chunk partial outputs, and zero-fills the
 // output rows of padded tokens so the whole [T, Hq, D] result is defined.
+//
+// One wavefront per (token, query head).  Lanes load the pieces' (max, sum) pairs, a cross-lane
+// max gives the global max, each lane turns its pair into a weight; the partial rows are then
+// accumulated with the weight broadcast from its lane, every lane owning D/64 output dims
+// (coalesced row reads).
 #include "rpa_common.h"
 
 namespace rpa {
 
 template <int QT>
 __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
-  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);  // (token, head) index
+  if (pair >= p.T * p.Hq) return;
+  const int t = pair / p.Hq, hq = pair - t * p.Hq;
   const int n_live = p.num_seqs[0];
   const int D = p.D;
-  const int units = p.Hq * (D / 4);  // D % 4 == 0 is checked by the host
-  bool zero = false, merge = false;
-  SeqPlan sp;
+  bool zero = false;
+  int n_pieces = 0;
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) {
     zero = true;
   } else {
-    sp = seq_plan(p, find_seq(p.qsl, n_live, t));
+    const int i = find_seq(p.qsl, n_live, t);
+    const SeqPlan sp = seq_plan(p, i);
     if (!sp.live) zero = true;
-    else merge = p.mfma_path && sp.small_rows && sp.n_chunks > 1;
+    else if (p.mfma_path && sp.small_rows) n_pieces = decode_pieces(p.plan, i);
   }
+  const bool merge = n_pieces > 1;
   if (!zero && !merge) return;
-  for (int u = threadIdx.x; u < units; u += blockDim.x) {
-    const int hq = u / (D / 4), dv = u - hq * (D / 4);
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (merge) {
-      float m = -INFINITY;
-      for (int c = 0; c < sp.n_chunks; ++c)
-        m = fmaxf(m, p.part_ml[(((int64_t)c * p.T + t) * p.Hq + hq) * 2]);
-      const float m_use = (m == -INFINITY) ? 0.f : m;
-      float l = 0.f;
-      for (int c = 0; c < sp.n_chunks; ++c) {
-        const int64_t slot = ((int64_t)c * p.T + t) * p.Hq + hq;
-        const float w = __builtin_amdgcn_exp2f(p.part_ml[slot * 2] - m_use);
-        l += w * p.part_ml[slot * 2 + 1];
-        const float4 o = ((const float4*)(p.part_o + slot * D))[dv];
-        acc.x += w * o.x; acc.y += w * o.y; acc.z += w * o.z; acc.w += w * o.w;
+
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, lane+128, lane+192
+  float inv = 0.f;
+  if (merge) {
+    const int64_t stride = (int64_t)p.T * p.Hq;  // slots between consecutive pieces
+    const int64_t slot0 = (int64_t)t * p.Hq + hq;
+    float m = -INFINITY;
+    for (int c = lane; c < n_pieces; c += 64) m = fmaxf(m, p.part_ml[(slot0 + c * stride) * 2]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    const float m_use = (m == -INFINITY) ? 0.f : m;
+    float l = 0.f;
+    for (int base = 0; base < n_pieces; base += 64) {
+      const int c_mine = base + lane;
+      float w_c = 0.f;
+      if (c_mine < n_pieces) {
+        const float2 ml = *(const float2*)(p.part_ml + (slot0 + c_mine * stride) * 2);
+        w_c = __builtin_amdgcn_exp2f(ml.x - m_use);
+        l += w_c * ml.y;
       }
-      const float inv = l > 0.f ? 1.f / l : 0.f;
-      acc.x *= inv; acc.y *= inv; acc.z *= inv; acc.w *= inv;
+      const int cnt = min(64, n_pieces - base);
+      for (int c = 0; c < cnt; ++c) {
+        const float w = __shfl(w_c, c);
+        const float* row = p.part_o + (slot0 + (base + c) * stride) * D;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int d = lane + 64 * k;
+          if (d < D) acc[k] = fmaf(w, row[d], acc[k]);
+        }
+      }
     }
-    const int64_t o = ((int64_t)t * p.Hq + hq) * D + dv * 4;
-    if constexpr (QT == RPA_F32) {
-      *(float4*)((float*)p.out + o) = acc;
-    } else {
-      uint2 r;
-      r.x = (uint32_t)float_to_bf16_bits(acc.x) | ((uint32_t)float_to_bf16_bits(acc.y) << 16);
-      r.y = (uint32_t)float_to_bf16_bits(acc.z) | ((uint32_t)float_to_bf16_bits(acc.w) << 16);
-      *(uint2*)((uint16_t*)p.out + o) = r;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    inv = l > 0.f ? 1.f / l : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int d = lane + 64 * k;
+    if (d < D) {
+      const int64_t o = ((int64_t)t * p.Hq + hq) * D + d;
+      const float r = acc[k] * inv;
+      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
+      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
     }
   }
 }
 
 int launch_attn_merge(hipStream_t stream, const AttnParams& p) {
-  if (p.q_dtype == RPA_F32) hipLaunchKernelGGL((attn_merge_kernel<RPA_F32>), dim3(p.T), dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL((attn_merge_kernel<RPA_BF16>), dim3(p.T), dim3(256), 0, stream, p);
+  const int blocks = (p.T * p.Hq + 3) / 4;
+  if (p.q_dtype == RPA_F32) hipLaunchKernelGGL((attn_merge_kernel<RPA_F32>), dim3(blocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((attn_merge_kernel<RPA_BF16>), dim3(blocks), dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }
 

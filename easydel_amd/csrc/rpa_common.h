@@ -9,7 +9,9 @@ namespace rpa {
 
 constexpr int kWave = 64;
 constexpr int kRowBlock = 16;      // MFMA M/N extent: rows (token, group-head pairs) per wave
-constexpr int kMaxSplitsCap = 64;  // hard upper bound on split-K partials per sequence
+constexpr int kMaxSplitsCap = 256;   // hard upper bound on split-K partials per sequence
+constexpr int kPlanHeader = 16;      // ints before the prefix array in the decode plan
+constexpr int kMaxDecodeWgs = 4096;  // persistent decode workgroups per KV-head group
 
 // Everything a kernel needs, passed by value.
 struct AttnParams {
@@ -23,6 +25,8 @@ struct AttnParams {
   void* out;
   float* part_o;   // [max_splits][T][Hq][D]
   float* part_ml;  // [max_splits][T][Hq][2]  (running max in log2 units, running sum)
+  int32_t* plan;   // decode plan: [0] = W (flattened keys), [1] = Q (keys per workgroup), then at kPlanHeader:
+                   // P[S+1] exclusive prefix of per-sequence key spans, then first_seq[n_wg]
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
   int64_t token_stride;  // bytes between consecutive tokens of a page = C*D*elem
   int64_t page_stride;   // bytes between pages
@@ -31,18 +35,19 @@ struct AttnParams {
   float scale_log2;  // softmax scale * log2(e)
   int window;        // <= 0: none
   float softcap;     // <= 0: none
-  int max_splits;    // >= 1
-  int chunk_target;  // tokens, multiple of 64
+  int max_splits;    // >= 2: most partial slots one sequence may use
+  int n_wg;          // persistent decode workgroups per KV-head group
+  int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
+  int decode_wpb;    // waves (KV heads) per decode workgroup, 0 = default
+  int decode_occ;    // waves per SIMD the decode kernel is compiled for, 0 = compiler's choice
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
 };
 
-// Per-sequence work plan.  Every kernel derives it from device metadata with this one function,
-// so producer (attention) and consumer (merge) always agree on who wrote what.
+// Per-sequence facts.  Every kernel derives them from device metadata with this one function, so the
+// producers (attention kernels) and the consumer (merge) always agree on who wrote what.
 struct SeqPlan {
   int q0, q_len, ctx;
   int lo, hi;       // key range any row of the sequence may see, lo rounded down to 64 tokens
-  int chunk;        // tokens per split
-  int n_chunks;     // number of splits that hold data
   bool live;        // has queries and keys
   bool small_rows;  // q_len * group <= 16: served by the split-K decode kernel
 };
@@ -62,13 +67,16 @@ __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
     s.lo = first > 0 ? (first & ~63) : 0;
   }
   s.small_rows = (s.q_len * p.group <= kRowBlock);
-  int span = s.hi - s.lo;
-  if (span < 1) span = 1;
-  int per = (span + p.max_splits - 1) / p.max_splits;
-  per = (per + 63) & ~63;
-  s.chunk = per > p.chunk_target ? per : p.chunk_target;
-  s.n_chunks = (span + s.chunk - 1) / s.chunk;
   return s;
+}
+
+// Partial slots the decode kernel filled for sequence i (0 or 1: the output row is already final).
+// P is the exclusive prefix of key spans in the decode plan, Q the span handled per workgroup.
+__device__ __forceinline__ int decode_pieces(const int32_t* __restrict__ plan, int i) {
+  const int Q = plan[1];
+  const int p0 = plan[kPlanHeader + i], p1 = plan[kPlanHeader + i + 1];
+  if (p1 <= p0) return 0;
+  return (p1 - 1) / Q - p0 / Q + 1;
 }
 
 // Largest i in [0, n) with qsl[i] <= t (qsl non-decreasing); callers guarantee qsl[0] <= t < qsl[n].

@@ -99,12 +99,12 @@ class Workload:
         return 4 * self.Hq * self.D * pairs
 
 
-def _tables(rng, context_lens, page_size, num_pages, max_pages):
+def _tables(rng, context_lens, page_size, num_pages, max_pages, shuffle=True):
     """Consecutive slices of one seeded permutation of pages 1..P-1 (no page shared)."""
     need = -(-context_lens.astype(np.int64) // page_size)
     if need.sum() > num_pages - 1:
         raise ValueError(f"pool of {num_pages} pages cannot hold {int(need.sum())} live pages")
-    perm = rng.permutation(np.arange(1, num_pages, dtype=np.int32))
+    perm = rng.permutation(np.arange(1, num_pages, dtype=np.int32)) if shuffle else np.arange(1, num_pages, dtype=np.int32)
     bt = np.zeros((len(context_lens), max_pages), dtype=np.int32)
     k = 0
     for i, n in enumerate(need):
@@ -121,12 +121,12 @@ def config1_tiny_mixed(seed: int = 0) -> Workload:
                     block_tables=_tables(rng, ctx, 16, 128, 16), q_dtype="f32", kv_dtype="f32", softmax_scale=1.0 / 8.0)
 
 
-def config2_llama_decode(seed: int = 0, n_seqs: int = 256, num_pages: int = 40_000) -> Workload:
+def config2_llama_decode(seed: int = 0, n_seqs: int = 256, num_pages: int = 40_000, shuffle_pages: bool = True) -> Workload:
     rng = np.random.default_rng(seed)
     ctx = rng.integers(512, 8193, size=n_seqs).astype(np.int32)
     return Workload("C2 Llama-3-8B-shaped pure decode", Hq=32, Hkv=8, D=128, page_size=64, num_pages=num_pages,
                     max_pages_per_seq=128, context_lens=ctx, q_lens=np.ones(n_seqs, dtype=np.int32),
-                    block_tables=_tables(rng, ctx, 64, num_pages, 128), softmax_scale=128.0 ** -0.5)
+                    block_tables=_tables(rng, ctx, 64, num_pages, 128, shuffle_pages), softmax_scale=128.0 ** -0.5)
 
 
 def config3_mixed_chunked(seed: int = 0, num_pages: int = 48_000) -> Workload:

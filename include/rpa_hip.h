@@ -140,8 +140,9 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
 
 /*
  * Tuning knobs (process-wide, read at call time).  Returns the previous value.
- *   "decode_chunk"   target tokens per split-K chunk of the decode kernel (multiple of 64)
- *   "max_splits"     upper bound on split-K partials per sequence (1..64)
+ *   "max_splits"     partial-output slots per sequence the decode kernel may use (2..256, 0 = sized
+ *                    from the shapes); set it before sizing the workspace
+ *   "decode_wgs"     persistent decode workgroups per KV-head group (0 = as many as are resident at once)
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
  *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
  *                    1 = decode kernel, 2 = prefill / large-row kernel, 4 = merge (default 7)

@@ -145,15 +145,16 @@ def test_generic_kernel_agrees_with_mfma_kernel(gpu):
     assert np.abs(fast - slow)[tl.valid_rows(b)].max() <= tl.TOL_BF16_MAX
 
 
-@pytest.mark.parametrize("chunk,splits", [(64, 64), (128, 2), (512, 1), (256, 5)])
-def test_split_k_settings_do_not_change_results(gpu, chunk, splits):
+@pytest.mark.parametrize("wgs,splits", [(1, 2), (3, 2), (7, 5), (64, 16), (1000, 64), (0, 0)])
+def test_split_k_settings_do_not_change_results(gpu, wgs, splits):
+    # the number of persistent workgroups and of partial slots decides where sequences are cut
     from easydel_amd import _lib
 
     ctx = [1, 63, 64, 65, 1000, 1999, 128]
     b = tl.make_batch(14, ctx, [1] * len(ctx), Hq=32, Hkv=8, D=128, page_size=64, max_pages=32)
-    p1, p2 = _lib.set_tunable("decode_chunk", chunk), _lib.set_tunable("max_splits", splits)
+    p1, p2 = _lib.set_tunable("decode_wgs", wgs), _lib.set_tunable("max_splits", splits)
     try:
-        _check(b, f"chunk {chunk} splits {splits}")
+        _check(b, f"wgs {wgs} splits {splits}")
     finally:
-        _lib.set_tunable("decode_chunk", p1)
+        _lib.set_tunable("decode_wgs", p1)
         _lib.set_tunable("max_splits", p2)
