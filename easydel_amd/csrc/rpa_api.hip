@@ -12,6 +12,7 @@ int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_
                           int64_t, int);
 int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int);
+int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
 }  // namespace rpa
 
 namespace {
@@ -22,7 +23,7 @@ std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are 
 std::atomic<int> g_force_generic{0};
 std::atomic<int> g_decode_wpb{0};
 std::atomic<int> g_decode_occ{0};
-std::atomic<int> g_stages{7};  // bit 0: decode kernel, bit 1: prefill / large-row kernel, bit 2: merge
+std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -78,8 +79,15 @@ int rpa_set_tunable(const char* name, int value) {
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
   if (!strcmp(name, "decode_wpb")) return g_decode_wpb.exchange(value);
   if (!strcmp(name, "decode_occ")) return g_decode_occ.exchange(value);
-  if (!strcmp(name, "stages")) return g_stages.exchange(value & 7);
+  if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
   return -1;
+}
+
+int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t bytes) {
+  if (!dst || !src || (bytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15))
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_calibration_copy: pointers and size must be 16-byte aligned");
+  if (bytes == 0) return RPA_OK;
+  return hip_fail(rpa::launch_calibration_copy((hipStream_t)stream, dst, src, bytes), "rpa_calibration_copy launch");
 }
 
 int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32_t* slice_indices,
@@ -176,16 +184,16 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
     p.part_o = (float*)(base + pb);
     p.part_ml = (float*)(base + pb + (size_t)splits * po);
     int err = 0;
-    if (stages & 1) err = rpa::launch_attn_decode(s, p);
+    if (stages & 3) err = rpa::launch_attn_decode(s, p, stages & 3);
     if (err) return hip_fail(err, "decode kernel launch");
     // Rows too large for the decode kernel: MFMA prefill kernel where it applies, fp32 kernel otherwise.
-    if (stages & 2) err = rpa::prefill_supported(p) ? rpa::launch_attn_prefill(s, p) : rpa::launch_attn_generic(s, p);
+    if (stages & 4) err = rpa::prefill_supported(p) ? rpa::launch_attn_prefill(s, p) : rpa::launch_attn_generic(s, p);
     if (err) return hip_fail(err, "prefill kernel launch");
   } else {
-    int err = (stages & 2) ? rpa::launch_attn_generic(s, p) : 0;
+    int err = (stages & 4) ? rpa::launch_attn_generic(s, p) : 0;
     if (err) return hip_fail(err, "fp32 kernel launch");
   }
-  if (!(stages & 4)) return RPA_OK;
+  if (!(stages & 8)) return RPA_OK;
   return hip_fail(rpa::launch_attn_merge(s, p), "merge kernel launch");
 }
 

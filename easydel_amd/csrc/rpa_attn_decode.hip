@@ -435,8 +435,9 @@ static int launch_one(hipStream_t stream, AttnParams p) {
   if (p.decode_wgs > 0) n_wg = p.decode_wgs;
   n_wg = max(1, min(n_wg, kMaxDecodeWgs));
   p.n_wg = n_wg;
-  hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(1024), 0, stream, p);
-  hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, OCC>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+  if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(1024), 0, stream, p);
+  if (p.decode_which & 2)
+    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, OCC>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();
 }
 
@@ -485,7 +486,9 @@ bool decode_supported(const AttnParams& p) {
   return true;
 }
 
-int launch_attn_decode(hipStream_t stream, const AttnParams& p) {
+int launch_attn_decode(hipStream_t stream, const AttnParams& p_in, int which) {
+  AttnParams p = p_in;
+  p.decode_which = which;
   switch (p.kv_dtype) {
     case RPA_BF16: return launch_kvt<RPA_BF16>(stream, p);
     case RPA_FP8_E4M3: return launch_kvt<RPA_FP8_E4M3>(stream, p);

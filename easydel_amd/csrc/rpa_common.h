@@ -38,6 +38,7 @@ struct AttnParams {
   int max_splits;    // >= 2: most partial slots one sequence may use
   int n_wg;          // persistent decode workgroups per KV-head group
   int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
+  int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel
   int decode_wpb;    // waves (KV heads) per decode workgroup, 0 = default
   int decode_occ;    // waves per SIMD the decode kernel is compiled for, 0 = compiler's choice
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
@@ -120,7 +121,7 @@ __device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
 
 // Launchers (one per translation unit); all return a hipError_t as int.
 int launch_attn_generic(hipStream_t stream, const AttnParams& p);
-int launch_attn_decode(hipStream_t stream, const AttnParams& p);
+int launch_attn_decode(hipStream_t stream, const AttnParams& p, int which = 3);  // bit 0: plan kernel, bit 1: decode kernel
 int launch_attn_prefill(hipStream_t stream, const AttnParams& p);
 int launch_attn_merge(hipStream_t stream, const AttnParams& p);
 bool decode_supported(const AttnParams& p);

@@ -109,6 +109,17 @@ __global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restr
   }
 }
 
+// Plain grid-stride copy of 16-byte vectors: the known-size kernel that calibrates HBM traffic counters.
+__global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < n16; k += stride) dst[k] = src[k];
+}
+
+int launch_calibration_copy(hipStream_t stream, void* dst, const void* src, size_t bytes) {
+  hipLaunchKernelGGL(calibration_copy_kernel, dim3(4096), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst, bytes >> 4);
+  return (int)hipGetLastError();
+}
+
 int launch_scatter_slices(hipStream_t stream, const void* new_kv, const int32_t* si, const int32_t* num_slices,
                           void* pages, int T, int N, int64_t num_positions, int page_size, int64_t row_bytes,
                           int shard) {

@@ -139,13 +139,21 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   float softmax_scale, int sliding_window, float logits_soft_cap);
 
 /*
+ * Measurement aid with no counterpart in the reference: copies `bytes` (a multiple of 16, both
+ * pointers 16-byte aligned) with a plain vector copy kernel.  Profiling a known-size copy next to
+ * the attention kernels gives the factor that turns raw HBM traffic counters into bytes.
+ */
+int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t bytes);
+
+/*
  * Tuning knobs (process-wide, read at call time).  Returns the previous value.
  *   "max_splits"     partial-output slots per sequence the decode kernel may use (2..256, 0 = sized
  *                    from the shapes); set it before sizing the workspace
  *   "decode_wgs"     persistent decode workgroups per KV-head group (0 = as many as are resident at once)
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
  *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
- *                    1 = decode kernel, 2 = prefill / large-row kernel, 4 = merge (default 7)
+ *                    1 = decode plan kernel, 2 = decode kernel, 4 = prefill / large-row kernel,
+ *                    8 = merge (default 15)
  */
 int rpa_set_tunable(const char* name, int value);
 
