@@ -155,6 +155,7 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
   }
 
   float m_run = -INFINITY, l_run = 0.f;
+  float v_unit = 1.f;  // V scale the accumulators are currently expressed in (8-bit pages)
   f32x4 o_acc[DPL];
 #pragma unroll
   for (int rt = 0; rt < DPL; ++rt) o_acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -252,13 +253,21 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
         pr[j] = __builtin_amdgcn_exp2f(s_acc[st][j] - m_use);
         psum += pr[j];
       }
-      pfrag[st][0] = pack_bf16(pr[0] * v_scale, pr[1] * v_scale);
-      pfrag[st][1] = pack_bf16(pr[2] * v_scale, pr[3] * v_scale);
+      pfrag[st][0] = pack_bf16(pr[0], pr[1]);
+      pfrag[st][1] = pack_bf16(pr[2], pr[3]);
     }
     l_run = l_run * alpha + psum;
-    if (__any(alpha != 1.f)) {
+    // The accumulators hold sum(p * v_code) in units of the current page's V scale, so P stays an exact
+    // softmax weight in bf16; when the scale changes (a new page) they are converted once.
+    float o_mul = alpha;
+    if constexpr (EB == 1) {
+      o_mul = alpha * (v_unit * __builtin_amdgcn_rcpf(v_scale));
+      if (v_unit == v_scale) o_mul = alpha;
+      v_unit = v_scale;
+    }
+    if (__any(o_mul != 1.f)) {
 #pragma unroll
-      for (int rt = 0; rt < DPL; ++rt) o_acc[rt] *= alpha;
+      for (int rt = 0; rt < DPL; ++rt) o_acc[rt] *= o_mul;
     }
 
     // ---- O^T += V^T . P^T ---------------------------------------------------------------------
@@ -333,7 +342,7 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
     const int head_out = h * G + r_head;
     const int d_base = 4 * DPL * g4;
     if (cur.single) {
-      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+      const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
       uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D + d_base;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -348,7 +357,7 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
 #pragma unroll
-        for (int rt = 0; rt < DPL; ++rt) prow[j * DPL + rt] = o_acc[rt][j];
+        for (int rt = 0; rt < DPL; ++rt) prow[j * DPL + rt] = o_acc[rt][j] * v_unit;
       }
       if (g4 == 0) {
         p.part_ml[slot * 2 + 0] = m_run;

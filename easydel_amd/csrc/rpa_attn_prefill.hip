@@ -1,8 +1,384 @@
-// MFMA prefill / chunked-prefill attention (placeholder until the tiled kernel lands): reports
-// "not supported", so sequences with more than 16 rows per KV head run on the fp32 kernel.
-#include "rpa_common.h"
+// MFMA prefill / chunked-prefill attention over the paged cache.
+//
+// Serves sequences with more than 16 query rows per KV head (row = (query token, head of the GQA
+// group), token-major).  A workgroup owns ROWS = NW*RB*16 consecutive rows of one (sequence, KV
+// head): each of its NW waves keeps RB 16-row blocks (Q as MFMA B operands, O^T accumulators,
+// running max / sum) in registers.  K/V tiles of TT keys are loaded once per workgroup with
+// 128-bit loads, one tile ahead, into a double-buffered swizzled LDS tile (8-bit pages are
+// widened to bf16 on the way in, so the compute path sees bf16 only); every wave then reads the
+// tile in MFMA operand order and reuses each K / V operand for its RB row blocks:
+//     S^T[key][row]  = K[key][:] . Q[row][:]            v_mfma_f32_16x16x32_bf16, k = head dim
+//     O^T[dim][row] += V^T[dim][key] . P^T[key][row]    v_mfma_f32_16x16x32_bf16, k = 32 keys
+// Causal and window limits are per row; key tiles wholly outside a workgroup's limits are never
+// loaded, tiles wholly inside skip the masking code.  Block index -> (row tile, KV head) keeps the
+// KV head fastest, so the row tiles of one (sequence, head) share an XCD and its L2.
+#include "rpa_mfma.h"
 
 namespace rpa {
-bool prefill_supported(const AttnParams&) { return false; }
-int launch_attn_prefill(hipStream_t, const AttnParams&) { return (int)hipErrorNotSupported; }
+
+template <int D, int KVT, int TT, int NW, int RB>
+__global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) {
+  constexpr int EB = ElemBytes<KVT>::v;
+  constexpr int RKL = D * 2;             // bytes of one K (or V) row in LDS (always bf16)
+  constexpr int HBG = 2 * D * EB;        // K_h | V_h span of one token in global memory
+  constexpr int LPTG = HBG / 16;         // 16-byte global chunks per token span
+  constexpr int THREADS = 64 * NW;
+  constexpr int NLD = (TT * LPTG + THREADS - 1) / THREADS;  // global loads per thread per tile
+  constexpr int NS = TT / 16;            // 16-key sub-tiles per tile
+  constexpr int DPL = D / 16;            // output dims per lane per accumulator column
+  constexpr int VB = DPL * 2;            // bytes of V one lane reads per key
+  constexpr int NKK = D / 32;            // k-steps of the score MFMA
+  constexpr int ROWS = NW * RB * 16;
+  constexpr int TILE_BYTES = TT * 2 * RKL;
+  static_assert(NS == 1 || NS == 2, "tile is one or two 16-key sub-tiles");
+
+  __shared__ __attribute__((aligned(16))) unsigned char lds_all[2 * TILE_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g4 = lane >> 4;
+  const int G = p.group;
+
+  // ---- block -> (sequence, row tile, KV head) ---------------------------------------------------
+  const int h = blockIdx.x % p.Hkv;
+  const int slot = blockIdx.x / p.Hkv;
+  const int n_live = p.num_seqs[0];
+  if (n_live <= 0) return;
+  // sequence i starts at slot floor(qsl[i]*G/ROWS) + i; find the last sequence starting at or before `slot`
+  int lo_i = 0, hi_i = n_live;
+  while (hi_i - lo_i > 1) {
+    const int mid = (lo_i + hi_i) >> 1;
+    if ((int)(((int64_t)p.qsl[mid] * G) / ROWS) + mid <= slot) lo_i = mid; else hi_i = mid;
+  }
+  const int i = lo_i;
+  const SeqPlan sp = seq_plan(p, i);
+  if (!sp.live || sp.small_rows) return;
+  const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * G) / ROWS) + i);
+  const int rows_total = sp.q_len * G;
+  const int R0 = tile_in_seq * ROWS;
+  if (tile_in_seq < 0 || R0 >= rows_total) return;
+
+  // ---- key range of the workgroup ----------------------------------------------------------------
+  const int last_row = min(R0 + ROWS, rows_total) - 1;
+  const int base_pos = sp.ctx - sp.q_len;  // position of the sequence's first query token
+  const int kv_hi = min(sp.ctx, base_pos + last_row / G + 1);
+  int kv_lo = 0;
+  if (p.window > 0) kv_lo = max(base_pos + R0 / G - p.window + 1, 0);
+  const int vis_lo = kv_lo;
+  kv_lo &= ~(TT - 1);
+  const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
+  if (n_tiles <= 0) return;  // only when the queries sit before position 0; such rows stay unwritten
+
+  // ---- per row-block lane state --------------------------------------------------------------------
+  int row_lo[RB], row_hi[RB];
+  bool row_ok[RB];
+  int out_tok[RB], out_head[RB];
+  bf16x8 qf[RB][NKK];
+  int wave_lo, wave_hi;          // keys every row of the wave sees: [max row_lo, min row_hi)
+  int wave_lo_min, wave_hi_max;  // keys some row of the wave sees: [min row_lo, max row_hi)
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = R0 + (wave * RB + rb) * 16 + n;
+    row_ok[rb] = row < rows_total;
+    const int r_tok = row_ok[rb] ? row / G : (rows_total - 1) / G;  // padded rows shadow the last row
+    const int r_head = row_ok[rb] ? row - r_tok * G : 0;
+    const int pos = base_pos + r_tok;
+    row_hi[rb] = min(pos + 1, sp.ctx);
+    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+    out_tok[rb] = sp.q0 + r_tok;
+    out_head[rb] = h * G + r_head;
+    const char* qrow = (const char*)p.q + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D * 2;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok[rb]) v = *(const u32x4*)(qrow + (kk * 32 + 8 * g4) * 2);
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  {
+    int lo_max = 0, hi_min = 0x7fffffff, lo_min = 0x7fffffff, hi_max = 0;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      lo_max = max(lo_max, row_lo[rb]);
+      hi_min = min(hi_min, row_hi[rb]);
+      lo_min = min(lo_min, row_lo[rb]);
+      hi_max = max(hi_max, row_hi[rb]);
+    }
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+      lo_max = max(lo_max, __shfl_xor(lo_max, o));
+      hi_min = min(hi_min, __shfl_xor(hi_min, o));
+      lo_min = min(lo_min, __shfl_xor(lo_min, o));
+      hi_max = max(hi_max, __shfl_xor(hi_max, o));
+    }
+    wave_lo = __builtin_amdgcn_readfirstlane(lo_max);
+    wave_hi = __builtin_amdgcn_readfirstlane(hi_min);
+    wave_lo_min = __builtin_amdgcn_readfirstlane(lo_min);
+    wave_hi_max = __builtin_amdgcn_readfirstlane(hi_max);
+  }
+  // a wave whose row blocks all lie past the sequence's rows only helps with the loads
+  const bool wave_active = (R0 + wave * RB * 16) < rows_total;
+
+  // ---- staging ---------------------------------------------------------------------------------------
+  const int32_t* bt = p.block_tables + (int64_t)i * p.M;
+  const char* pages = (const char*)p.kv_pages;
+  const int pg = p.page_size;
+  int st_tok[NLD], st_cc[NLD];
+  bool st_v[NLD], st_ok[NLD];
+  int64_t st_off[NLD];
+#pragma unroll
+  for (int u = 0; u < NLD; ++u) {
+    const int idx = u * THREADS + tid;
+    st_ok[u] = idx < TT * LPTG;
+    st_tok[u] = st_ok[u] ? idx / LPTG : 0;
+    const int c = idx % LPTG;
+    st_v[u] = c >= LPTG / 2;
+    st_cc[u] = st_v[u] ? c - LPTG / 2 : c;
+    st_off[u] = (int64_t)st_tok[u] * p.token_stride + (int64_t)h * HBG + c * 16;
+  }
+  u32x4 stage[NLD];
+  auto page_of = [&](int tok) -> int {
+    int pgid = bt[tok / pg];
+    pgid = __builtin_amdgcn_readfirstlane(pgid);
+    return min(max(pgid, 0), p.P - 1);
+  };
+  auto issue = [&](int tb, int page) {
+    const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride;
+#pragma unroll
+    for (int u = 0; u < NLD; ++u)
+      if (st_ok[u]) stage[u] = *(const u32x4*)(base + st_off[u]);
+  };
+  auto commit = [&](int tb, unsigned char* buf) {  // registers -> LDS tile (zeroing keys nobody may see)
+    const bool edge = (tb + TT > sp.ctx) || (tb < vis_lo);
+#pragma unroll
+    for (int u = 0; u < NLD; ++u) {
+      if (!st_ok[u]) continue;
+      u32x4 v = stage[u];
+      if (edge) {
+        const int tok = tb + st_tok[u];
+        if (tok >= sp.ctx || tok < vis_lo) v = (u32x4){0u, 0u, 0u, 0u};
+      }
+      unsigned char* row = buf + (st_v[u] ? TT * RKL : 0) + st_tok[u] * RKL;
+      const int key = swz_key<RKL>(st_tok[u]);
+      if constexpr (EB == 2) {
+        *(u32x4*)(row + ((st_cc[u] ^ key) << 4)) = v;
+      } else {  // 16 codes -> 16 bf16 = two LDS chunks
+        const bf16x8 a = codes8_to_bf16x8<KVT>(v[0], v[1]);
+        const bf16x8 b = codes8_to_bf16x8<KVT>(v[2], v[3]);
+        *(u32x4*)(row + (((2 * st_cc[u]) ^ key) << 4)) = __builtin_bit_cast(u32x4, a);
+        *(u32x4*)(row + (((2 * st_cc[u] + 1) ^ key) << 4)) = __builtin_bit_cast(u32x4, b);
+      }
+    }
+  };
+
+  const bool has_cap = p.softcap > 0.f;
+  const float cap_out = p.softcap * 1.4426950408889634f;
+  const float cap_in = has_cap ? p.scale / p.softcap : 0.f;
+
+  float m_run[RB], l_run[RB];
+  float v_unit = 1.f;  // V scale the accumulators are currently expressed in (8-bit pages)
+  f32x4 o_acc[RB][DPL];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    m_run[rb] = -INFINITY;
+    l_run[rb] = 0.f;
+#pragma unroll
+    for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  int page_cur = page_of(kv_lo);
+  issue(kv_lo, page_cur);
+  commit(kv_lo, lds_all);
+  __syncthreads();
+
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    const int tb = kv_lo + tile * TT;
+    unsigned char* lds_k = lds_all + (tile & 1) * TILE_BYTES;
+    unsigned char* lds_v = lds_k + TT * RKL;
+    float k_scale = 1.f, v_scale = 1.f;
+    if constexpr (EB == 1) {
+      const float* sc = p.kv_scales + (int64_t)page_cur * p.C + 2 * h;
+      k_scale = sc[0];
+      v_scale = sc[1];
+    }
+    const bool more = tile + 1 < n_tiles;
+    if (more) {
+      page_cur = page_of(tb + TT);
+      issue(tb + TT, page_cur);
+    }
+
+    if (wave_active && tb < wave_hi_max && tb + TT > wave_lo_min) {
+      // ---- S^T = K . Q^T for every row block (K operands shared) --------------------------------
+      f32x4 s_acc[RB][NS];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int st = 0; st < NS; ++st) s_acc[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < NS; ++st) {
+        const int tk = st * 16 + n;
+        const unsigned char* krow = lds_k + tk * RKL;
+        const int key = swz_key<RKL>(tk);
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+          const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
+        }
+      }
+
+      // ---- online softmax per row block -------------------------------------------------------------
+      const bool inside = (tb >= wave_lo) && (tb + TT <= wave_hi);  // no row of the wave masks any key here
+      uint32_t pfrag[RB][NS][2];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        if (has_cap) {
+#pragma unroll
+          for (int st = 0; st < NS; ++st)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s_acc[rb][st][j] = fast_tanh(s_acc[rb][st][j] * (cap_in * k_scale));
+        }
+        const float sc_mul = has_cap ? cap_out : p.scale_log2 * k_scale;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int st = 0; st < NS; ++st) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float s = s_acc[rb][st][j] * sc_mul;
+            if (!inside) {
+              const int tok = tb + st * 16 + 4 * g4 + j;
+              s = (tok >= row_lo[rb] && tok < row_hi[rb]) ? s : -INFINITY;
+            }
+            s_acc[rb][st][j] = s;
+            mx = fmaxf(mx, s);
+          }
+        }
+        mx = xor32_max(xor16_max(mx));
+        const float m_new = fmaxf(m_run[rb], mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_use);
+        m_run[rb] = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int st = 0; st < NS; ++st) {
+          float pr[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            pr[j] = __builtin_amdgcn_exp2f(s_acc[rb][st][j] - m_use);
+            psum += pr[j];
+          }
+          pfrag[rb][st][0] = pack_bf16(pr[0], pr[1]);
+          pfrag[rb][st][1] = pack_bf16(pr[2], pr[3]);
+        }
+        l_run[rb] = l_run[rb] * alpha + psum;
+        // accumulators are kept in units of the current page's V scale (see the decode kernel)
+        float o_mul = alpha;
+        if constexpr (EB == 1) {
+          if (v_unit != v_scale) o_mul = alpha * (v_unit * __builtin_amdgcn_rcpf(v_scale));
+        }
+        if (__any(o_mul != 1.f)) {
+#pragma unroll
+          for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] *= o_mul;
+        }
+      }
+      v_unit = v_scale;
+
+      // ---- O^T += V^T . P^T (V operands shared by the row blocks) -----------------------------------
+      uint32_t raw[4 * NS][DPL / 2];  // raw[e][w]: key (e < 4 ? 4g4+e : 16+4g4+e-4), dword w of this lane's DPL dims
+#pragma unroll
+      for (int e = 0; e < 4 * NS; ++e) {
+        const int tk = (e >> 2) * 16 + 4 * g4 + (e & 3);
+        const unsigned char* vrow = lds_v + tk * RKL;
+        const int key = swz_key<RKL>(tk);
+        if constexpr (VB >= 16) {
+#pragma unroll
+          for (int r = 0; r < VB / 16; ++r) {
+            const u32x4 v = *(const u32x4*)(vrow + ((((n * VB) / 16 + r) ^ key) << 4));
+            raw[e][4 * r + 0] = v[0]; raw[e][4 * r + 1] = v[1]; raw[e][4 * r + 2] = v[2]; raw[e][4 * r + 3] = v[3];
+          }
+        } else {  // VB == 8
+          const u32x2 v = *(const u32x2*)(vrow + ((((n * VB) >> 4) ^ key) << 4) + ((n * VB) & 15));
+          raw[e][0] = v[0]; raw[e][1] = v[1];
+        }
+      }
+#pragma unroll
+      for (int rt = 0; rt < DPL; ++rt) {
+        const uint32_t sel = (rt & 1) ? 0x07060302u : 0x05040100u;
+        const int w = rt >> 1;
+        if constexpr (NS == 2) {
+          const u32x4 a4 = {__builtin_amdgcn_perm(raw[1][w], raw[0][w], sel), __builtin_amdgcn_perm(raw[3][w], raw[2][w], sel),
+                            __builtin_amdgcn_perm(raw[5][w], raw[4][w], sel), __builtin_amdgcn_perm(raw[7][w], raw[6][w], sel)};
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
+            o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
+                                                                    o_acc[rb][rt], 0, 0, 0);
+          }
+        } else {
+          const u32x2 a2 = {__builtin_amdgcn_perm(raw[1][w], raw[0][w], sel), __builtin_amdgcn_perm(raw[3][w], raw[2][w], sel)};
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            const u32x2 b2 = {pfrag[rb][0][0], pfrag[rb][0][1]};
+            o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), __builtin_bit_cast(s16x4, b2),
+                                                                      o_acc[rb][rt], 0, 0, 0);
+          }
+        }
+      }
+    }
+
+    if (more) commit(tb + TT, lds_all + ((tile + 1) & 1) * TILE_BYTES);
+    __syncthreads();
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------------------
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    if (row_ok[rb]) {
+      const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
+      uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * DPL * g4;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int rt = 0; rt < DPL; rt += 2)
+          *(uint32_t*)(orow + j * DPL + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
+    }
+  }
+}
+
+template <int D, int KVT, int TT, int NW, int RB>
+static int launch_one(hipStream_t stream, const AttnParams& p) {
+  constexpr int ROWS = NW * RB * 16;
+  const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
+  const int64_t blocks = slots * p.Hkv;
+  if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL((attn_prefill_kernel<D, KVT, TT, NW, RB>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+template <int KVT>
+static int launch_kvt(hipStream_t stream, const AttnParams& p) {
+  const bool tt32 = (p.page_size % 32 == 0);
+  switch (p.D) {
+    case 64: return tt32 ? launch_one<64, KVT, 32, 4, 2>(stream, p) : launch_one<64, KVT, 16, 4, 2>(stream, p);
+    case 128: return tt32 ? launch_one<128, KVT, 32, 4, 2>(stream, p) : launch_one<128, KVT, 16, 4, 2>(stream, p);
+    case 256: return tt32 ? launch_one<256, KVT, 32, 8, 1>(stream, p) : launch_one<256, KVT, 16, 8, 1>(stream, p);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
+bool prefill_supported(const AttnParams& p) { return decode_supported(p); }
+
+int launch_attn_prefill(hipStream_t stream, const AttnParams& p) {
+  switch (p.kv_dtype) {
+    case RPA_BF16: return launch_kvt<RPA_BF16>(stream, p);
+    case RPA_FP8_E4M3: return launch_kvt<RPA_FP8_E4M3>(stream, p);
+    case RPA_INT8: return launch_kvt<RPA_INT8>(stream, p);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
 }  // namespace rpa

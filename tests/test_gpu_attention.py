@@ -158,3 +158,56 @@ def test_split_k_settings_do_not_change_results(gpu, wgs, splits):
     finally:
         _lib.set_tunable("decode_wgs", p1)
         _lib.set_tunable("max_splits", p2)
+
+
+@pytest.mark.parametrize("D,page_size,Hq,Hkv,kv_dtype", [
+    (128, 64, 32, 8, BF16), (64, 16, 8, 2, BF16), (256, 128, 16, 8, BF16), (128, 16, 40, 8, BF16),
+    (128, 64, 40, 8, FP8), (128, 32, 8, 8, INT8), (256, 32, 16, 8, FP8), (64, 64, 32, 1, BF16), (64, 16, 4, 2, INT8)])
+def test_prefill_mfma_kernel(gpu, D, page_size, Hq, Hkv, kv_dtype):
+    # full prefill (prior context 0), chunked prefill deep into a context, ragged tile edges, one decode row
+    ctx = [300, 1000, 129, 47, 2100, 700]
+    q_lens = [300, 200, 129, 33, 17, 1]
+    b = tl.make_batch(40 + D, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype, pad_rows=2, pad_tokens=5)
+    _check(b, f"prefill D{D} pg{page_size} {Hq}/{Hkv} kv{kv_dtype}")
+
+
+@pytest.mark.parametrize("window", [1, 16, 100, 513])
+def test_prefill_sliding_window(gpu, window):
+    ctx = [600, 1500, window + 40, 64]
+    q_lens = [600, 300, 40, 64]
+    b = tl.make_batch(50, ctx, q_lens, Hq=16, Hkv=4, D=128, page_size=64, max_pages=24)
+    _check(b, f"prefill window {window}", sliding_window=window)
+
+
+def test_prefill_soft_cap_gemma_shape(gpu):
+    ctx = [900, 2500]
+    q_lens = [256, 200]
+    b = tl.make_batch(51, ctx, q_lens, Hq=16, Hkv=8, D=256, page_size=128, max_pages=20)
+    _check(b, "prefill softcap", logits_soft_cap=50.0, softmax_scale=1.0 / 16.0)
+    _check(b, "prefill softcap + window", logits_soft_cap=50.0, softmax_scale=1.0 / 16.0, sliding_window=300)
+
+
+def test_prefill_window_with_null_pages(gpu):
+    W, pg = 200, 64
+    ctx = [1500, 900]
+    q_lens = [100, 64]
+    b = tl.make_batch(52, ctx, q_lens, Hq=16, Hkv=4, D=128, page_size=pg, max_pages=24)
+    want = tl.oracle_out(b, sliding_window=W)
+    for i, (c, ql) in enumerate(zip(ctx, q_lens)):
+        first_needed = max(c - ql - W + 1, 0) // pg
+        b.block_tables[i, :first_needed] = 0
+    b.kv_raw[0] = 0x7FC0
+    got = tl.run_gpu_attention(b, sliding_window=W)
+    tl.assert_close(got, want, b, "prefill window + null pages")
+
+
+def test_chunked_prefill_equals_rows_of_single_shot_prefill(gpu):
+    # the same keys, queried as one 384-token prefill and as its last 128-token chunk
+    b_full = tl.make_batch(53, [384], [384], Hq=32, Hkv=8, D=128, page_size=64)
+    full = tl.run_gpu_attention(b_full)
+    b_chunk = tl.make_batch(53, [384], [128], Hq=32, Hkv=8, D=128, page_size=64)
+    b_chunk.kv_raw, b_chunk.kv_val, b_chunk.block_tables = b_full.kv_raw, b_full.kv_val, b_full.block_tables
+    b_chunk.q_raw, b_chunk.q_val = b_full.q_raw[256:], b_full.q_val[256:]
+    chunk = tl.run_gpu_attention(b_chunk)
+    assert np.abs(chunk - full[256:]).max() <= 2e-2
+    tl.assert_close(chunk, tl.oracle_out(b_chunk), b_chunk, "chunk")
