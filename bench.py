@@ -27,6 +27,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 
 
 def parse_args():
@@ -34,7 +35,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c4-fp8", "c4-int8"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
@@ -53,9 +54,13 @@ def build_workload(name, seed, sequential=False):
 
     if name == "c2":
         return workloads.config2_llama_decode(seed, shuffle_pages=not sequential)
+    if name == "c3":
+        return workloads.config3_mixed_chunked(seed)
     if name == "c4-fp8":
         return workloads.config4_quantised_decode(seed, "fp8")
-    return workloads.config4_quantised_decode(seed, "int8")
+    if name == "c4-int8":
+        return workloads.config4_quantised_decode(seed, "int8")
+    return workloads.config5_gemma_long_prefill(seed, windowed=(name == "c5-window"))
 
 
 def measured_traffic(workload):
@@ -180,28 +185,50 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # dominant kernel in isolation: one call that only runs the plan kernel, then calls that only launch
-    # the decode kernel (it reuses the plan left in the workspace), bracketed by events on the launch stream
+    # kernels in isolation: one call that only runs the plan kernel, then calls that launch only the decode
+    # kernel (it reuses the plan left in the workspace) or only the prefill kernel, bracketed by events on the
+    # launch stream
     stream = torch.cuda.current_stream(dev)
     att = lambda: kernels.ragged_paged_attention(  # noqa: E731
         tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
         tens["num_seqs"], softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
         logits_soft_cap=w.logits_soft_cap, kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv, out=out)
+
+    def time_stage(mask, reps):
+        _lib.set_tunable("stages", mask)
+        for _ in range(3):
+            att()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for a, b in evs:
+            a.record(stream)
+            att()
+            b.record(stream)
+        torch.cuda.synchronize()
+        return float(np.mean([a.elapsed_time(b) for a, b in evs]))
+
     prev = _lib.set_tunable("stages", 1)
     att()
-    _lib.set_tunable("stages", 2)
-    for _ in range(3):
-        att()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for a, b in evs:
-        a.record(stream)
-        att()
-        b.record(stream)
-    torch.cuda.synchronize()
+    small = w.small_row_mask()
+    kern = {}
+    if small.any():
+        ms = time_stage(2, args.steps)
+        nbytes = w.attention_bytes(small)
+        kern["attn_decode_kernel"] = {
+            "bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload),
+            "algorithmic_bytes_per_launch": nbytes, "kernel_ms": ms}
+    if (~small & (w.q_lens > 0)).any():
+        ms = time_stage(4, args.steps)
+        flops = w.attention_flops(~small)
+        kern["attn_prefill_kernel"] = {
+            "bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": w.attention_bytes(~small),
+            "kernel_ms": ms}
     _lib.set_tunable("stages", prev)
-    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    dominant = max(kern, key=lambda k: kern[k]["kernel_ms"])
+    roofline = dict(kern[dominant], kernel=dominant)
     att_bytes = w.attention_bytes()
-    achieved = att_bytes / (kernel_ms * 1e-3) / 1e9
 
     result = {
         "metric": "decode tokens/s + attn HBM TB/s (% of 8 TB/s), Llama-3-8B-shaped, 1 GPU",
@@ -227,24 +254,18 @@ def main():
             "pool_pages": w.num_pages,
             "context_tokens_total": int(w.context_lens.sum()),
             "context_range": [int(w.context_lens.min()), int(w.context_lens.max())],
+            "sliding_window": w.sliding_window,
+            "logits_soft_cap": w.logits_soft_cap,
             "seed": args.seed,
         },
         "attention_only_model_tokens_per_s_32_layers": w.T / (ms_per_step * 1e-3) / 32.0,
-        "attn_hbm_tb_s": achieved / 1e3,
-        "attn_hbm_pct_of_8tb_s": 100.0 * achieved / HBM_PEAK_GBS,
         "step_hbm_tb_s": (att_bytes + w.scatter_bytes()) / (ms_per_step * 1e-3) / 1e12,
-        "roofline": {
-            "kernel": "attn_decode_kernel",
-            "bound": "hbm",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBS,
-            "traffic": measured_traffic(args.workload),
-            "algorithmic_bytes_per_launch": att_bytes,
-            "kernel_ms": kernel_ms,
-        },
+        "roofline": roofline,
+        "kernels": kern,
     }
+    if "attn_decode_kernel" in kern:
+        result["attn_hbm_tb_s"] = kern["attn_decode_kernel"]["achieved"] / 1e3
+        result["attn_hbm_pct_of_8tb_s"] = 100.0 * kern["attn_decode_kernel"]["frac"]
 
     if not args.no_cpu_baseline:
         # the whole batch fits the host here; it is re-run for about 10 s

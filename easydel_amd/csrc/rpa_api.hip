@@ -58,7 +58,15 @@ int static_splits(int T, int M, int page_size, int Hq, int D) {
   return (int)want;
 }
 
-size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + S + 1 + rpa::kMaxDecodeWgs) * 4); }
+size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + 2 * ((size_t)S + 1) + rpa::kMaxDecodeWgs) * 4); }
+
+// Static bound on query tokens the decode kernel can own: sequences with at most 16 rows per KV head.
+int decode_token_bound(int T, int S, int Hq, int Hkv) {
+  const int group = Hq / Hkv;
+  if (group > 16) return 1;
+  const long bound = (long)S * (16 / group);
+  return (int)(bound < T ? bound : T);
+}
 
 }  // namespace
 
@@ -122,10 +130,12 @@ int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* va
 
 size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int q_dtype,
                                      int kv_dtype) {
-  (void)Hkv; (void)q_dtype; (void)kv_dtype;
+  (void)q_dtype; (void)kv_dtype;
   if (T <= 0 || S <= 0 || M <= 0 || page_size <= 0 || Hq <= 0 || D <= 0) return 256;
-  const int splits = static_splits(T, M, page_size, Hq, D);
-  return (size_t)splits * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) + plan_bytes(S) + 256;
+  if (Hkv <= 0 || Hq % Hkv != 0) return 256;
+  const int td = decode_token_bound(T, S, Hq, Hkv);
+  const int splits = static_splits(td, M, page_size, Hq, D);
+  return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + plan_bytes(S) + 256;
 }
 
 int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages, const float* kv_scales,
@@ -171,8 +181,10 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   hipStream_t s = (hipStream_t)stream;
   const int stages = g_stages.load();
   if (p.mfma_path) {
-    const size_t po = part_o_bytes(T, Hq, D), pml = part_ml_bytes(T, Hq), pb = plan_bytes(S);
-    int splits = static_splits(T, M, page_size, Hq, D);
+    const int td = decode_token_bound(T, S, Hq, Hkv);
+    p.t_dec_max = td;
+    const size_t po = part_o_bytes(td, Hq, D), pml = part_ml_bytes(td, Hq), pb = plan_bytes(S);
+    int splits = static_splits(td, M, page_size, Hq, D);
     const size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
     if (!workspace || usable < 2 * (po + pml))
       return fail(RPA_ERR_WORKSPACE, "rpa_ragged_paged_attention: workspace %zu bytes < %zu needed for two partial slots",

@@ -24,6 +24,7 @@ namespace rpa {
 // Per-workgroup piece of the flattened key stream: a token range of one sequence.
 struct Piece {
   int i, q0, q_len, ctx;
+  int part_row;        // row of the sequence's first query token in the partial buffers
   int t_begin, t_end;  // keys [t_begin, t_end) of sequence i
   int slot;            // which partial slot of the sequence this piece fills
   int single;          // the sequence lies in one piece: write the final output directly
@@ -43,6 +44,7 @@ __device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* 
   const SeqPlan sp = seq_plan(p, i);
   Piece pc;
   pc.i = i; pc.q0 = sp.q0; pc.q_len = sp.q_len; pc.ctx = sp.ctx;
+  pc.part_row = P[p.S + 1 + i];
   pc.flat_end = min(span_end, p1);
   pc.t_begin = sp.lo + (pos - p0);
   pc.t_end = min(sp.hi, sp.lo + (pc.flat_end - p0));
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
   const float cap_out = p.softcap * 1.4426950408889634f;
   const float cap_in = has_cap ? p.scale / p.softcap : 0.f;
 
-  Piece cur = make_piece(p, P, plan[kPlanHeader + p.S + 1 + blockIdx.x], span_begin, span_end, Q);
+  Piece cur = make_piece(p, P, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
   int page_cur = page_of(cur.i, cur.t_begin);
   issue(cur.t_begin, page_cur);  // first tile in flight before anything else is set up
 
@@ -352,7 +354,7 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
         }
       }
     } else {
-      const int64_t slot = ((int64_t)cur.slot * p.T + tok_out) * p.Hq + head_out;
+      const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok) * p.Hq + head_out;
       float* prow = p.part_o + slot * D + d_base;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -373,32 +375,42 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
 // One block: exclusive prefix sum of the 64-token-rounded key spans of the decode-class sequences
 // (the flattened key stream), the per-workgroup span length Q, and each workgroup's first sequence.
 __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
-  __shared__ int part[1024];
+  __shared__ int part[1024], part2[1024];
   __shared__ int s_Q;
   int32_t* plan = p.plan;
   int32_t* P = plan + kPlanHeader;
   const int S = p.S, tid = threadIdx.x;
   const int per = (S + 1023) / 1024;
   const int i0 = min(S, tid * per), i1 = min(S, i0 + per);
-  auto span_of = [&](int i) -> int {
+  auto span_of = [&](int i, int& toks) -> int {
     const SeqPlan sp = seq_plan(p, i);
+    toks = 0;
     if (!sp.live || !sp.small_rows) return 0;
+    toks = sp.q_len;
     return (sp.hi - sp.lo + 63) & ~63;
   };
-  int sum = 0;
-  for (int i = i0; i < i1; ++i) sum += span_of(i);
+  int sum = 0, tsum = 0, toks;
+  for (int i = i0; i < i1; ++i) {
+    sum += span_of(i, toks);
+    tsum += toks;
+  }
   part[tid] = sum;
+  part2[tid] = tsum;
   __syncthreads();
-  for (int off = 1; off < 1024; off <<= 1) {  // inclusive Hillis-Steele scan
+  for (int off = 1; off < 1024; off <<= 1) {  // inclusive Hillis-Steele scans
     const int v = (tid >= off) ? part[tid - off] : 0;
+    const int v2 = (tid >= off) ? part2[tid - off] : 0;
     __syncthreads();
     part[tid] += v;
+    part2[tid] += v2;
     __syncthreads();
   }
-  int run = part[tid] - sum;
+  int run = part[tid] - sum, trun = part2[tid] - tsum;
   for (int i = i0; i < i1; ++i) {
     P[i] = run;
-    run += span_of(i);
+    P[S + 1 + i] = min(trun, max(p.t_dec_max - 1, 0));
+    run += span_of(i, toks);
+    trun += toks;
   }
   const int W = part[1023];
   if (tid == 0) {
@@ -418,12 +430,12 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   for (int j = tid; j < p.n_wg; j += 1024) {
     const int64_t target = (int64_t)j * Q;
     int lo = 0, hi = S;  // invariant: P[lo] <= target (P[0] = 0); answer in [lo, hi)
-    if (target >= W) { plan[kPlanHeader + S + 1 + j] = 0; continue; }
+    if (target >= W) { plan[kPlanHeader + 2 * (S + 1) + j] = 0; continue; }
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (P[mid] <= target) lo = mid; else hi = mid;
     }
-    plan[kPlanHeader + S + 1 + j] = lo;
+    plan[kPlanHeader + 2 * (S + 1) + j] = lo;
   }
 }
 

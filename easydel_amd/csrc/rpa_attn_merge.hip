@@ -18,14 +18,17 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   const int n_live = p.num_seqs[0];
   const int D = p.D;
   bool zero = false;
-  int n_pieces = 0;
+  int n_pieces = 0, part_row = 0;
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) {
     zero = true;
   } else {
     const int i = find_seq(p.qsl, n_live, t);
     const SeqPlan sp = seq_plan(p, i);
     if (!sp.live) zero = true;
-    else if (p.mfma_path && sp.small_rows) n_pieces = decode_pieces(p.plan, i);
+    else if (p.mfma_path && sp.small_rows) {
+      n_pieces = decode_pieces(p.plan, i);
+      part_row = p.plan[kPlanHeader + p.S + 1 + i] + (t - sp.q0);
+    }
   }
   const bool merge = n_pieces > 1;
   if (!zero && !merge) return;
@@ -33,8 +36,8 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   float acc[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, lane+128, lane+192
   float inv = 0.f;
   if (merge) {
-    const int64_t stride = (int64_t)p.T * p.Hq;  // slots between consecutive pieces
-    const int64_t slot0 = (int64_t)t * p.Hq + hq;
+    const int64_t stride = (int64_t)p.t_dec_max * p.Hq;  // slots between consecutive pieces
+    const int64_t slot0 = (int64_t)part_row * p.Hq + hq;
     float m = -INFINITY;
     for (int c = lane; c < n_pieces; c += 64) m = fmaxf(m, p.part_ml[(slot0 + c * stride) * 2]);
 #pragma unroll

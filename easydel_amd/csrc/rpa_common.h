@@ -23,10 +23,11 @@ struct AttnParams {
   const int32_t* qsl;
   const int32_t* num_seqs;
   void* out;
-  float* part_o;   // [max_splits][T][Hq][D]
-  float* part_ml;  // [max_splits][T][Hq][2]  (running max in log2 units, running sum)
+  float* part_o;   // [max_splits][Tdec][Hq][D]   Tdec = t_dec_max: decode-class query tokens, compacted
+  float* part_ml;  // [max_splits][Tdec][Hq][2]   (running max in log2 units, running sum)
   int32_t* plan;   // decode plan: [0] = W (flattened keys), [1] = Q (keys per workgroup), then at kPlanHeader:
-                   // P[S+1] exclusive prefix of per-sequence key spans, then first_seq[n_wg]
+                   // P[S+1] exclusive prefix of per-sequence key spans, R[S+1] exclusive prefix of
+                   // decode-class query tokens (row of a token in the partial buffers), first_seq[n_wg]
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
   int64_t token_stride;  // bytes between consecutive tokens of a page = C*D*elem
   int64_t page_stride;   // bytes between pages
@@ -36,6 +37,7 @@ struct AttnParams {
   int window;        // <= 0: none
   float softcap;     // <= 0: none
   int max_splits;    // >= 2: most partial slots one sequence may use
+  int t_dec_max;     // static bound on decode-class query tokens = rows of one partial slot
   int n_wg;          // persistent decode workgroups per KV-head group
   int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
   int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel

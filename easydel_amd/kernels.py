@@ -92,6 +92,7 @@ def page_scatter_slices(new_kv, slice_indices, num_slices, kv_cache_pages, *, pa
     if T == 0 or N == 0 or n_pos == 0:
         return kv_cache_pages
     row_bytes = math.prod(new_kv.shape[1:]) * new_kv.element_size()
+    _dev(kv_cache_pages, "kv_cache_pages")
     _lib.check(lib.rpa_page_scatter_slices(
         _stream(kv_cache_pages), _dev(new_kv, "new_kv"), _i32(slice_indices, "slice_indices"),
         _i32(num_slices, "num_slices"), _dev(kv_cache_pages, "kv_cache_pages"), T, N, n_pos, int(page_size), row_bytes,
@@ -110,6 +111,7 @@ def page_scatter_ragged(key, value, kv_pages, context_lens, block_tables, query_
     M = block_tables.numel() // S
     if T == 0:
         return kv_pages
+    _dev(kv_pages, "kv_pages")
     _lib.check(lib.rpa_page_scatter_ragged(
         _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
         _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
@@ -143,6 +145,8 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
     if T == 0:
         return out
     qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
+    for name, t in (("query", query), ("kv_pages", kv_pages), ("out", out)):
+        _dev(t, name)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
     scales_ptr = None
     if kv_scales is not None:
@@ -171,6 +175,8 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
     if T == 0:
         return out, kv_pages
     qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
+    for name, t in (("query", query), ("key", key), ("value", value), ("kv_pages", kv_pages), ("out", out)):
+        _dev(t, name)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
     _lib.check(lib.rpa_ragged_paged_attention_v3(
         _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),

@@ -1,0 +1,18 @@
+from ._attention_outputs import AttentionOutput
+from ._base_operation import BaseOperation, EasyDeLBackends, OperationImpl, OperationMetadata, OperationRegistry
+from .ragged_page_attention import RaggedPageAttnV2, RaggedPageAttnV3
+from .requirements import (
+    CacheRequirements,
+    CacheType,
+    ExecutionMode,
+    MetadataField,
+    MetadataRequirements,
+    OperationRequirements,
+    RequirementsBuilder,
+)
+
+__all__ = [
+    "AttentionOutput", "BaseOperation", "EasyDeLBackends", "OperationImpl", "OperationMetadata", "OperationRegistry",
+    "RaggedPageAttnV2", "RaggedPageAttnV3", "CacheRequirements", "CacheType", "ExecutionMode", "MetadataField",
+    "MetadataRequirements", "OperationRequirements", "RequirementsBuilder",
+]

@@ -1,0 +1,156 @@
+"""``ragged_page_attention_v2`` / ``_v3`` operations backed by the MI355X HIP kernels.
+
+Drop-in for the reference's ``easydel/operations/kernels/ragged_page_attention.py``: the same class names,
+registry names, call signature (``query, key, value, cache_view, cache_metadata, softmax_scale,
+logits_soft_cap, sliding_window`` plus swallowed extras), 4-D <-> ragged reshape (:881-918), cast of K/V to
+the cache dtype with a warning when it narrows (:570-580), write-back of the updated pages into the view
+(:747) and ``AttentionOutput`` result.  Where the reference hands the arrays to ``ejkernel`` (:281-313,
+:732-746), this module hands device pointers to ``librpa_hip.so`` through ``easydel_amd.kernels``.
+"""
+
+from __future__ import annotations
+
+import logging
+
+import torch
+
+from .. import kernels
+from ..caching.ragged_page import RaggedPagesCacheView, RaggedPagesMetadata
+from ._attention_outputs import AttentionOutput
+from ._base_operation import OperationImpl, OperationRegistry
+from .requirements import CacheType, ExecutionMode, MetadataField, OperationRequirements, RequirementsBuilder
+
+logger = logging.getLogger(__name__)
+
+
+def _request_distribution_bounds(scheduled: torch.Tensor, context_lens: torch.Tensor) -> torch.Tensor:
+    """``[decode_end, prefill_end, total]`` on the device (reference :177-187)."""
+    scheduled = scheduled.to(torch.int32)
+    context_lens = context_lens.to(torch.int32)
+    has_tokens = scheduled > 0
+    is_decode = (scheduled == 1) & (context_lens > 1) & has_tokens
+    decode = is_decode.sum()
+    prefill = (has_tokens & ~is_decode).sum()
+    return torch.stack((decode, decode + prefill, has_tokens.sum())).to(torch.int32)
+
+
+class _RaggedPageAttn(OperationImpl):
+    """Attention over a paged KV cache for ragged batches (prefill, chunked prefill and decode rows mixed)."""
+
+    @classmethod
+    def get_impl_name(cls) -> str | tuple[str]:
+        raise NotImplementedError()
+
+    # -- v2: read-only attention over pages the cache view already updated ------------------------------
+    def forward_v2(self, query, cache_view: RaggedPagesCacheView, cache_metadata: RaggedPagesMetadata,
+                   softmax_scale: float | None = None, logits_soft_cap: float | None = None, compute_dtype=None,
+                   optimized: bool = False, sliding_window: int | None = None, softmax_aux=None,
+                   mask_value: float | None = None, vmem_limit_bytes: int | None = None, **ignore) -> AttentionOutput:
+        if softmax_aux is not None:
+            raise NotImplementedError("attention sinks (softmax_aux) are not implemented by the ROCm ragged-page kernels")
+        output = kernels.ragged_paged_attention(
+            query, cache_view.kv_pages, cache_metadata.context_lens, cache_metadata.pages_tables,
+            cache_metadata.query_start_loc, cache_metadata.num_seqs.reshape(-1), softmax_scale=softmax_scale,
+            sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
+            kv_scales=getattr(cache_view, "kv_scales", None), num_kv_heads=_num_kv_heads(cache_view))
+        return AttentionOutput(attention_weights=None, attention_outputs=output)
+
+    # -- v3: fused page write + attention ------------------------------------------------------------------
+    def forward_v3(self, query, key, value, cache_view: RaggedPagesCacheView, cache_metadata: RaggedPagesMetadata,
+                   softmax_scale: float | None = None, logits_soft_cap: float | None = None,
+                   sliding_window: int | None = None, softmax_aux=None, **ignore) -> AttentionOutput:
+        if softmax_aux is not None:
+            raise NotImplementedError("attention sinks (softmax_aux) are not implemented by the ROCm ragged-page kernels")
+        kv_pages = cache_view.kv_pages
+        if getattr(cache_view, "kv_scales", None) is not None:
+            # quantised pages are read-only for this path: whoever owns the cache wrote codes and scales
+            output = kernels.ragged_paged_attention(
+                query, kv_pages, cache_metadata.context_lens, cache_metadata.pages_tables.reshape(-1),
+                cache_metadata.query_start_loc, cache_metadata.request_distribution[2:3], softmax_scale=softmax_scale,
+                sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, kv_scales=cache_view.kv_scales,
+                num_kv_heads=_num_kv_heads(cache_view))
+            return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
+        if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
+            if kv_pages.element_size() < max(key.element_size(), value.element_size()):
+                logger.warning("Casting key/value from %s to lower-precision KV cache dtype %s; "
+                               "this may reduce numerical fidelity.", key.dtype, kv_pages.dtype)
+            key = key.to(kv_pages.dtype)
+            value = value.to(kv_pages.dtype)
+        output, kv_pages = kernels.ragged_paged_attention_v3(
+            query, key.contiguous(), value.contiguous(), kv_pages, cache_metadata.context_lens,
+            cache_metadata.pages_tables.reshape(-1), cache_metadata.query_start_loc, cache_metadata.request_distribution,
+            softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap)
+        cache_view.kv_pages = kv_pages
+        return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
+
+    def forward_native(self, query, key, value, cache_view, cache_metadata, softmax_scale: float | None = None,
+                       logits_soft_cap: float | None = None, sliding_window: int | None = None, softmax_aux=None,
+                       vmem_limit_bytes: int | None = None, mask_value: float | None = None, compute_dtype=None,
+                       optimized: bool = False, **ignore):
+        fn = self.forward_v3 if self.get_impl_name() == "ragged_page_attention_v3" else self.forward_v2
+        return fn(query=query, key=key, value=value, cache_view=cache_view, cache_metadata=cache_metadata,
+                  softmax_scale=softmax_scale, logits_soft_cap=logits_soft_cap, vmem_limit_bytes=vmem_limit_bytes,
+                  optimized=optimized, compute_dtype=compute_dtype, softmax_aux=softmax_aux, mask_value=mask_value,
+                  sliding_window=sliding_window, **ignore)
+
+    def forward_gpu(self, *args, **kwargs) -> AttentionOutput:
+        return self.forward_native(*args, **kwargs)
+
+    def forward_rocm(self, *args, **kwargs) -> AttentionOutput:
+        return self.forward_native(*args, **kwargs)
+
+    def __call__(self, query, key, value, cache_view, cache_metadata, softmax_scale: float | None = None,
+                 logits_soft_cap: float | None = None, compute_dtype=None, optimized: bool = False,
+                 sliding_window: int | None = None, softmax_aux=None, mask_value: float | None = None,
+                 vmem_limit_bytes: int | None = None, **ignore) -> AttentionOutput:
+        is_4d = query.ndim == 4
+        shape4 = tuple(query.shape) if is_4d else None
+        query_r = query.reshape(-1, *query.shape[-2:]).contiguous()
+        key_r = None if key is None else key.reshape(-1, *key.shape[-2:])
+        value_r = None if value is None else value.reshape(-1, *value.shape[-2:])
+        output = super().__call__(query=query_r, key=key_r, value=value_r, cache_view=cache_view,
+                                  cache_metadata=cache_metadata, softmax_scale=softmax_scale,
+                                  logits_soft_cap=logits_soft_cap, vmem_limit_bytes=vmem_limit_bytes, optimized=optimized,
+                                  compute_dtype=compute_dtype, softmax_aux=softmax_aux, mask_value=mask_value,
+                                  sliding_window=sliding_window, **ignore)
+        if is_4d:
+            output.attention_outputs = output.attention_outputs.reshape(shape4)
+        return output
+
+
+def _num_kv_heads(cache_view) -> int | None:
+    meta = getattr(cache_view, "metadata", None)
+    n = getattr(meta, "num_kv_heads", None)
+    return int(n) if n else None
+
+
+def _requirements(name: str, extra: MetadataField) -> OperationRequirements:
+    return (RequirementsBuilder(name)
+            .require_metadata(MetadataField.SEQ_LENS | MetadataField.CONTEXT_LENS | MetadataField.POSITIONS
+                              | MetadataField.QUERY_START_LOC | MetadataField.PAGES_TABLES | extra)
+            .optional_metadata(MetadataField.LOGITS_INDICES)
+            .support_cache(CacheType.RAGGED_PAGES)
+            .use_cache_view(RaggedPagesCacheView)
+            .build())
+
+
+@OperationRegistry.register
+class RaggedPageAttnV2(_RaggedPageAttn):
+    @classmethod
+    def get_impl_name(cls) -> str | tuple[str]:
+        return "ragged_page_attention_v2"
+
+    @classmethod
+    def get_requirements(cls, mode: ExecutionMode = ExecutionMode.MIXED) -> OperationRequirements:
+        return _requirements("ragged_page_attention_v2", MetadataField.SLOT_MAPPING)
+
+
+@OperationRegistry.register
+class RaggedPageAttnV3(_RaggedPageAttn):
+    @classmethod
+    def get_impl_name(cls) -> str | tuple[str]:
+        return "ragged_page_attention_v3"
+
+    @classmethod
+    def get_requirements(cls, mode: ExecutionMode = ExecutionMode.MIXED) -> OperationRequirements:
+        return _requirements("ragged_page_attention_v3", MetadataField.REQUEST_DISTRIBUTION)

@@ -70,12 +70,20 @@ class Workload:
             return np.minimum(ctx, self.sliding_window + self.q_lens.astype(np.int64) - 1)
         return ctx
 
-    def attention_bytes(self) -> int:
+    def small_row_mask(self) -> np.ndarray:
+        """Sequences the split-K decode kernel serves: at most 16 (token, group-head) rows per KV head."""
+        return (self.q_lens > 0) & (self.q_lens * (self.Hq // self.Hkv) <= 16)
+
+    def attention_bytes(self, select: np.ndarray | None = None) -> int:
         """Algorithmic HBM bytes of one attention call: every visible K/V element once per sequence,
-        q and out once, the block-table entries and lengths that are consulted, per-page scales if any."""
-        vis = self.visible_keys()[self.q_lens > 0]
+        q and out once, the block-table entries and lengths that are consulted, per-page scales if any.
+        ``select`` restricts the count to a subset of sequences (boolean mask)."""
+        live = self.q_lens > 0
+        if select is not None:
+            live = live & select
+        vis = self.visible_keys()[live]
         kv = int(vis.sum()) * self.Hkv * self.D * 2 * self.kv_elem_bytes
-        qo = self.T * self.Hq * self.D * 2 * self.q_elem_bytes
+        qo = int(self.q_lens[live].sum()) * self.Hq * self.D * 2 * self.q_elem_bytes
         pages = int(np.ceil(vis / self.page_size).sum())
         meta = pages * 4 + (2 * self.S + 1) * 4
         scales = pages * 2 * self.Hkv * 4 if self.kv_dtype in ("fp8", "int8") else 0
@@ -85,11 +93,11 @@ class Workload:
         """Read + write of the new K/V rows."""
         return 2 * self.T * 2 * self.Hkv * self.D * self.kv_elem_bytes
 
-    def attention_flops(self) -> int:
+    def attention_flops(self, select: np.ndarray | None = None) -> int:
         """4 * Hq * D flops per visible (query row, key) pair."""
         pairs = 0
-        for ctx, ql in zip(self.context_lens.astype(np.int64), self.q_lens.astype(np.int64)):
-            if ql <= 0:
+        for k, (ctx, ql) in enumerate(zip(self.context_lens.astype(np.int64), self.q_lens.astype(np.int64))):
+            if ql <= 0 or (select is not None and not select[k]):
                 continue
             pos = ctx - ql + np.arange(ql)
             n = pos + 1

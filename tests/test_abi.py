@@ -1,0 +1,53 @@
+"""The C-ABI library loads and exports every symbol include/rpa_hip.h declares (no compute calls: no GPU here)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from easydel_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rpa_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rpa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    names = _declared_symbols()
+    assert {"rpa_ragged_paged_attention", "rpa_ragged_paged_attention_v3", "rpa_page_scatter_slices", "rpa_page_scatter_ragged",
+            "rpa_attention_workspace_bytes", "rpa_version", "rpa_last_error", "rpa_set_tunable", "rpa_calibration_copy"} <= set(names)
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in rpa_hip.h but not exported by librpa_hip.so"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes prototype in easydel_amd/_lib.py"
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_host_only_entry_points():
+    lib = _lib.load()
+    assert re.fullmatch(r"\d+\.\d+\.\d+", lib.rpa_version().decode())
+    # argument validation happens before any device work
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 1, 1, 1, 16, 8, 3, 64, 6, 1, 1, 1.0, 0, 0.0)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"multiple of Hkv" in lib.rpa_last_error()
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 5, 1, 1.0, 0, 0.0)
+    assert rc == _lib.RPA_ERR_UNSUPPORTED
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 2, 1.0, 0, 0.0)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"kv_scales" in lib.rpa_last_error()
+    with pytest.raises(_lib.RpaError):
+        _lib.check(rc)
+    assert lib.rpa_page_scatter_slices(None, None, None, None, None, 0, 0, 0, 4, 16, 0) == 0  # empty input is a no-op
+    assert lib.rpa_page_scatter_slices(None, None, None, None, None, 4, 4, 64, 0, 16, 0) == _lib.RPA_ERR_INVALID_ARGUMENT
+    n = lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1)
+    assert n > 2 * 256 * 32 * 130 * 4
+    prev = _lib.set_tunable("max_splits", 4)
+    assert lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1) < n
+    _lib.set_tunable("max_splits", prev)
+    assert _lib.set_tunable("no_such_knob", 1) == -1
