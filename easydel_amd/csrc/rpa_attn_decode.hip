@@ -54,7 +54,7 @@ __device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* 
   return pc;
 }
 
-template <int D, int KVT, int TT, int WPB, int OCC>
+template <int D, int KVT, int TT, int WPB, int OCC, bool CAP>
 __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
@@ -111,9 +111,8 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
     for (int u = 0; u < NLD; ++u) stage[u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
   };
 
-  const bool has_cap = p.softcap > 0.f;
   const float cap_out = p.softcap * 1.4426950408889634f;
-  const float cap_in = has_cap ? p.scale / p.softcap : 0.f;
+  const float cap_in = CAP ? p.scale / p.softcap : 0.f;
 
   Piece cur = make_piece(p, P, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
   int page_cur = page_of(cur.i, cur.t_begin);
@@ -131,6 +130,9 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
   const int row_hi = min(pos + 1, cur.ctx);            // exclusive
   const int row_lo = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
   const int vis_lo = (p.window > 0) ? max(cur.ctx - cur.q_len - p.window + 1, 0) : 0;  // lowest key any row sees
+  // keys every row sees: from the last row's window start to the first row's causal limit
+  const int all_lo = (p.window > 0) ? max(cur.ctx - p.window, 0) : 0;
+  const int all_hi = cur.ctx - cur.q_len + 1;
 
   // ---- Q as B operands -----------------------------------------------------------------
   bf16x8 qf[NKK];
@@ -221,50 +223,18 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
     }
 
     // ---- online softmax (log2 domain) -------------------------------------------------------
-    if (has_cap) {
-#pragma unroll
-      for (int st = 0; st < NS; ++st)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) s_acc[st][j] = fast_tanh(s_acc[st][j] * (cap_in * k_scale));
-    }
-    const float sc_mul = has_cap ? cap_out : p.scale_log2 * k_scale;
-    float mx = -INFINITY;
-#pragma unroll
-    for (int st = 0; st < NS; ++st) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int tok = tb + st * 16 + 4 * g4 + j;
-        float s = s_acc[st][j] * sc_mul;
-        s = (tok >= row_lo && tok < row_hi) ? s : -INFINITY;
-        s_acc[st][j] = s;
-        mx = fmaxf(mx, s);
-      }
-    }
-    mx = xor32_max(xor16_max(mx));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-    m_run = m_new;
-    float psum = 0.f;
+    const float sc_mul = CAP ? cap_out : p.scale_log2 * k_scale;
     uint32_t pfrag[NS][2];
-#pragma unroll
-    for (int st = 0; st < NS; ++st) {
-      float pr[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        pr[j] = __builtin_amdgcn_exp2f(s_acc[st][j] - m_use);
-        psum += pr[j];
-      }
-      pfrag[st][0] = pack_bf16(pr[0], pr[1]);
-      pfrag[st][1] = pack_bf16(pr[2], pr[3]);
-    }
-    l_run = l_run * alpha + psum;
+    float alpha;
+    if (tb >= all_lo && tb + TT <= all_hi)
+      alpha = softmax_step<false, CAP, NS>(s_acc, sc_mul, cap_in * k_scale, tb, g4, row_lo, row_hi, m_run, l_run, pfrag);
+    else
+      alpha = softmax_step<true, CAP, NS>(s_acc, sc_mul, cap_in * k_scale, tb, g4, row_lo, row_hi, m_run, l_run, pfrag);
     // The accumulators hold sum(p * v_code) in units of the current page's V scale, so P stays an exact
     // softmax weight in bf16; when the scale changes (a new page) they are converted once.
     float o_mul = alpha;
     if constexpr (EB == 1) {
-      o_mul = alpha * (v_unit * __builtin_amdgcn_rcpf(v_scale));
-      if (v_unit == v_scale) o_mul = alpha;
+      if (v_unit != v_scale) o_mul = alpha * (v_unit * __builtin_amdgcn_rcpf(v_scale));
       v_unit = v_scale;
     }
     if (__any(o_mul != 1.f)) {
@@ -273,37 +243,27 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
     }
 
     // ---- O^T += V^T . P^T ---------------------------------------------------------------------
+    // bf16 pages: ds_read_b64_tr_b16 hands each lane the key-major column it needs (inside a 16-lane group,
+    // lane l addresses key 4g4 + l/4, dims d0 + 4(l%4).. and receives dim d0 + l of keys 4g4..4g4+3).
+    // 8-bit pages: each lane reads 4 keys x 4 consecutive dims of codes and widens them while transposing.
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
       const u32x2 pb2 = {pfrag[st][0], pfrag[st][1]};
       const s16x4 pb = __builtin_bit_cast(s16x4, pb2);
       if constexpr (EB == 2) {
-        // raw[e][w]: token 4g4+e, dword w of this lane's DPL dims (2 dims per dword)
-        uint32_t raw[4][DPL / 2];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int tk = st * 16 + 4 * g4 + e;
-          const unsigned char* vrow = lds_v + tk * RK;
-          const int key = swz_key<RK>(tk);
-          if constexpr (VB >= 16) {
-#pragma unroll
-            for (int r = 0; r < VB / 16; ++r) {
-              const u32x4 v = *(const u32x4*)(vrow + ((((n * VB) / 16 + r) ^ key) << 4));
-              raw[e][4 * r + 0] = v[0]; raw[e][4 * r + 1] = v[1]; raw[e][4 * r + 2] = v[2]; raw[e][4 * r + 3] = v[3];
-            }
-          } else {  // VB == 8
-            const u32x2 v = *(const u32x2*)(vrow + ((((n * VB) >> 4) ^ key) << 4) + ((n * VB) & 15));
-            raw[e][0] = v[0]; raw[e][1] = v[1];
-          }
-        }
+        const int tk = st * 16 + 4 * g4 + (n >> 2);
+        const unsigned char* vrow = lds_v + tk * RK;
+        const int key = swz_key<RK>(tk);
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) {
-          const uint32_t sel = (rt & 1) ? 0x07060302u : 0x05040100u;
-          const u32x2 a2 = {__builtin_amdgcn_perm(raw[1][rt >> 1], raw[0][rt >> 1], sel),
-                            __builtin_amdgcn_perm(raw[3][rt >> 1], raw[2][rt >> 1], sel)};
-          o_acc[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), pb, o_acc[rt], 0, 0, 0);
+          const int off = rt * 32 + (n & 3) * 8;
+          const unsigned char* ptr = vrow + (((off >> 4) ^ key) << 4) + (off & 15);
+          const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr);
+          o_acc[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, o_acc[rt], 0, 0, 0);
         }
       } else {
+        // lane (n, g4) reads DPL consecutive dims (DPL*n ..) of keys 4g4..4g4+3 and widens them; row tile rt
+        // of this path therefore holds dims DPL*i + rt (any dim permutation works for O^T, see the epilogue)
         float vf[4][DPL];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -336,30 +296,40 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
     __builtin_amdgcn_wave_barrier();
   }
 
-  // ---- epilogue: lane (n, g4) holds dims [4*DPL*g4, 4*DPL*(g4+1)) of row n, ordered j*DPL + rt ----
+  // ---- epilogue ---------------------------------------------------------------------------------
+  // accumulator column j of row tile rt is dim 16rt + 4g4 + j (bf16 pages) or DPL*(4g4 + j) + rt (8-bit pages)
   float l_tot = l_run + __shfl_xor(l_run, 16);
   l_tot += __shfl_xor(l_tot, 32);
   if (n < rows) {
     const int tok_out = cur.q0 + r_tok;
     const int head_out = h * G + r_head;
-    const int d_base = 4 * DPL * g4;
     if (cur.single) {
       const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
-      uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D + d_base;
+      uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D;
+      if constexpr (EB == 2) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-#pragma unroll
-        for (int rt = 0; rt < DPL; rt += 2) {
-          *(uint32_t*)(orow + j * DPL + rt) = pack_bf16(o_acc[rt][j] * inv, o_acc[rt + 1][j] * inv);
+        for (int rt = 0; rt < DPL; ++rt) {
+          const u32x2 w = {pack_bf16(o_acc[rt][0] * inv, o_acc[rt][1] * inv), pack_bf16(o_acc[rt][2] * inv, o_acc[rt][3] * inv)};
+          *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
         }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int rt = 0; rt < DPL; rt += 2)
+            *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rt][j] * inv, o_acc[rt + 1][j] * inv);
       }
     } else {
       const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok) * p.Hq + head_out;
-      float* prow = p.part_o + slot * D + d_base;
+      float* prow = p.part_o + slot * D;
+      if constexpr (EB == 2) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+        for (int rt = 0; rt < DPL; ++rt) *(f32x4*)(prow + 16 * rt + 4 * g4) = o_acc[rt];
+      } else {
 #pragma unroll
-        for (int rt = 0; rt < DPL; ++rt) prow[j * DPL + rt] = o_acc[rt][j] * v_unit;
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int rt = 0; rt < DPL; ++rt) prow[DPL * (4 * g4 + j) + rt] = o_acc[rt][j] * v_unit;
       }
       if (g4 == 0) {
         p.part_ml[slot * 2 + 0] = m_run;
@@ -439,15 +409,15 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   }
 }
 
-template <int D, int KVT, int TT, int WPB, int OCC>
-static int launch_one(hipStream_t stream, AttnParams p) {
+template <int D, int KVT, int TT, int WPB, int OCC, bool CAP>
+static int launch_cap(hipStream_t stream, AttnParams p) {
   // persistent grid: as many workgroups as are resident at once, per KV-head group
   static int resident = 0;
   if (resident == 0) {
     int dev = 0, cus = 0, per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, OCC>, 64 * WPB, 0) != hipSuccess)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, OCC, CAP>, 64 * WPB, 0) != hipSuccess)
       return (int)hipGetLastError();
     resident = max(1, cus * max(1, per_cu));
   }
@@ -458,8 +428,13 @@ static int launch_one(hipStream_t stream, AttnParams p) {
   p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2)
-    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, OCC>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, OCC, CAP>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();
+}
+
+template <int D, int KVT, int TT, int WPB, int OCC>
+static int launch_one(hipStream_t stream, const AttnParams& p) {
+  return p.softcap > 0.f ? launch_cap<D, KVT, TT, WPB, OCC, true>(stream, p) : launch_cap<D, KVT, TT, WPB, OCC, false>(stream, p);
 }
 
 template <int D, int KVT, int TT, int WPB>

@@ -16,7 +16,7 @@
 
 namespace rpa {
 
-template <int D, int KVT, int TT, int NW, int RB>
+template <int D, int KVT, int TT, int NW, int RB, bool CAP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
   constexpr int RKL = D * 2;             // bytes of one K (or V) row in LDS (always bf16)
@@ -24,9 +24,9 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
   constexpr int LPTG = HBG / 16;         // 16-byte global chunks per token span
   constexpr int THREADS = 64 * NW;
   constexpr int NLD = (TT * LPTG + THREADS - 1) / THREADS;  // global loads per thread per tile
+  constexpr bool FULL = (TT * LPTG) % THREADS == 0;         // every thread has NLD chunks of every tile
   constexpr int NS = TT / 16;            // 16-key sub-tiles per tile
-  constexpr int DPL = D / 16;            // output dims per lane per accumulator column
-  constexpr int VB = DPL * 2;            // bytes of V one lane reads per key
+  constexpr int DPL = D / 16;            // 16-dim row tiles of O^T
   constexpr int NKK = D / 32;            // k-steps of the score MFMA
   constexpr int ROWS = NW * RB * 16;
   constexpr int TILE_BYTES = TT * 2 * RKL;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
 #pragma unroll
   for (int u = 0; u < NLD; ++u) {
     const int idx = u * THREADS + tid;
-    st_ok[u] = idx < TT * LPTG;
+    st_ok[u] = FULL || idx < TT * LPTG;
     st_tok[u] = st_ok[u] ? idx / LPTG : 0;
     const int c = idx % LPTG;
     st_v[u] = c >= LPTG / 2;
@@ -147,13 +147,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride;
 #pragma unroll
     for (int u = 0; u < NLD; ++u)
-      if (st_ok[u]) stage[u] = *(const u32x4*)(base + st_off[u]);
+      if (FULL || st_ok[u]) stage[u] = *(const u32x4*)(base + st_off[u]);
   };
   auto commit = [&](int tb, unsigned char* buf) {  // registers -> LDS tile (zeroing keys nobody may see)
     const bool edge = (tb + TT > sp.ctx) || (tb < vis_lo);
 #pragma unroll
     for (int u = 0; u < NLD; ++u) {
-      if (!st_ok[u]) continue;
+      if (!FULL && !st_ok[u]) continue;
       u32x4 v = stage[u];
       if (edge) {
         const int tok = tb + st_tok[u];
@@ -172,9 +172,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     }
   };
 
-  const bool has_cap = p.softcap > 0.f;
   const float cap_out = p.softcap * 1.4426950408889634f;
-  const float cap_in = has_cap ? p.scale / p.softcap : 0.f;
+  const float cap_in = CAP ? p.scale / p.softcap : 0.f;
 
   float m_run[RB], l_run[RB];
   float v_unit = 1.f;  // V scale the accumulators are currently expressed in (8-bit pages)
@@ -231,48 +230,14 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
 
       // ---- online softmax per row block -------------------------------------------------------------
       const bool inside = (tb >= wave_lo) && (tb + TT <= wave_hi);  // no row of the wave masks any key here
+      const float sc_mul = CAP ? cap_out : p.scale_log2 * k_scale;
+      const float cap_k = cap_in * k_scale;
       uint32_t pfrag[RB][NS][2];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        if (has_cap) {
-#pragma unroll
-          for (int st = 0; st < NS; ++st)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) s_acc[rb][st][j] = fast_tanh(s_acc[rb][st][j] * (cap_in * k_scale));
-        }
-        const float sc_mul = has_cap ? cap_out : p.scale_log2 * k_scale;
-        float mx = -INFINITY;
-#pragma unroll
-        for (int st = 0; st < NS; ++st) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            float s = s_acc[rb][st][j] * sc_mul;
-            if (!inside) {
-              const int tok = tb + st * 16 + 4 * g4 + j;
-              s = (tok >= row_lo[rb] && tok < row_hi[rb]) ? s : -INFINITY;
-            }
-            s_acc[rb][st][j] = s;
-            mx = fmaxf(mx, s);
-          }
-        }
-        mx = xor32_max(xor16_max(mx));
-        const float m_new = fmaxf(m_run[rb], mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_use);
-        m_run[rb] = m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int st = 0; st < NS; ++st) {
-          float pr[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            pr[j] = __builtin_amdgcn_exp2f(s_acc[rb][st][j] - m_use);
-            psum += pr[j];
-          }
-          pfrag[rb][st][0] = pack_bf16(pr[0], pr[1]);
-          pfrag[rb][st][1] = pack_bf16(pr[2], pr[3]);
-        }
-        l_run[rb] = l_run[rb] * alpha + psum;
+        float alpha;
+        if (inside) alpha = softmax_step<false, CAP, NS>(s_acc[rb], sc_mul, cap_k, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+        else alpha = softmax_step<true, CAP, NS>(s_acc[rb], sc_mul, cap_k, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
         // accumulators are kept in units of the current page's V scale (see the decode kernel)
         float o_mul = alpha;
         if constexpr (EB == 1) {
@@ -286,30 +251,26 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
       v_unit = v_scale;
 
       // ---- O^T += V^T . P^T (V operands shared by the row blocks) -----------------------------------
-      uint32_t raw[4 * NS][DPL / 2];  // raw[e][w]: key (e < 4 ? 4g4+e : 16+4g4+e-4), dword w of this lane's DPL dims
-#pragma unroll
-      for (int e = 0; e < 4 * NS; ++e) {
-        const int tk = (e >> 2) * 16 + 4 * g4 + (e & 3);
-        const unsigned char* vrow = lds_v + tk * RKL;
-        const int key = swz_key<RKL>(tk);
-        if constexpr (VB >= 16) {
-#pragma unroll
-          for (int r = 0; r < VB / 16; ++r) {
-            const u32x4 v = *(const u32x4*)(vrow + ((((n * VB) / 16 + r) ^ key) << 4));
-            raw[e][4 * r + 0] = v[0]; raw[e][4 * r + 1] = v[1]; raw[e][4 * r + 2] = v[2]; raw[e][4 * r + 3] = v[3];
-          }
-        } else {  // VB == 8
-          const u32x2 v = *(const u32x2*)(vrow + ((((n * VB) >> 4) ^ key) << 4) + ((n * VB) & 15));
-          raw[e][0] = v[0]; raw[e][1] = v[1];
-        }
-      }
+      // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16
+      // (key 4g4 + l/4, dims d0 + 4(l%4)..) and receives the transposed column: for dim d0 + (l&15) the
+      // values of keys 4g4..4g4+3, which is the A operand of the product with k = keys.
+      const int tr_key = 4 * g4 + (n >> 2);          // key (within a 16-key sub-tile) this lane addresses
+      const int tr_byte = (n & 3) * 8;               // byte offset of its 4 dims inside the 32-byte row-tile span
 #pragma unroll
       for (int rt = 0; rt < DPL; ++rt) {
-        const uint32_t sel = (rt & 1) ? 0x07060302u : 0x05040100u;
-        const int w = rt >> 1;
+        u32x2 a_lo, a_hi;
+        {
+          const int tk = tr_key;
+          const int off = rt * 32 + tr_byte;
+          const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+          a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
+        }
         if constexpr (NS == 2) {
-          const u32x4 a4 = {__builtin_amdgcn_perm(raw[1][w], raw[0][w], sel), __builtin_amdgcn_perm(raw[3][w], raw[2][w], sel),
-                            __builtin_amdgcn_perm(raw[5][w], raw[4][w], sel), __builtin_amdgcn_perm(raw[7][w], raw[6][w], sel)};
+          const int tk = 16 + tr_key;
+          const int off = rt * 32 + tr_byte;
+          const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+          a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
+          const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
             const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
@@ -317,11 +278,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
                                                                     o_acc[rb][rt], 0, 0, 0);
           }
         } else {
-          const u32x2 a2 = {__builtin_amdgcn_perm(raw[1][w], raw[0][w], sel), __builtin_amdgcn_perm(raw[3][w], raw[2][w], sel)};
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
             const u32x2 b2 = {pfrag[rb][0][0], pfrag[rb][0][1]};
-            o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), __builtin_bit_cast(s16x4, b2),
+            o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a_lo), __builtin_bit_cast(s16x4, b2),
                                                                       o_acc[rb][rt], 0, 0, 0);
           }
         }
@@ -339,12 +299,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     l_tot += __shfl_xor(l_tot, 32);
     if (row_ok[rb]) {
       const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
-      uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * DPL * g4;
+      uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int rt = 0; rt < DPL; rt += 2)
-          *(uint32_t*)(orow + j * DPL + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
+      for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
+        const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                         pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+        *(u32x2*)(orow + 16 * rt) = w;
+      }
     }
   }
 }
@@ -355,7 +316,10 @@ static int launch_one(hipStream_t stream, const AttnParams& p) {
   const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
   const int64_t blocks = slots * p.Hkv;
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL((attn_prefill_kernel<D, KVT, TT, NW, RB>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  if (p.softcap > 0.f)
+    hipLaunchKernelGGL((attn_prefill_kernel<D, KVT, TT, NW, RB, true>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  else
+    hipLaunchKernelGGL((attn_prefill_kernel<D, KVT, TT, NW, RB, false>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
   return (int)hipGetLastError();
 }
 

@@ -70,4 +70,50 @@ __device__ __forceinline__ float fast_tanh(float x) {
   return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
 }
 
+
+// Online-softmax step of one 16-row block over NS 16-key sub-tiles held as S^T accumulators (lane = query row
+// n, 4 keys 4*g4 + j per sub-tile).  Scales the raw scores (soft cap first if CAP), masks keys outside
+// [row_lo, row_hi) if MASK, updates the running max / sum, and leaves the probabilities as packed bf16 B
+// operands.  Returns the factor the output accumulators must be multiplied by (exp2 of the max change).
+template <bool MASK, bool CAP, int NS>
+__device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, float cap_in, int tb, int g4,
+                                              int row_lo, int row_hi, float& m_run, float& l_run,
+                                              uint32_t (&pfrag)[NS][2]) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int st = 0; st < NS; ++st) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float s = s_acc[st][j];
+      if constexpr (CAP) s = fast_tanh(s * cap_in);
+      s *= sc_mul;
+      if constexpr (MASK) {
+        const int tok = tb + st * 16 + 4 * g4 + j;
+        s = (tok >= row_lo && tok < row_hi) ? s : -INFINITY;
+      }
+      s_acc[st][j] = s;
+      mx = fmaxf(mx, s);
+    }
+  }
+  mx = xor32_max(xor16_max(mx));
+  const float m_new = fmaxf(m_run, mx);
+  const float m_use = (MASK && m_new == -INFINITY) ? 0.f : m_new;
+  const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+  m_run = m_new;
+  float psum = 0.f;
+#pragma unroll
+  for (int st = 0; st < NS; ++st) {
+    float pr[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      pr[j] = __builtin_amdgcn_exp2f(s_acc[st][j] - m_use);
+      psum += pr[j];
+    }
+    pfrag[st][0] = pack_bf16(pr[0], pr[1]);
+    pfrag[st][1] = pack_bf16(pr[2], pr[3]);
+  }
+  l_run = l_run * alpha + psum;
+  return alpha;
+}
+
 }  // namespace rpa
