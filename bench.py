@@ -40,6 +40,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
     ap.add_argument("--decode-wgs", type=int, default=0)
+    ap.add_argument("--prefill-chunks", type=int, default=0)
+    ap.add_argument("--decode-sync", type=int, default=-1)
     ap.add_argument("--max-splits", type=int, default=0)
     ap.add_argument("--sequential-pages", action="store_true", help="experiment: block tables in pool order")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -142,6 +144,10 @@ def main():
     _lib.load()
     if args.decode_wgs:
         _lib.set_tunable("decode_wgs", args.decode_wgs)
+    if args.decode_sync >= 0:
+        _lib.set_tunable("decode_sync", args.decode_sync)
+    if args.prefill_chunks:
+        _lib.set_tunable("prefill_chunks", args.prefill_chunks)
     if args.max_splits:
         _lib.set_tunable("max_splits", args.max_splits)
     if args.decode_wpb:

@@ -19,6 +19,8 @@ namespace {
 
 thread_local char g_err[512] = "";
 std::atomic<int> g_max_splits{0};   // 0 = sized from the shapes
+std::atomic<int> g_prefill_chunks{0};  // 0 = default (kMaxPrefillChunks)
+std::atomic<int> g_decode_sync{8};  // workgroup barrier every this many decode tiles (power of two, 0 = never)
 std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are resident at once
 std::atomic<int> g_force_generic{0};
 std::atomic<int> g_decode_wpb{0};
@@ -58,6 +60,24 @@ int static_splits(int T, int M, int page_size, int Hq, int D) {
   return (int)want;
 }
 
+// Prefill split-K: keys per chunk and number of chunks the partial buffers hold, from the static bounds.
+// A row tile's key range is cut into at most kMaxPrefillChunks chunks of at least 2048 keys; the partial
+// buffers ([chunks][T][Hq][D+2] floats) are kept under ~1 GiB by allowing fewer, longer chunks.
+void prefill_split(int T, int M, int page_size, int Hq, int D, int* chunk_keys, int* max_chunks) {
+  const long span = (long)M * page_size;
+  int chunks = g_prefill_chunks.load() > 0 ? g_prefill_chunks.load() : rpa::kMaxPrefillChunks;
+  if (chunks > rpa::kMaxPrefillChunks) chunks = rpa::kMaxPrefillChunks;
+  const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
+  while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
+  long keys = (span + chunks - 1) / chunks;
+  if (keys < 2048) keys = 2048;
+  keys = (keys + 63) & ~63L;
+  chunks = (int)((span + keys - 1) / keys);
+  if (chunks < 1) chunks = 1;
+  *chunk_keys = (int)keys;
+  *max_chunks = chunks;
+}
+
 size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + 2 * ((size_t)S + 1) + rpa::kMaxDecodeWgs) * 4); }
 
 // Static bound on query tokens the decode kernel can own: sequences with at most 16 rows per KV head.
@@ -82,6 +102,12 @@ int rpa_set_tunable(const char* name, int value) {
     if (value < 0) value = 0;
     if (value > rpa::kMaxSplitsCap) value = rpa::kMaxSplitsCap;
     return g_max_splits.exchange(value);
+  }
+  if (!strcmp(name, "prefill_chunks")) return g_prefill_chunks.exchange(value < 0 ? 0 : value);
+  if (!strcmp(name, "decode_sync")) {
+    int pow2 = 0;
+    if (value > 0) for (pow2 = 1; pow2 * 2 <= value && pow2 < 1024; pow2 *= 2) {}
+    return g_decode_sync.exchange(pow2);
   }
   if (!strcmp(name, "decode_wgs")) return g_decode_wgs.exchange(value < 0 ? 0 : value);
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
@@ -135,7 +161,10 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
   if (Hkv <= 0 || Hq % Hkv != 0) return 256;
   const int td = decode_token_bound(T, S, Hq, Hkv);
   const int splits = static_splits(td, M, page_size, Hq, D);
-  return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + plan_bytes(S) + 256;
+  int pre_keys, pre_chunks;
+  prefill_split(T, M, page_size, Hq, D, &pre_keys, &pre_chunks);
+  const size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) : 0;
+  return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256;
 }
 
 int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages, const float* kv_scales,
@@ -154,6 +183,8 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   if (D > 256 || D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: head_dim %d (want a multiple of 4, <= 256)", D);
   if ((kv_dtype == RPA_FP8_E4M3 || kv_dtype == RPA_INT8) && !kv_scales)
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: 8-bit KV pages need kv_scales");
+  if (kv_scales && ((uintptr_t)kv_scales & 7))
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: kv_scales must be 8-byte aligned");
   if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: softmax_scale is not finite");
   if (T == 0) return RPA_OK;
   if (!q || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs || !out)
@@ -173,9 +204,12 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   p.window = sliding_window > 0 ? sliding_window : 0;
   p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
   p.decode_wgs = g_decode_wgs.load();
+  p.decode_sync = g_decode_sync.load();
   p.decode_wpb = g_decode_wpb.load();
   p.decode_occ = g_decode_occ.load();
   p.max_splits = 2;
+  p.pre_chunk = 1 << 30;
+  p.pre_max_chunks = 1;
   p.mfma_path = (!g_force_generic.load() && rpa::decode_supported(p)) ? 1 : 0;
 
   hipStream_t s = (hipStream_t)stream;
@@ -185,16 +219,30 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
     p.t_dec_max = td;
     const size_t po = part_o_bytes(td, Hq, D), pml = part_ml_bytes(td, Hq), pb = plan_bytes(S);
     int splits = static_splits(td, M, page_size, Hq, D);
-    const size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
+    int pre_keys, pre_chunks;
+    prefill_split(T, M, page_size, Hq, D, &pre_keys, &pre_chunks);
+    const size_t pre_po = part_o_bytes(T, Hq, D), pre_pml = part_ml_bytes(T, Hq);
+    size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (pre_po + pre_pml) : 0;
+    size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
     if (!workspace || usable < 2 * (po + pml))
       return fail(RPA_ERR_WORKSPACE, "rpa_ragged_paged_attention: workspace %zu bytes < %zu needed for two partial slots",
                   workspace_bytes, 2 * (po + pml) + pb + 256);
+    if (usable < pre + 2 * (po + pml)) {  // a small workspace: prefill rows are not split over keys
+      pre = 0;
+      pre_chunks = 1;
+    }
+    usable -= pre;
     if ((size_t)splits * (po + pml) > usable) splits = (int)(usable / (po + pml));
     p.max_splits = splits;
+    p.pre_chunk = pre_keys;
+    p.pre_max_chunks = pre_chunks;
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     p.plan = (int32_t*)base;
     p.part_o = (float*)(base + pb);
     p.part_ml = (float*)(base + pb + (size_t)splits * po);
+    char* pre_base = base + pb + (size_t)splits * (po + pml);
+    p.pre_o = (float*)pre_base;
+    p.pre_ml = (float*)(pre_base + (size_t)pre_chunks * pre_po);
     int err = 0;
     if (stages & 3) err = rpa::launch_attn_decode(s, p, stages & 3);
     if (err) return hip_fail(err, "decode kernel launch");

@@ -17,6 +17,8 @@
 // fp8 / int8 pages are widened to bf16 (exactly) after the LDS read; their per-(page, head)
 // scales fold into the score scale (K) and into P (V).
 // No barriers: LDS tiles are wave-private and LDS operations of one wave execute in order.
+#include <type_traits>
+
 #include "rpa_mfma.h"
 
 namespace rpa {
@@ -67,6 +69,10 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
   constexpr int DPL = D / 16;          // output dims per lane per accumulator register column
   constexpr int VB = DPL * EB;         // bytes of V one lane reads per token
   constexpr int NKK = D / 32;          // k-steps of the score MFMA
+  // Tiles in flight per wave (register staging buffers).  Two were measured slower than one on MI355X (780 vs
+  // 766 us on the Llama-shaped decode batch): eight waves with one 8 KiB tile each already saturate a CU's
+  // memory pipe, and the extra registers and code only delay the next issue.
+  constexpr int DEPTH = 1;
   static_assert(LPT <= 64 && TT % TPI == 0 && TT % 16 == 0, "tile shape");
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_all[WPB * TT * HB];
@@ -99,24 +105,30 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
   const char* pages = (const char*)p.kv_pages;
   const int64_t lane_goff = (int64_t)h * HB + c32 * 16 + (int64_t)sub * p.token_stride;
 
-  u32x4 stage[NLD];
+  u32x4 stage[DEPTH][NLD];
+  u32x2 sc_stage[DEPTH];  // (K scale, V scale) of the staged tile's page: fetched with the tile, in order behind it
   auto page_of = [&](int seq, int tok) -> int {
     int pgid = p.block_tables[(int64_t)seq * p.M + tok / pg];
     pgid = __builtin_amdgcn_readfirstlane(pgid);
     return min(max(pgid, 0), p.P - 1);
   };
-  auto issue = [&](int tb, int page) {
+  auto issue = [&](auto buf, int tb, int page) {  // buf: std::integral_constant, so the register array index is static
+    constexpr int B = decltype(buf)::value;
     const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride + lane_goff;
 #pragma unroll
-    for (int u = 0; u < NLD; ++u) stage[u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
+    for (int u = 0; u < NLD; ++u) stage[B][u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
+    // a vector load on purpose: a scalar load would be waited for together with the next LDS read
+    if constexpr (EB == 1) sc_stage[B] = *(const u32x2*)(p.kv_scales + (int64_t)page * p.C + 2 * h);
   };
+  using Buf0 = std::integral_constant<int, 0>;
+  using Buf1 = std::integral_constant<int, DEPTH - 1>;
 
   const float cap_out = p.softcap * 1.4426950408889634f;
   const float cap_in = CAP ? p.scale / p.softcap : 0.f;
 
   Piece cur = make_piece(p, P, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
-  int page_cur = page_of(cur.i, cur.t_begin);
-  issue(cur.t_begin, page_cur);  // first tile in flight before anything else is set up
+  int page_a = page_of(cur.i, cur.t_begin), page_b = 0;  // pages of the tiles in staging buffers 0 and 1
+  issue(Buf0{}, cur.t_begin, page_a);  // first tile in flight before anything else is set up
 
   for (;;) {
   const int rows = cur.q_len * G;
@@ -164,37 +176,26 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
 #pragma unroll
   for (int rt = 0; rt < DPL; ++rt) o_acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    const int tb = t_begin + tile * TT;
-    // ---- registers -> LDS (zero rows past the context end or left of every row's window, so stale
-    //      or null-page bytes cannot reach P.V as 0 * NaN)
+  // ---- registers -> LDS (zero rows past the context end or left of every row's window, so stale or
+  //      null-page bytes cannot reach P.V as 0 * NaN)
+  auto commit = [&](auto buf, int tb) {
+    constexpr int B = decltype(buf)::value;
     if (tb + TT > cur.ctx || tb < vis_lo) {
 #pragma unroll
       for (int u = 0; u < NLD; ++u) {
         const int tok = tb + u * TPI + sub;
-        if (tok >= cur.ctx || tok < vis_lo) stage[u] = (u32x4){0u, 0u, 0u, 0u};
+        if (tok >= cur.ctx || tok < vis_lo) stage[B][u] = (u32x4){0u, 0u, 0u, 0u};
       }
     }
 #pragma unroll
     for (int u = 0; u < NLD; ++u) {
       const int tk = u * TPI + sub;
       unsigned char* dst = (is_v ? lds_v : lds_k) + tk * RK + ((cc ^ swz_key<RK>(tk)) << 4);
-      *(u32x4*)dst = stage[u];
+      *(u32x4*)dst = stage[B][u];
     }
-    float k_scale = 1.f, v_scale = 1.f;
-    if constexpr (EB == 1) {
-      const float* sc = p.kv_scales + (int64_t)page_cur * p.C + 2 * h;
-      k_scale = sc[0];
-      v_scale = sc[1];
-    }
-    // ---- prefetch the next tile into registers ---------------------------------------------
-    if (tile + 1 < n_tiles) {
-      page_cur = page_of(cur.i, tb + TT);
-      issue(tb + TT, page_cur);
-    } else if (has_next) {
-      page_cur = page_nxt;
-      issue(nxt.t_begin, page_nxt);
-    }
+  };
+
+  auto compute = [&](int tb, float k_scale, float v_scale) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 
@@ -294,6 +295,49 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
       }
     }
     __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---- tile loop: DEPTH tiles in flight; the next piece's first tile is issued into buffer 0 as soon as this
+  //      piece no longer needs it, so the stream of loads never drains at a piece boundary
+  if (DEPTH == 2 && n_tiles > 1) {
+    page_b = page_of(cur.i, t_begin + TT);
+    issue(Buf1{}, t_begin + TT, page_b);
+  }
+  for (int tile = 0; tile < n_tiles; tile += DEPTH) {
+    const int tb = t_begin + tile * TT;
+    // The waves of a workgroup read adjacent 512-byte spans of the same token rows; a barrier every few tiles
+    // keeps them in step so each DRAM row is opened once (740 vs 764 us).  All waves of a workgroup walk the
+    // same pieces and tiles, so every live wave reaches every barrier.
+    if (p.decode_sync > 0 && (tile & (p.decode_sync - 1)) == 0) __builtin_amdgcn_s_barrier();
+    commit(Buf0{}, tb);
+    float ks = 1.f, vs = 1.f;
+    if constexpr (EB == 1) {
+      ks = __uint_as_float(sc_stage[0][0]);
+      vs = __uint_as_float(sc_stage[0][1]);
+    }
+    if (tile + DEPTH < n_tiles) {
+      page_a = page_of(cur.i, tb + DEPTH * TT);
+      issue(Buf0{}, tb + DEPTH * TT, page_a);
+    } else if (has_next) {
+      page_a = page_nxt;
+      issue(Buf0{}, nxt.t_begin, page_nxt);
+    }
+    compute(tb, ks, vs);
+    if constexpr (DEPTH == 2) {
+      if (tile + 1 < n_tiles) {
+        commit(Buf1{}, tb + TT);
+        float ks_b = 1.f, vs_b = 1.f;
+        if constexpr (EB == 1) {
+          ks_b = __uint_as_float(sc_stage[DEPTH - 1][0]);
+          vs_b = __uint_as_float(sc_stage[DEPTH - 1][1]);
+        }
+        if (tile + 3 < n_tiles) {
+          page_b = page_of(cur.i, tb + 3 * TT);
+          issue(Buf1{}, tb + 3 * TT, page_b);
+        }
+        compute(tb + TT, ks_b, vs_b);
+      }
+    }
   }
 
   // ---- epilogue ---------------------------------------------------------------------------------
@@ -352,9 +396,13 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   const int S = p.S, tid = threadIdx.x;
   const int per = (S + 1023) / 1024;
   const int i0 = min(S, tid * per), i1 = min(S, i0 + per);
+  __shared__ int s_large;
+  if (tid == 0) s_large = 0;
+  __syncthreads();
   auto span_of = [&](int i, int& toks) -> int {
     const SeqPlan sp = seq_plan(p, i);
     toks = 0;
+    if (sp.live && !sp.small_rows) s_large = 1;  // benign race: every writer stores 1
     if (!sp.live || !sp.small_rows) return 0;
     toks = sp.q_len;
     return (sp.hi - sp.lo + 63) & ~63;
@@ -391,6 +439,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     q = max(max(q, q_min), 256);
     plan[0] = W;
     plan[1] = q;
+    plan[2] = s_large;  // any sequence for the large-row (prefill) kernel?
     s_Q = q;
   }
   __threadfence_block();

@@ -19,6 +19,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   const int D = p.D;
   bool zero = false;
   int n_pieces = 0, part_row = 0;
+  const float* part_o = p.part_o;
+  const float* part_ml = p.part_ml;
+  int64_t stride = (int64_t)p.t_dec_max * p.Hq;  // slots between consecutive pieces
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) {
     zero = true;
   } else {
@@ -28,6 +31,13 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
     else if (p.mfma_path && sp.small_rows) {
       n_pieces = decode_pieces(p.plan, i);
       part_row = p.plan[kPlanHeader + p.S + 1 + i] + (t - sp.q0);
+    } else if (p.mfma_path && p.pre_max_chunks > 1) {  // prefill row tile split over key chunks
+      const int row = (t - sp.q0) * p.group + hq % p.group;
+      n_pieces = prefill_tile(p, sp, (row / kPrefillRows) * kPrefillRows).n_chunks;
+      part_row = t;
+      part_o = p.pre_o;
+      part_ml = p.pre_ml;
+      stride = (int64_t)p.T * p.Hq;
     }
   }
   const bool merge = n_pieces > 1;
@@ -36,10 +46,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   float acc[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, lane+128, lane+192
   float inv = 0.f;
   if (merge) {
-    const int64_t stride = (int64_t)p.t_dec_max * p.Hq;  // slots between consecutive pieces
     const int64_t slot0 = (int64_t)part_row * p.Hq + hq;
     float m = -INFINITY;
-    for (int c = lane; c < n_pieces; c += 64) m = fmaxf(m, p.part_ml[(slot0 + c * stride) * 2]);
+    for (int c = lane; c < n_pieces; c += 64) m = fmaxf(m, part_ml[(slot0 + c * stride) * 2]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
     const float m_use = (m == -INFINITY) ? 0.f : m;
@@ -48,14 +57,14 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
       const int c_mine = base + lane;
       float w_c = 0.f;
       if (c_mine < n_pieces) {
-        const float2 ml = *(const float2*)(p.part_ml + (slot0 + c_mine * stride) * 2);
+        const float2 ml = *(const float2*)(part_ml + (slot0 + c_mine * stride) * 2);
         w_c = __builtin_amdgcn_exp2f(ml.x - m_use);
         l += w_c * ml.y;
       }
       const int cnt = min(64, n_pieces - base);
       for (int c = 0; c < cnt; ++c) {
         const float w = __shfl(w_c, c);
-        const float* row = p.part_o + (slot0 + (base + c) * stride) * D;
+        const float* row = part_o + (slot0 + (base + c) * stride) * D;
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
           const int d = lane + 64 * k;

@@ -29,6 +29,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
   constexpr int DPL = D / 16;            // 16-dim row tiles of O^T
   constexpr int NKK = D / 32;            // k-steps of the score MFMA
   constexpr int ROWS = NW * RB * 16;
+  static_assert(ROWS == kPrefillRows, "merge kernel assumes this row-tile height");
   constexpr int TILE_BYTES = TT * 2 * RKL;
   static_assert(NS == 1 || NS == 2, "tile is one or two 16-key sub-tiles");
 
@@ -42,7 +43,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
 
   // ---- block -> (sequence, row tile, KV head) ---------------------------------------------------
   const int h = blockIdx.x % p.Hkv;
-  const int slot = blockIdx.x / p.Hkv;
+  const int n_slots = gridDim.x / (p.Hkv * p.pre_max_chunks);
+  const int slot = (blockIdx.x / p.Hkv) % n_slots;
+  const int chunk = blockIdx.x / (p.Hkv * n_slots);  // slowest: neighbouring blocks share a key chunk (L2 reuse)
+  if (p.plan[2] == 0) return;  // the plan kernel saw no sequence with more than 16 rows per KV head
   const int n_live = p.num_seqs[0];
   if (n_live <= 0) return;
   // sequence i starts at slot floor(qsl[i]*G/ROWS) + i; find the last sequence starting at or before `slot`
@@ -59,16 +63,15 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
   const int R0 = tile_in_seq * ROWS;
   if (tile_in_seq < 0 || R0 >= rows_total) return;
 
-  // ---- key range of the workgroup ----------------------------------------------------------------
-  const int last_row = min(R0 + ROWS, rows_total) - 1;
+  // ---- key range of the workgroup: one chunk of the row tile's range ----------------------------
+  const PrefillTile pt = prefill_tile(p, sp, R0);
+  if (chunk >= pt.n_chunks) return;  // also: queries before position 0 have no keys; such rows stay unwritten
   const int base_pos = sp.ctx - sp.q_len;  // position of the sequence's first query token
-  const int kv_hi = min(sp.ctx, base_pos + last_row / G + 1);
-  int kv_lo = 0;
-  if (p.window > 0) kv_lo = max(base_pos + R0 / G - p.window + 1, 0);
-  const int vis_lo = kv_lo;
-  kv_lo &= ~(TT - 1);
+  const int vis_lo = pt.vis_lo;
+  const int kv_lo = pt.kv_lo + chunk * p.pre_chunk;
+  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : kv_lo + p.pre_chunk;
   const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
-  if (n_tiles <= 0) return;  // only when the queries sit before position 0; such rows stay unwritten
+  const bool single = pt.n_chunks == 1;
 
   // ---- per row-block lane state --------------------------------------------------------------------
   int row_lo[RB], row_hi[RB];
@@ -298,13 +301,24 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 16);
     l_tot += __shfl_xor(l_tot, 32);
     if (row_ok[rb]) {
-      const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
-      uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
+      if (single) {
+        const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
+        uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
 #pragma unroll
-      for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
-        const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
-                         pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
-        *(u32x2*)(orow + 16 * rt) = w;
+        for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
+          const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                           pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+          *(u32x2*)(orow + 16 * rt) = w;
+        }
+      } else {
+        const int64_t pslot = ((int64_t)chunk * p.T + out_tok[rb]) * p.Hq + out_head[rb];
+        float* prow = p.pre_o + pslot * D + 4 * g4;
+#pragma unroll
+        for (int rt = 0; rt < DPL; ++rt) *(f32x4*)(prow + 16 * rt) = o_acc[rb][rt] * v_unit;
+        if (g4 == 0) {
+          p.pre_ml[pslot * 2 + 0] = m_run[rb];
+          p.pre_ml[pslot * 2 + 1] = l_tot;
+        }
       }
     }
   }
@@ -314,7 +328,7 @@ template <int D, int KVT, int TT, int NW, int RB>
 static int launch_one(hipStream_t stream, const AttnParams& p) {
   constexpr int ROWS = NW * RB * 16;
   const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
-  const int64_t blocks = slots * p.Hkv;
+  const int64_t blocks = slots * p.Hkv * p.pre_max_chunks;
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
   if (p.softcap > 0.f)
     hipLaunchKernelGGL((attn_prefill_kernel<D, KVT, TT, NW, RB, true>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);

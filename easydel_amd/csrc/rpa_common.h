@@ -12,6 +12,8 @@ constexpr int kRowBlock = 16;      // MFMA M/N extent: rows (token, group-head p
 constexpr int kMaxSplitsCap = 256;   // hard upper bound on split-K partials per sequence
 constexpr int kPlanHeader = 16;      // ints before the prefix array in the decode plan
 constexpr int kMaxDecodeWgs = 4096;  // persistent decode workgroups per KV-head group
+constexpr int kPrefillRows = 128;    // query rows (token x group head) one prefill workgroup owns
+constexpr int kMaxPrefillChunks = 8; // key chunks one prefill row tile may be split into
 
 // Everything a kernel needs, passed by value.
 struct AttnParams {
@@ -25,7 +27,10 @@ struct AttnParams {
   void* out;
   float* part_o;   // [max_splits][Tdec][Hq][D]   Tdec = t_dec_max: decode-class query tokens, compacted
   float* part_ml;  // [max_splits][Tdec][Hq][2]   (running max in log2 units, running sum)
-  int32_t* plan;   // decode plan: [0] = W (flattened keys), [1] = Q (keys per workgroup), then at kPlanHeader:
+  float* pre_o;    // prefill split-K partials [pre_max_chunks][T][Hq][D]
+  float* pre_ml;   // [pre_max_chunks][T][Hq][2]
+  int32_t* plan;   // decode plan: [0] = W (flattened keys), [1] = Q (keys per workgroup), [2] = 1 if any sequence needs
+                   // the large-row kernel, then at kPlanHeader:
                    // P[S+1] exclusive prefix of per-sequence key spans, R[S+1] exclusive prefix of
                    // decode-class query tokens (row of a token in the partial buffers), first_seq[n_wg]
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
@@ -40,6 +45,9 @@ struct AttnParams {
   int t_dec_max;     // static bound on decode-class query tokens = rows of one partial slot
   int n_wg;          // persistent decode workgroups per KV-head group
   int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
+  int pre_chunk;     // keys per prefill split-K chunk (multiple of 64)
+  int pre_max_chunks;  // chunks the prefill partial buffers hold; 1 = never split
+  int decode_sync;   // decode workgroups re-align their waves with a barrier every this many tiles (power of two), 0 = never
   int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel
   int decode_wpb;    // waves (KV heads) per decode workgroup, 0 = default
   int decode_occ;    // waves per SIMD the decode kernel is compiled for, 0 = compiler's choice
@@ -71,6 +79,24 @@ __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
   }
   s.small_rows = (s.q_len * p.group <= kRowBlock);
   return s;
+}
+
+// Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + kPrefillRows) of a sequence) must visit, kv_lo
+// rounded down to 64, and the number of split-K chunks the prefill kernel cuts it into.
+struct PrefillTile {
+  int kv_lo, kv_hi, vis_lo, n_chunks;
+};
+__device__ __forceinline__ PrefillTile prefill_tile(const AttnParams& p, const SeqPlan& sp, int R0) {
+  PrefillTile t;
+  const int rows_total = sp.q_len * p.group;
+  const int last_row = min(R0 + kPrefillRows, rows_total) - 1;
+  const int base_pos = sp.ctx - sp.q_len;
+  t.kv_hi = min(sp.ctx, base_pos + last_row / p.group + 1);
+  t.vis_lo = (p.window > 0) ? max(base_pos + R0 / p.group - p.window + 1, 0) : 0;
+  t.kv_lo = t.vis_lo & ~63;
+  const int span = t.kv_hi - t.kv_lo;
+  t.n_chunks = span <= 0 ? 0 : min((span + p.pre_chunk - 1) / p.pre_chunk, p.pre_max_chunks);
+  return t;
 }
 
 // Partial slots the decode kernel filled for sequence i (0 or 1: the output row is already final).

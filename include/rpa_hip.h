@@ -150,6 +150,9 @@ int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t
  *   "max_splits"     partial-output slots per sequence the decode kernel may use (2..256, 0 = sized
  *                    from the shapes); set it before sizing the workspace
  *   "decode_wgs"     persistent decode workgroups per KV-head group (0 = as many as are resident at once)
+ *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
+ *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
+ *                    set it before sizing the workspace
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
  *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
  *                    1 = decode plan kernel, 2 = decode kernel, 4 = prefill / large-row kernel,
