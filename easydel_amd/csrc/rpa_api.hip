@@ -61,7 +61,7 @@ int static_splits(int T, int M, int page_size, int Hq, int D) {
 }
 
 // Prefill split-K: keys per chunk and number of chunks the partial buffers hold, from the static bounds.
-// A row tile's key range is cut into at most kMaxPrefillChunks chunks of at least 2048 keys; the partial
+// A row tile's key range is cut into at most kMaxPrefillChunks chunks of at least 8192 keys; the partial
 // buffers ([chunks][T][Hq][D+2] floats) are kept under ~1 GiB by allowing fewer, longer chunks.
 void prefill_split(int T, int M, int page_size, int Hq, int D, int* chunk_keys, int* max_chunks) {
   const long span = (long)M * page_size;
@@ -70,7 +70,7 @@ void prefill_split(int T, int M, int page_size, int Hq, int D, int* chunk_keys, 
   const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   long keys = (span + chunks - 1) / chunks;
-  if (keys < 2048) keys = 2048;
+  if (keys < 8192) keys = 8192;
   keys = (keys + 63) & ~63L;
   chunks = (int)((span + keys - 1) / keys);
   if (chunks < 1) chunks = 1;

@@ -211,3 +211,70 @@ def test_chunked_prefill_equals_rows_of_single_shot_prefill(gpu):
     chunk = tl.run_gpu_attention(b_chunk)
     assert np.abs(chunk - full[256:]).max() <= 2e-2
     tl.assert_close(chunk, tl.oracle_out(b_chunk), b_chunk, "chunk")
+
+
+def test_single_long_sequence_spreads_over_many_workgroups(gpu):
+    # one decode row over 70k keys: the key stream is cut into hundreds of pieces and merged in several rounds
+    from easydel_amd import _lib
+
+    b = tl.make_batch(70, [70_001], [1], Hq=32, Hkv=8, D=128, page_size=64)
+    _check(b, "single long sequence")
+    prev = _lib.set_tunable("max_splits", 256)
+    try:
+        _check(b, "single long sequence, 256 slots")
+    finally:
+        _lib.set_tunable("max_splits", prev)
+
+
+def test_many_short_sequences(gpu):
+    rng = np.random.default_rng(71)
+    ctx = rng.integers(1, 200, size=1500).tolist()
+    b = tl.make_batch(71, ctx, [1] * len(ctx), Hq=8, Hkv=2, D=64, page_size=16, pad_rows=48)
+    _check(b, "1500 short sequences")
+
+
+def test_hip_graph_replay_matches_eager(gpu):
+    # the C ABI neither allocates nor synchronises, so a whole layer call can be captured and replayed
+    import torch
+    from easydel_amd import kernels
+
+    b = tl.make_batch(72, [700, 65, 1500, 300, 2000], [1, 1, 2, 40, 1], Hq=32, Hkv=8, D=128, page_size=64, pad_rows=2)
+    d = tl.device_batch(b, gpu)
+    rng = np.random.default_rng(3)
+    key = tl.to_torch(tl.orc.f32_to_bf16_bits(rng.standard_normal((b.T, 8, 128), dtype=np.float32)), BF16, gpu)
+    val = tl.to_torch(tl.orc.f32_to_bf16_bits(rng.standard_normal((b.T, 8, 128), dtype=np.float32)), BF16, gpu)
+    dist = torch.tensor([3, 5, 5], dtype=torch.int32, device=gpu)
+    out = torch.empty_like(d["query"])
+
+    def call():
+        kernels.ragged_paged_attention_v3(d["query"], key, val, d["kv_pages"], d["context_lens"], d["block_tables"].reshape(-1),
+                                          d["query_start_loc"], dist, out=out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()  # warm-up on the capture stream: sizes the cached workspace outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call()
+    for rep in range(4):
+        out.zero_()
+        d["query"].mul_(1.0)  # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
+    # new metadata in the same buffers is picked up by the next replay (nothing is baked in on the host)
+    d["context_lens"][0] = 650
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    b.context_lens[0] = 650
+    pages_after = tl.orc.page_scatter_ragged_ref(key.view(torch.int16).cpu().numpy().view(np.uint16), val.view(torch.int16).cpu().numpy().view(np.uint16),
+                                                 d["kv_pages"].view(torch.int16).cpu().numpy().view(np.uint16), b.context_lens,
+                                                 b.block_tables, b.query_start_loc, b.num_seqs)
+    want = tl.oracle_out(b, kv_val=tl.orc.bf16_bits_to_f32(pages_after).astype(np.float64))
+    tl.assert_close(tl.from_torch(out, BF16), want, b, "graph replay with new metadata")
