@@ -528,6 +528,7 @@ bool decode_supported(const AttnParams& p) {
   if (p.D != 64 && p.D != 128 && p.D != 256) return false;
   if (p.page_size % 16 != 0) return false;
   if (p.kv_dtype != RPA_BF16 && p.kv_scales == nullptr) return false;
+  if (!(p.scale > 0.f)) return false;  // the MFMA kernels take the running max before scaling
   return true;
 }
 

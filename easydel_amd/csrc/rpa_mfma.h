@@ -60,8 +60,20 @@ __device__ __forceinline__ int swz_key(int tok) {
   else return 0;
 }
 
-__device__ __forceinline__ float xor16_max(float v) { return fmaxf(v, __shfl_xor(v, 16)); }
-__device__ __forceinline__ float xor32_max(float v) { return fmaxf(v, __shfl_xor(v, 32)); }
+// Maximum over the lanes l, l^16 (xor16_max) or l, l^32 (xor32_max), through the gfx950 row-swap instructions:
+// v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second,
+// v_permlane32_swap the upper half of the first with the lower half of the second.  Fed two copies of v, the
+// results are (own-or-partner, partner-or-own) in every lane.  Pure VALU: no LDS round trip as with ds_bpermute.
+__device__ __forceinline__ float xor16_max(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_max(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
 
 // tanh through the hardware exp2: tanh(x) = 1 - 2 / (exp(2x) + 1).  Good to ~1e-6 relative, far inside
 // the bf16 tolerance of the MFMA kernels (the fp32 kernel uses tanhf).
@@ -72,9 +84,10 @@ __device__ __forceinline__ float fast_tanh(float x) {
 
 
 // Online-softmax step of one 16-row block over NS 16-key sub-tiles held as S^T accumulators (lane = query row
-// n, 4 keys 4*g4 + j per sub-tile).  Scales the raw scores (soft cap first if CAP), masks keys outside
-// [row_lo, row_hi) if MASK, updates the running max / sum, and leaves the probabilities as packed bf16 B
-// operands.  Returns the factor the output accumulators must be multiplied by (exp2 of the max change).
+// n, 4 keys 4*g4 + j per sub-tile).  Applies the soft cap if CAP, masks keys outside [row_lo, row_hi) if MASK,
+// updates the running max / sum, and leaves the probabilities as packed bf16 B operands.  The maximum is taken
+// over the raw scores and scaled once (sc_mul > 0, so scaling commutes with max); each probability is then one
+// fused multiply-add and one exp2.  Returns the factor the output accumulators must be multiplied by.
 template <bool MASK, bool CAP, int NS>
 __device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, float cap_in, int tb, int g4,
                                               int row_lo, int row_hi, float& m_run, float& l_run,
@@ -86,7 +99,6 @@ __device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, 
     for (int j = 0; j < 4; ++j) {
       float s = s_acc[st][j];
       if constexpr (CAP) s = fast_tanh(s * cap_in);
-      s *= sc_mul;
       if constexpr (MASK) {
         const int tok = tb + st * 16 + 4 * g4 + j;
         s = (tok >= row_lo && tok < row_hi) ? s : -INFINITY;
@@ -95,7 +107,7 @@ __device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, 
       mx = fmaxf(mx, s);
     }
   }
-  mx = xor32_max(xor16_max(mx));
+  mx = xor32_max(xor16_max(mx)) * sc_mul;
   const float m_new = fmaxf(m_run, mx);
   const float m_use = (MASK && m_new == -INFINITY) ? 0.f : m_new;
   const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
@@ -106,7 +118,7 @@ __device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, 
     float pr[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      pr[j] = __builtin_amdgcn_exp2f(s_acc[st][j] - m_use);
+      pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[st][j], sc_mul, -m_use));
       psum += pr[j];
     }
     pfrag[st][0] = pack_bf16(pr[0], pr[1]);
