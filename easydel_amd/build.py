@@ -24,6 +24,7 @@ SOURCES = [
     "rpa_attn_generic.hip",
     "rpa_attn_decode.hip",
     "rpa_attn_prefill.hip",
+    "rpa_attn_prefill_dma.hip",
     "rpa_attn_merge.hip",
 ]
 

@@ -25,6 +25,7 @@ std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are 
 std::atomic<int> g_force_generic{0};
 std::atomic<int> g_decode_wpb{0};
 std::atomic<int> g_decode_occ{0};
+std::atomic<int> g_prefill_dma{1};
 std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
 
 int fail(int code, const char* fmt, ...) {
@@ -113,6 +114,7 @@ int rpa_set_tunable(const char* name, int value) {
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
   if (!strcmp(name, "decode_wpb")) return g_decode_wpb.exchange(value);
   if (!strcmp(name, "decode_occ")) return g_decode_occ.exchange(value);
+  if (!strcmp(name, "prefill_dma")) return g_prefill_dma.exchange(value != 0);
   if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
   return -1;
 }
@@ -207,6 +209,7 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   p.decode_sync = g_decode_sync.load();
   p.decode_wpb = g_decode_wpb.load();
   p.decode_occ = g_decode_occ.load();
+  p.prefill_dma = g_prefill_dma.load();
   p.max_splits = 2;
   p.pre_chunk = 1 << 30;
   p.pre_max_chunks = 1;

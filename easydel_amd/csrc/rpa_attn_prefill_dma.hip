@@ -1,0 +1,354 @@
+// MFMA prefill / chunked-prefill attention for bf16 pages, K/V tiles moved global -> LDS by the
+// load unit itself (global_load_lds_dwordx4), three tiles deep.
+//
+// Same work split and arithmetic as attn_prefill_kernel (rpa_attn_prefill.hip): a workgroup owns 128
+// query rows of one (sequence, KV head), each wave keeps RB 16-row blocks in registers and every wave
+// reads the shared K/V tile in MFMA operand order.  What differs is how a tile reaches LDS.  There the
+// tile passes through registers (load, wait, ds_write), which costs staging registers, address and
+// write instructions, and leaves one tile of prefetch.  Here every lane hands the load unit one 16-byte
+// global address and the unit writes the 64 lanes' chunks to 1 KiB of LDS in lane order; the XOR swizzle
+// of the tile is applied on the global side (lane for LDS chunk c' of row r fetches global chunk
+// c' ^ key(r)).  No registers are held while a tile is in flight, so tiles t+1 and t+2 are on their way
+// while tile t is computed, and the compute loop holds no global-memory instructions of its own.
+//
+// The loads are issued through inline assembly: the compiler then neither tracks them nor orders its
+// own waits around them, and the kernel states its waits itself (s_waitcnt vmcnt(n) + s_barrier before a
+// tile is read).  Every other global access of the kernel (queries before the loop, results after it)
+// is ordinary code; the compiler's waits for those can only be stricter than needed, never weaker,
+// because the counter retires loads in order.
+#include "rpa_mfma.h"
+
+namespace rpa {
+
+// One LDS DMA of 1 KiB: every lane fetches 16 bytes from base + voff; lane L's bytes land at LDS byte
+// address lds_addr + 16 L.  (An instruction offset would move the LDS address as well, so none is used.)
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
+// Waits until at most N of this wave's loads are in flight, then joins the workgroup barrier.
+template <int N>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int D, int NW, int RB, bool CAP>
+__global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams p) {
+  constexpr int TT = 32;                 // keys per tile
+  constexpr int RKL = D * 2;             // bytes of one K (or V) row
+  constexpr int HBG = 2 * RKL;           // K_h | V_h span of one token in global memory
+  constexpr int CPR = RKL / 16;          // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;          // rows one DMA instruction covers
+  constexpr int NLH = TT / (RPI * NW);   // DMA instructions per wave per tile, for K and again for V
+  static_assert(TT % (RPI * NW) == 0 && NLH >= 1, "the waves' DMA instructions tile the 32 rows exactly");
+  static_assert(NLH == 1 || (RPI * NW) % 16 == 0, "a lane's swizzle key must not depend on the instruction");
+  constexpr int NS = TT / 16;            // 16-key sub-tiles per tile
+  constexpr int DPL = D / 16;            // 16-dim row tiles of O^T
+  constexpr int NKK = D / 32;            // k-steps of the score MFMA
+  constexpr int ROWS = NW * RB * 16;
+  static_assert(ROWS == kPrefillRows, "merge kernel assumes this row-tile height");
+  constexpr int TILE_BYTES = TT * 2 * RKL;
+  constexpr int NBUF = 3;
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[NBUF * TILE_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g4 = lane >> 4;
+  const int G = p.group;
+
+  // ---- block -> (sequence, row tile, KV head, key chunk) ---------------------------------------------
+  const int h = blockIdx.x % p.Hkv;
+  const int n_slots = gridDim.x / (p.Hkv * p.pre_max_chunks);
+  const int slot = (blockIdx.x / p.Hkv) % n_slots;
+  const int chunk = blockIdx.x / (p.Hkv * n_slots);  // slowest: neighbouring blocks share a key chunk (L2 reuse)
+  if (p.plan[2] == 0) return;  // the plan kernel saw no sequence with more than 16 rows per KV head
+  const int n_live = p.num_seqs[0];
+  if (n_live <= 0) return;
+  // sequence i starts at slot floor(qsl[i]*G/ROWS) + i; find the last sequence starting at or before `slot`
+  int lo_i = 0, hi_i = n_live;
+  while (hi_i - lo_i > 1) {
+    const int mid = (lo_i + hi_i) >> 1;
+    if ((int)(((int64_t)p.qsl[mid] * G) / ROWS) + mid <= slot) lo_i = mid; else hi_i = mid;
+  }
+  const int i = lo_i;
+  const SeqPlan sp = seq_plan(p, i);
+  if (!sp.live || sp.small_rows) return;
+  const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * G) / ROWS) + i);
+  const int rows_total = sp.q_len * G;
+  const int R0 = tile_in_seq * ROWS;
+  if (tile_in_seq < 0 || R0 >= rows_total) return;
+
+  // ---- key range of the workgroup: one chunk of the row tile's range ----------------------------
+  const PrefillTile pt = prefill_tile(p, sp, R0);
+  if (chunk >= pt.n_chunks) return;  // also: queries before position 0 have no keys; such rows stay unwritten
+  const int base_pos = sp.ctx - sp.q_len;  // position of the sequence's first query token
+  const int vis_lo = pt.vis_lo;
+  // the first tile must hold vis_lo, so that rows of it that nobody may see can borrow a visible row's address
+  const int kv_lo = max(pt.kv_lo + chunk * p.pre_chunk, vis_lo & ~(TT - 1));
+  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : pt.kv_lo + (chunk + 1) * p.pre_chunk;
+  const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
+  const bool single = pt.n_chunks == 1;
+
+  // ---- per row-block lane state --------------------------------------------------------------------
+  int row_lo[RB], row_hi[RB];
+  bool row_ok[RB];
+  int out_tok[RB], out_head[RB];
+  bf16x8 qf[RB][NKK];
+  int wave_lo, wave_hi;          // keys every row of the wave sees: [max row_lo, min row_hi)
+  int wave_lo_min, wave_hi_max;  // keys some row of the wave sees: [min row_lo, max row_hi)
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = R0 + (wave * RB + rb) * 16 + n;
+    row_ok[rb] = row < rows_total;
+    const int r_tok = row_ok[rb] ? row / G : (rows_total - 1) / G;  // padded rows shadow the last row
+    const int r_head = row_ok[rb] ? row - r_tok * G : 0;
+    const int pos = base_pos + r_tok;
+    row_hi[rb] = min(pos + 1, sp.ctx);
+    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+    out_tok[rb] = sp.q0 + r_tok;
+    out_head[rb] = h * G + r_head;
+    const char* qrow = (const char*)p.q + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D * 2;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok[rb]) v = *(const u32x4*)(qrow + (kk * 32 + 8 * g4) * 2);
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  // Use the query registers once here, so that the compiler waits for these loads now and not at their first use
+  // inside the loop, where its wait would also cover every tile in flight.
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = __builtin_bit_cast(u32x4, qf[rb][kk]);
+      asm volatile("" : "+v"(v));
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  {
+    int lo_max = 0, hi_min = 0x7fffffff, lo_min = 0x7fffffff, hi_max = 0;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      lo_max = max(lo_max, row_lo[rb]);
+      hi_min = min(hi_min, row_hi[rb]);
+      lo_min = min(lo_min, row_lo[rb]);
+      hi_max = max(hi_max, row_hi[rb]);
+    }
+#pragma unroll
+    for (int o = 1; o < 16; o <<= 1) {
+      lo_max = max(lo_max, __shfl_xor(lo_max, o));
+      hi_min = min(hi_min, __shfl_xor(hi_min, o));
+      lo_min = min(lo_min, __shfl_xor(lo_min, o));
+      hi_max = max(hi_max, __shfl_xor(hi_max, o));
+    }
+    wave_lo = __builtin_amdgcn_readfirstlane(lo_max);
+    wave_hi = __builtin_amdgcn_readfirstlane(hi_min);
+    wave_lo_min = __builtin_amdgcn_readfirstlane(lo_min);
+    wave_hi_max = __builtin_amdgcn_readfirstlane(hi_max);
+  }
+  // a wave whose row blocks all lie past the sequence's rows only helps with the loads
+  const bool wave_active = (R0 + wave * RB * 16) < rows_total;
+
+  // ---- tile loads ------------------------------------------------------------------------------------
+  // DMA instruction u of wave w fills LDS rows (u NW + w) RPI .. + RPI - 1 of the K half, and again of the V
+  // half; lane L sits at row + L / CPR, LDS chunk L % CPR, and fetches the global chunk that the swizzle maps there.
+  // The block table is read through the constant address space: it does not change while the kernel runs, and
+  // only so may the compiler keep these loads scalar after the assembly statements above have "written memory".
+  typedef const __attribute__((address_space(4))) int32_t* ConstI32;
+  ConstI32 bt = (ConstI32)(uintptr_t)(p.block_tables + (int64_t)i * p.M);
+  const char* pages = (const char*)p.kv_pages;
+  const int pg = p.page_size;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
+  const int dma_row = wave * RPI + lane / CPR;          // row for u = 0; instruction u adds u * NW * RPI
+  const int dma_chunk = (lane % CPR) ^ swz_key<RKL>(dma_row);
+  const uint32_t dma_wave_lds = (uint32_t)wave * 1024u;
+  // issue cursor: the next tile to load (block-table column, token offset inside that page, page id)
+  int cur_idx = kv_lo / pg;
+  int cur_off = kv_lo - cur_idx * pg;
+  int cur_tb = kv_lo;
+  int cur_buf = 0;
+  auto load_page = [&](int idx) -> int {
+    int pgid = bt[min(idx, p.M - 1)];
+    pgid = __builtin_amdgcn_readfirstlane(pgid);
+    return min(max(pgid, 0), p.P - 1);
+  };
+  int cur_page = load_page(cur_idx);
+  auto issue = [&]() {  // starts the DMA of the cursor's tile into LDS buffer cur_buf and advances the cursor
+    const char* base = pages + (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride + (int64_t)h * HBG;
+    const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
+    const uint32_t buf_lds = lds_base + (uint32_t)cur_buf * TILE_BYTES + dma_wave_lds;
+#pragma unroll
+    for (int u = 0; u < NLH; ++u) {
+      int r = dma_row + u * NW * RPI;
+      if (edge) r = min(max(cur_tb + r, vis_lo), sp.ctx - 1) - cur_tb;  // keys nobody may see: any visible row's bytes
+      const uint32_t voff = (uint32_t)r * (uint32_t)p.token_stride + (uint32_t)(dma_chunk << 4);
+      dma16(buf_lds + u * NW * 1024, voff, base);                      // K rows
+      dma16(buf_lds + TT * RKL + u * NW * 1024, voff, base + RKL);     // V rows
+    }
+    cur_tb += TT;
+    cur_off += TT;
+    if (cur_off >= pg) {
+      cur_off -= pg;
+      ++cur_idx;
+    }
+    cur_buf = (cur_buf == NBUF - 1) ? 0 : cur_buf + 1;
+    cur_page = load_page(cur_idx);  // consumed by the next issue, a whole tile later
+  };
+
+  const float cap_out = p.softcap * 1.4426950408889634f;
+  const float cap_in = CAP ? p.scale / p.softcap : 0.f;
+
+  float m_run[RB], l_run[RB];
+  f32x4 o_acc[RB][DPL];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    m_run[rb] = -INFINITY;
+    l_run[rb] = 0.f;
+#pragma unroll
+    for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  issue();                   // tile 0
+  if (n_tiles > 1) issue();  // tile 1
+
+  int rd_buf = 0;
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    const int tb = kv_lo + tile * TT;
+    // Tile `tile` has landed once at most the loads of tile + 1 are still in flight.  The barrier also tells that
+    // every wave has finished the previous step, whose LDS buffer the next issue overwrites.
+    if (tile + 1 < n_tiles) wait_loads_and_barrier<2 * NLH>();
+    else wait_loads_and_barrier<0>();
+    if (tile + 2 < n_tiles) issue();
+
+    const unsigned char* lds_k = lds_all + rd_buf * TILE_BYTES;
+    const unsigned char* lds_v = lds_k + TT * RKL;
+    rd_buf = (rd_buf == NBUF - 1) ? 0 : rd_buf + 1;
+
+    if (wave_active && tb < wave_hi_max && tb + TT > wave_lo_min) {
+      // ---- S^T = K . Q^T for every row block (K operands shared) --------------------------------
+      f32x4 s_acc[RB][NS];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int st = 0; st < NS; ++st) s_acc[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int st = 0; st < NS; ++st) {
+        const int tk = st * 16 + n;
+        const unsigned char* krow = lds_k + tk * RKL;
+        const int key = swz_key<RKL>(tk);
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) {
+          const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
+        }
+      }
+
+      // ---- online softmax per row block -------------------------------------------------------------
+      const bool inside = (tb >= wave_lo) && (tb + TT <= wave_hi);  // no row of the wave masks any key here
+      const float sc_mul = CAP ? cap_out : p.scale_log2;
+      uint32_t pfrag[RB][NS][2];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        float alpha;
+        if (inside) alpha = softmax_step<false, CAP, NS>(s_acc[rb], sc_mul, cap_in, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+        else alpha = softmax_step<true, CAP, NS>(s_acc[rb], sc_mul, cap_in, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+        if (__any(alpha != 1.f)) {
+#pragma unroll
+          for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] *= alpha;
+        }
+      }
+
+      // ---- O^T += V^T . P^T (V operands shared by the row blocks) -----------------------------------
+      // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16
+      // (key 4g4 + l/4, dims d0 + 4(l%4)..) and receives the transposed column: for dim d0 + (l&15) the
+      // values of keys 4g4..4g4+3, which is the A operand of the product with k = keys.
+      const int tr_key = 4 * g4 + (n >> 2);          // key (within a 16-key sub-tile) this lane addresses
+      const int tr_byte = (n & 3) * 8;               // byte offset of its 4 dims inside the 32-byte row-tile span
+#pragma unroll
+      for (int rt = 0; rt < DPL; ++rt) {
+        u32x2 a_lo, a_hi;
+        {
+          const int tk = tr_key;
+          const int off = rt * 32 + tr_byte;
+          const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+          a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
+        }
+        {
+          const int tk = 16 + tr_key;
+          const int off = rt * 32 + tr_byte;
+          const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+          a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
+        }
+        const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
+          o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
+                                                                  o_acc[rb][rt], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue -----------------------------------------------------------------------------------------
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    if (row_ok[rb]) {
+      if (single) {
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
+#pragma unroll
+        for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
+          const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                           pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+          *(u32x2*)(orow + 16 * rt) = w;
+        }
+      } else {
+        const int64_t pslot = ((int64_t)chunk * p.T + out_tok[rb]) * p.Hq + out_head[rb];
+        float* prow = p.pre_o + pslot * D + 4 * g4;
+#pragma unroll
+        for (int rt = 0; rt < DPL; ++rt) *(f32x4*)(prow + 16 * rt) = o_acc[rb][rt];
+        if (g4 == 0) {
+          p.pre_ml[pslot * 2 + 0] = m_run[rb];
+          p.pre_ml[pslot * 2 + 1] = l_tot;
+        }
+      }
+    }
+  }
+}
+
+template <int D, int NW, int RB>
+static int launch_dma(hipStream_t stream, const AttnParams& p) {
+  constexpr int ROWS = NW * RB * 16;
+  const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
+  const int64_t blocks = slots * p.Hkv * p.pre_max_chunks;
+  if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
+  if (p.softcap > 0.f)
+    hipLaunchKernelGGL((attn_prefill_dma_kernel<D, NW, RB, true>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  else
+    hipLaunchKernelGGL((attn_prefill_dma_kernel<D, NW, RB, false>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+// bf16 pages whose size is a multiple of the 32-key tile, and page rows that a 32-bit byte offset can address
+bool prefill_dma_supported(const AttnParams& p) {
+  return p.kv_dtype == RPA_BF16 && p.page_size % 32 == 0 && (p.D == 64 || p.D == 128 || p.D == 256) &&
+         (int64_t)32 * p.token_stride < ((int64_t)1 << 31);
+}
+
+int launch_attn_prefill_dma(hipStream_t stream, const AttnParams& p) {
+  switch (p.D) {
+    case 64: return launch_dma<64, 4, 2>(stream, p);
+    case 128: return launch_dma<128, 4, 2>(stream, p);
+    case 256: return launch_dma<256, 8, 1>(stream, p);
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
+}  // namespace rpa

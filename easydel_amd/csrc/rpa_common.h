@@ -51,6 +51,7 @@ struct AttnParams {
   int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel
   int decode_wpb;    // waves (KV heads) per decode workgroup, 0 = default
   int decode_occ;    // waves per SIMD the decode kernel is compiled for, 0 = compiler's choice
+  int prefill_dma;   // 1: bf16 prefill tiles go global -> LDS directly where that kernel applies; 0: always through registers
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
 };
 
@@ -151,8 +152,10 @@ __device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
 int launch_attn_generic(hipStream_t stream, const AttnParams& p);
 int launch_attn_decode(hipStream_t stream, const AttnParams& p, int which = 3);  // bit 0: plan kernel, bit 1: decode kernel
 int launch_attn_prefill(hipStream_t stream, const AttnParams& p);
+int launch_attn_prefill_dma(hipStream_t stream, const AttnParams& p);  // bf16 pages, tiles loaded straight into LDS
 int launch_attn_merge(hipStream_t stream, const AttnParams& p);
 bool decode_supported(const AttnParams& p);
 bool prefill_supported(const AttnParams& p);
+bool prefill_dma_supported(const AttnParams& p);
 
 }  // namespace rpa

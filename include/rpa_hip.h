@@ -153,6 +153,8 @@ int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t
  *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
  *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
  *                    set it before sizing the workspace
+ *   "prefill_dma"    1 (default): bf16 prefill tiles are loaded global -> LDS by the load unit where that kernel
+ *                    applies (page_size % 32 == 0); 0: every prefill tile is staged through registers
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
  *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
  *                    1 = decode plan kernel, 2 = decode kernel, 4 = prefill / large-row kernel,

@@ -201,6 +201,52 @@ def test_prefill_window_with_null_pages(gpu):
     tl.assert_close(got, want, b, "prefill window + null pages")
 
 
+def test_prefill_window_with_null_pages_smaller_than_the_alignment(gpu):
+    # 32-token pages: the 64-aligned start of the key range can fall on a page that lies wholly left of the window
+    W, pg = 200, 32
+    ctx = [1500, 900, 333]
+    q_lens = [100, 64, 40]
+    b = tl.make_batch(54, ctx, q_lens, Hq=16, Hkv=4, D=128, page_size=pg, max_pages=48)
+    want = tl.oracle_out(b, sliding_window=W)
+    for i, (c, ql) in enumerate(zip(ctx, q_lens)):
+        first_needed = max(c - ql - W + 1, 0) // pg
+        b.block_tables[i, :first_needed] = 0
+    b.kv_raw[0] = 0x7FC0
+    got = tl.run_gpu_attention(b, sliding_window=W)
+    tl.assert_close(got, want, b, "prefill window + 32-token null pages")
+
+
+@pytest.mark.parametrize("D,page_size", [(128, 64), (256, 128), (64, 32)])
+def test_prefill_ignores_cache_slots_past_the_context(gpu, D, page_size):
+    # slots of the last page beyond ctx hold NaN: they must never reach the accumulators, not even times zero
+    ctx = [300, 1000, 129, 47, 2100]
+    q_lens = [300, 200, 129, 33, 17]
+    b = tl.make_batch(55, ctx, q_lens, Hq=16, Hkv=4, D=D, page_size=page_size)
+    want = tl.oracle_out(b)
+    for i, c in enumerate(ctx):
+        if c % page_size:
+            b.kv_raw[b.block_tables[i, c // page_size], c % page_size:] = 0x7FC0
+    got = tl.run_gpu_attention(b)
+    tl.assert_close(got, want, b, f"prefill with NaN past ctx D{D}")
+
+
+@pytest.mark.parametrize("D,page_size,Hq,Hkv", [(128, 64, 32, 8), (256, 128, 16, 8), (64, 32, 8, 2)])
+def test_prefill_register_staged_kernel_serves_bf16_too(gpu, D, page_size, Hq, Hkv):
+    # bf16 pages normally take the kernel that loads tiles straight into LDS; the other one must agree
+    from easydel_amd import _lib
+
+    ctx = [300, 1000, 129, 47, 2100, 700]
+    q_lens = [300, 200, 129, 33, 17, 1]
+    b = tl.make_batch(56 + D, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, pad_rows=2, pad_tokens=5)
+    direct = _check(b, f"prefill D{D}, tiles loaded into LDS directly", sliding_window=700)
+    prev = _lib.set_tunable("prefill_dma", 0)
+    try:
+        staged = _check(b, f"prefill D{D}, tiles staged through registers", sliding_window=700)
+    finally:
+        _lib.set_tunable("prefill_dma", prev)
+    assert np.abs(direct[tl.valid_rows(b)] - staged[tl.valid_rows(b)]).max() <= 2e-2
+
+
 def test_chunked_prefill_equals_rows_of_single_shot_prefill(gpu):
     # the same keys, queried as one 384-token prefill and as its last 128-token chunk
     b_full = tl.make_batch(53, [384], [384], Hq=32, Hkv=8, D=128, page_size=64)
