@@ -16,6 +16,8 @@
 // tile is read).  Every other global access of the kernel (queries before the loop, results after it)
 // is ordinary code; the compiler's waits for those can only be stricter than needed, never weaker,
 // because the counter retires loads in order.
+#include <type_traits>
+
 #include "rpa_mfma.h"
 
 namespace rpa {
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   constexpr int ROWS = NW * RB * 16;
   static_assert(ROWS == kPrefillRows, "merge kernel assumes this row-tile height");
   constexpr int TILE_BYTES = TT * 2 * RKL;
-  constexpr int NBUF = 3;
+  constexpr int NBUF = 4;
 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_all[NBUF * TILE_BYTES];
 
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     return min(max(pgid, 0), p.P - 1);
   };
   int cur_page = load_page(cur_idx);
-  auto issue = [&]() {  // starts the DMA of the cursor's tile into LDS buffer cur_buf and advances the cursor
+  auto issue = [&]() __attribute__((always_inline)) {  // starts the DMA of the cursor's tile into LDS buffer cur_buf and advances the cursor
     const char* base = pages + (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride + (int64_t)h * HBG;
     const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
     const uint32_t buf_lds = lds_base + (uint32_t)cur_buf * TILE_BYTES + dma_wave_lds;
@@ -193,7 +195,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       cur_off -= pg;
       ++cur_idx;
     }
-    cur_buf = (cur_buf == NBUF - 1) ? 0 : cur_buf + 1;
+    cur_buf = (cur_buf + 1) & (NBUF - 1);
     cur_page = load_page(cur_idx);  // consumed by the next issue, a whole tile later
   };
 
@@ -210,89 +212,132 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  issue();                   // tile 0
-  if (n_tiles > 1) issue();  // tile 1
-
-  int rd_buf = 0;
-  for (int tile = 0; tile < n_tiles; ++tile) {
-    const int tb = kv_lo + tile * TT;
-    // Tile `tile` has landed once at most the loads of tile + 1 are still in flight.  The barrier also tells that
-    // every wave has finished the previous step, whose LDS buffer the next issue overwrites.
-    if (tile + 1 < n_tiles) wait_loads_and_barrier<2 * NLH>();
-    else wait_loads_and_barrier<0>();
-    if (tile + 2 < n_tiles) issue();
-
-    const unsigned char* lds_k = lds_all + rd_buf * TILE_BYTES;
-    const unsigned char* lds_v = lds_k + TT * RKL;
-    rd_buf = (rd_buf == NBUF - 1) ? 0 : rd_buf + 1;
-
-    if (wave_active && tb < wave_hi_max && tb + TT > wave_lo_min) {
-      // ---- S^T = K . Q^T for every row block (K operands shared) --------------------------------
-      f32x4 s_acc[RB][NS];
+  // ---- S^T = K . Q^T for every row block (K operands shared) ------------------------------------------
+  auto qk = [&](const unsigned char* lds_k, f32x4 (&sa)[RB][NS]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int st = 0; st < NS; ++st) sa[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+      const int tk = st * 16 + n;
+      const unsigned char* krow = lds_k + tk * RKL;
+      const int key = swz_key<RKL>(tk);
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+          sa[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], sa[rb][st], 0, 0, 0);
+      }
+    }
+  };
+  // ---- online softmax of the scores of tile tb, then O^T += V^T . P^T ---------------------------------
+  auto soft_pv = [&](auto mask_tag, f32x4 (&sa)[RB][NS], int tb, const unsigned char* lds_v) __attribute__((always_inline)) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+    const float sc_mul = CAP ? cap_out : p.scale_log2;
+    uint32_t pfrag[RB][NS][2];
+    float alpha[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+      alpha[rb] = softmax_step<MASK, CAP, NS>(sa[rb], sc_mul, cap_in, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+    // Pin the probabilities here: otherwise the compiler sinks their exponentials below the branch that follows,
+    // out of the stretch where they overlap with the score MFMAs of the next tile.
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int st = 0; st < NS; ++st) asm volatile("" : "+v"(pfrag[rb][st][0]), "+v"(pfrag[rb][st][1]));
+    bool changed = false;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) changed |= (alpha[rb] != 1.f);
+    if (__any(changed)) {
+      // In place, through assembly: left to the compiler, the two arms of this branch meet in a second copy of the
+      // accumulators, which costs their registers again and a move of each on every tile.
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int st = 0; st < NS; ++st) s_acc[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int rt = 0; rt < DPL; ++rt)
 #pragma unroll
-      for (int st = 0; st < NS; ++st) {
-        const int tk = st * 16 + n;
-        const unsigned char* krow = lds_k + tk * RKL;
-        const int key = swz_key<RKL>(tk);
+          for (int j = 0; j < 4; ++j) asm("v_mul_f32 %0, %1, %0" : "+v"(o_acc[rb][rt][j]) : "v"(alpha[rb]));
+    }
+    // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16
+    // (key 4g4 + l/4, dims d0 + 4(l%4)..) and receives the transposed column: for dim d0 + (l&15) the
+    // values of keys 4g4..4g4+3, which is the A operand of the product with k = keys.
+    const int tr_key = 4 * g4 + (n >> 2);          // key (within a 16-key sub-tile) this lane addresses
+    const int tr_byte = (n & 3) * 8;               // byte offset of its 4 dims inside the 32-byte row-tile span
+    __builtin_amdgcn_sched_barrier(0);  // keep the V operand reads out of the softmax: they would only pile up in registers
 #pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) {
-          const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb)
-            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
-        }
+    for (int rt = 0; rt < DPL; ++rt) {
+      if (rt > 0 && rt % 4 == 0) __builtin_amdgcn_sched_barrier(0);
+      u32x2 a_lo, a_hi;
+      {
+        const int tk = tr_key;
+        const int off = rt * 32 + tr_byte;
+        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+        a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
       }
-
-      // ---- online softmax per row block -------------------------------------------------------------
-      const bool inside = (tb >= wave_lo) && (tb + TT <= wave_hi);  // no row of the wave masks any key here
-      const float sc_mul = CAP ? cap_out : p.scale_log2;
-      uint32_t pfrag[RB][NS][2];
+      {
+        const int tk = 16 + tr_key;
+        const int off = rt * 32 + tr_byte;
+        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+        a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
+      }
+      const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        float alpha;
-        if (inside) alpha = softmax_step<false, CAP, NS>(s_acc[rb], sc_mul, cap_in, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
-        else alpha = softmax_step<true, CAP, NS>(s_acc[rb], sc_mul, cap_in, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-          for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] *= alpha;
-        }
-      }
-
-      // ---- O^T += V^T . P^T (V operands shared by the row blocks) -----------------------------------
-      // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16
-      // (key 4g4 + l/4, dims d0 + 4(l%4)..) and receives the transposed column: for dim d0 + (l&15) the
-      // values of keys 4g4..4g4+3, which is the A operand of the product with k = keys.
-      const int tr_key = 4 * g4 + (n >> 2);          // key (within a 16-key sub-tile) this lane addresses
-      const int tr_byte = (n & 3) * 8;               // byte offset of its 4 dims inside the 32-byte row-tile span
-#pragma unroll
-      for (int rt = 0; rt < DPL; ++rt) {
-        u32x2 a_lo, a_hi;
-        {
-          const int tk = tr_key;
-          const int off = rt * 32 + tr_byte;
-          const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
-          a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
-        }
-        {
-          const int tk = 16 + tr_key;
-          const int off = rt * 32 + tr_byte;
-          const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
-          a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
-        }
-        const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-          const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
-          o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
-                                                                  o_acc[rb][rt], 0, 0, 0);
-        }
+        const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
+        o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
+                                                                o_acc[rb][rt], 0, 0, 0);
       }
     }
-  }
+  };
+  auto needs_mask = [&](int tb) { return !((tb >= wave_lo) && (tb + TT <= wave_hi)); };
+  auto buf_k = [&](int t) -> const unsigned char* { return lds_all + (t & (NBUF - 1)) * TILE_BYTES; };
+  auto buf_v = [&](int t) -> const unsigned char* { return lds_all + (t & (NBUF - 1)) * TILE_BYTES + TT * RKL; };
+
+  // ---- pipeline ----------------------------------------------------------------------------------------
+  // Step t: the matrix cores compute the scores of tile t+1 while the vector ALU does the softmax of tile t,
+  // then the PV product of tile t runs.  Four LDS buffers: during step t tiles t (V) and t+1 (K) are read and
+  // tiles t+2 and t+3 are in flight; tile t+3 goes where tile t-1 lay, whose last reader finished before the
+  // barrier that opens step t.
+  issue();                   // tile 0
+  if (n_tiles > 1) issue();  // tile 1
+  if (n_tiles > 2) issue();  // tile 2
+  if (n_tiles > 2) wait_loads_and_barrier<4 * NLH>();
+  else if (n_tiles > 1) wait_loads_and_barrier<2 * NLH>();
+  else wait_loads_and_barrier<0>();
+  // (A wave whose rows all lie past the sequence's end computes like the others, on zero queries: its rows are
+  // never stored, and the loop stays free of a branch around every step.)
+  f32x4 s_cur[RB][NS];
+  qk(buf_k(0), s_cur);
+  int t = 0;
+  // Steps [t, t_end) with or without the masking code.  Two variants side by side in one loop body (an if / else
+  // around the step) make the compiler keep a second copy of every accumulator, so the choice is made per run of
+  // steps instead: masked steps at the window's lower edge, unmasked ones, masked ones at the causal edge.
+  auto run = [&](auto mask_tag, int t_end) __attribute__((always_inline)) {
+    for (; t < t_end; ++t) {
+      const int tb = kv_lo + t * TT;
+      if (t + 2 < n_tiles) wait_loads_and_barrier<2 * NLH>();  // tile t+1 has landed; tile t+2 may still be in flight
+      else wait_loads_and_barrier<0>();
+      if (t + 3 < n_tiles) issue();
+      f32x4 s_nxt[RB][NS];
+      qk(buf_k(t + 1), s_nxt);
+      soft_pv(mask_tag, s_cur, tb, buf_v(t));
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int st = 0; st < NS; ++st) s_cur[rb][st] = s_nxt[rb][st];
+    }
+  };
+  const int t_plain_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT);  // first tile no row of the wave masks from below
+  const int t_plain_hi = (wave_hi - kv_lo) / TT;                   // first tile some row of the wave masks from above
+  run(std::true_type{}, min(t_plain_lo, n_tiles - 1));
+  run(std::false_type{}, min(t_plain_hi, n_tiles - 1));
+  run(std::true_type{}, n_tiles - 1);
+  soft_pv(std::true_type{}, s_cur, kv_lo + t * TT, buf_v(t));  // last tile: nothing left to overlap with
+  (void)needs_mask;
+  (void)wave_active;
+  (void)wave_lo_min; (void)wave_hi_max;
 
   // ---- epilogue -----------------------------------------------------------------------------------------
 #pragma unroll
