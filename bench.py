@@ -35,7 +35,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill"])
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
@@ -62,6 +62,8 @@ def build_workload(name, seed, sequential=False):
         return workloads.config4_quantised_decode(seed, "fp8")
     if name == "c4-int8":
         return workloads.config4_quantised_decode(seed, "int8")
+    if name == "llama-prefill":  # tuning shape for the prefill kernel, not one of the benchmark configurations
+        return workloads.llama_long_prefill(seed)
     return workloads.config5_gemma_long_prefill(seed, windowed=(name == "c5-window"))
 
 

@@ -165,29 +165,44 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
   const int dma_row = wave * RPI + lane / CPR;          // row for u = 0; instruction u adds u * NW * RPI
   const int dma_chunk = (lane % CPR) ^ swz_key<RKL>(dma_row);
+  const int dma_chunk_v = (lane % CPR) ^ swz_key_v<RKL>(dma_row);  // the V half is swizzled for its transposing reads
   const uint32_t dma_wave_lds = (uint32_t)wave * 1024u;
   // issue cursor: the next tile to load (block-table column, token offset inside that page, page id)
   int cur_idx = kv_lo / pg;
   int cur_off = kv_lo - cur_idx * pg;
   int cur_tb = kv_lo;
   int cur_buf = 0;
-  auto load_page = [&](int idx) -> int {
-    int pgid = bt[min(idx, p.M - 1)];
-    pgid = __builtin_amdgcn_readfirstlane(pgid);
-    return min(max(pgid, 0), p.P - 1);
-  };
-  int cur_page = load_page(cur_idx);
+  // Lane offsets of an ordinary tile, loop-invariant; only a tile that holds keys nobody may see recomputes them.
+  uint32_t voff_k[NLH], voff_v[NLH];
+#pragma unroll
+  for (int u = 0; u < NLH; ++u) {
+    const uint32_t roff = (uint32_t)(dma_row + u * NW * RPI) * (uint32_t)p.token_stride;
+    voff_k[u] = roff + (uint32_t)(dma_chunk << 4);
+    voff_v[u] = roff + (uint32_t)(dma_chunk_v << 4);
+  }
+  // The page id of the cursor's tile is fetched one issue ahead and only clamped when it is used, so that no issue
+  // waits for the scalar load it has just made.
+  auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
+  int cur_page_raw = load_page(cur_idx);
   auto issue = [&]() __attribute__((always_inline)) {  // starts the DMA of the cursor's tile into LDS buffer cur_buf and advances the cursor
+    const int cur_page = min(max(cur_page_raw, 0), p.P - 1);
     const char* base = pages + (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride + (int64_t)h * HBG;
     const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
     const uint32_t buf_lds = lds_base + (uint32_t)cur_buf * TILE_BYTES + dma_wave_lds;
+    if (!edge) {
 #pragma unroll
-    for (int u = 0; u < NLH; ++u) {
-      int r = dma_row + u * NW * RPI;
-      if (edge) r = min(max(cur_tb + r, vis_lo), sp.ctx - 1) - cur_tb;  // keys nobody may see: any visible row's bytes
-      const uint32_t voff = (uint32_t)r * (uint32_t)p.token_stride + (uint32_t)(dma_chunk << 4);
-      dma16(buf_lds + u * NW * 1024, voff, base);                      // K rows
-      dma16(buf_lds + TT * RKL + u * NW * 1024, voff, base + RKL);     // V rows
+      for (int u = 0; u < NLH; ++u) {
+        dma16(buf_lds + u * NW * 1024, voff_k[u], base);                  // K rows
+        dma16(buf_lds + TT * RKL + u * NW * 1024, voff_v[u], base + RKL); // V rows
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < NLH; ++u) {  // keys nobody may see: any visible row's bytes
+        const int r = min(max(cur_tb + dma_row + u * NW * RPI, vis_lo), sp.ctx - 1) - cur_tb;
+        const uint32_t roff = (uint32_t)r * (uint32_t)p.token_stride;
+        dma16(buf_lds + u * NW * 1024, roff + (uint32_t)(dma_chunk << 4), base);
+        dma16(buf_lds + TT * RKL + u * NW * 1024, roff + (uint32_t)(dma_chunk_v << 4), base + RKL);
+      }
     }
     cur_tb += TT;
     cur_off += TT;
@@ -196,18 +211,19 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       ++cur_idx;
     }
     cur_buf = (cur_buf + 1) & (NBUF - 1);
-    cur_page = load_page(cur_idx);  // consumed by the next issue, a whole tile later
+    cur_page_raw = load_page(cur_idx);
   };
 
   const float cap_out = p.softcap * 1.4426950408889634f;
   const float cap_in = CAP ? p.scale / p.softcap : 0.f;
 
-  float m_run[RB], l_run[RB];
+  float m_run[RB];
+  f32x4 l_acc[RB];  // row sums, replicated over the four elements (see soft_pv)
   f32x4 o_acc[RB][DPL];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     m_run[rb] = -INFINITY;
-    l_run[rb] = 0.f;
+    l_acc[rb] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
@@ -237,28 +253,74 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     constexpr bool MASK = decltype(mask_tag)::value;
     const float sc_mul = CAP ? cap_out : p.scale_log2;
     uint32_t pfrag[RB][NS][2];
-    float alpha[RB];
+    // Soft cap and mask in place; each lane's maximum over its own 8 keys of the row.
+    float lmx[RB];
+    bool grow = false;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
-      alpha[rb] = softmax_step<MASK, CAP, NS>(sa[rb], sc_mul, cap_in, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
-    // Pin the probabilities here: otherwise the compiler sinks their exponentials below the branch that follows,
-    // out of the stretch where they overlap with the score MFMAs of the next tile.
+    for (int rb = 0; rb < RB; ++rb) {
+      lmx[rb] = -INFINITY;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb)
+      for (int st = 0; st < NS; ++st)
 #pragma unroll
-      for (int st = 0; st < NS; ++st) asm volatile("" : "+v"(pfrag[rb][st][0]), "+v"(pfrag[rb][st][1]));
-    bool changed = false;
+        for (int j = 0; j < 4; ++j) {
+          float sv = sa[rb][st][j];
+          if constexpr (CAP) sv = fast_tanh(sv * cap_in);
+          if constexpr (MASK) {
+            const int tok = tb + st * 16 + 4 * g4 + j;
+            sv = (tok >= row_lo[rb] && tok < row_hi[rb]) ? sv : -INFINITY;
+          }
+          sa[rb][st][j] = sv;
+          lmx[rb] = fmaxf(lmx[rb], sv);
+        }
+      lmx[rb] *= sc_mul;  // sc_mul > 0: scaling commutes with the maximum
+      grow |= lmx[rb] > m_run[rb];
+    }
+    // The running maximum is the reference every probability of a row is taken against.  Only when some key of
+    // the tile exceeds it (rare once a few tiles are behind) is it raised: the lanes of a row then agree on the new
+    // maximum and everything accumulated so far is scaled down.  Otherwise the tile costs neither the lane
+    // exchange nor a rescale.
+    if (__any(grow)) {
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) changed |= (alpha[rb] != 1.f);
-    if (__any(changed)) {
-      // In place, through assembly: left to the compiler, the two arms of this branch meet in a second copy of the
-      // accumulators, which costs their registers again and a move of each on every tile.
+      for (int rb = 0; rb < RB; ++rb) {
+        const float m_new = fmaxf(m_run[rb], xor32_max(xor16_max(lmx[rb])));
+        const float m_use = (MASK && m_new == -INFINITY) ? 0.f : m_new;
+        float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_use);
+        m_run[rb] = m_new;
+        // The multiplications below are opaque to the compiler, so it does not pad the distance this chip wants
+        // between a transcendental instruction and a reader of its result; the padding is put here by hand.
+        asm volatile("s_nop 1" : "+v"(alpha));
+        // In place, through assembly: left to the compiler, the two arms of this branch meet in a second copy of the
+        // accumulators, which costs their registers again and a move of each on every tile.
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+        for (int j = 0; j < 4; ++j) asm("v_mul_f32 %0, %1, %0" : "+v"(l_acc[rb][j]) : "v"(alpha));
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) asm("v_mul_f32 %0, %1, %0" : "+v"(o_acc[rb][rt][j]) : "v"(alpha[rb]));
+          for (int j = 0; j < 4; ++j) asm("v_mul_f32 %0, %1, %0" : "+v"(o_acc[rb][rt][j]) : "v"(alpha));
+      }
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      const float m_use = (MASK && m_run[rb] == -INFINITY) ? 0.f : m_run[rb];
+#pragma unroll
+      for (int st = 0; st < NS; ++st) {
+        float pr[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[rb][st][j], sc_mul, -m_use));
+        pfrag[rb][st][0] = pack_bf16(pr[0], pr[1]);
+        pfrag[rb][st][1] = pack_bf16(pr[2], pr[3]);
+      }
+    }
+    // The row sums come from the matrix cores as well: a V^T tile of ones times P^T leaves, in every accumulator
+    // element of column n, the sum of row n's probabilities over all 32 keys (as rounded to bf16, i.e. exactly the
+    // weights the PV product uses).  Two MFMAs replace 16 additions per lane and the cross-lane sum at the end.
+    {
+      const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
+        l_acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones), __builtin_bit_cast(bf16x8, b4), l_acc[rb], 0, 0, 0);
+      }
     }
     // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16
     // (key 4g4 + l/4, dims d0 + 4(l%4)..) and receives the transposed column: for dim d0 + (l&15) the
@@ -273,13 +335,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       {
         const int tk = tr_key;
         const int off = rt * 32 + tr_byte;
-        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key_v<RKL>(tk)) << 4) + (off & 15);
         a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
       }
       {
         const int tk = 16 + tr_key;
         const int off = rt * 32 + tr_byte;
-        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key<RKL>(tk)) << 4) + (off & 15);
+        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key_v<RKL>(tk)) << 4) + (off & 15);
         a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
       }
       const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
@@ -308,25 +370,28 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   else wait_loads_and_barrier<0>();
   // (A wave whose rows all lie past the sequence's end computes like the others, on zero queries: its rows are
   // never stored, and the loop stays free of a branch around every step.)
-  f32x4 s_cur[RB][NS];
+  f32x4 s_cur[RB][NS], s_alt[RB][NS];
   qk(buf_k(0), s_cur);
   int t = 0;
+  auto step = [&](auto mask_tag, f32x4 (&s_in)[RB][NS], f32x4 (&s_out)[RB][NS], int ts) __attribute__((always_inline)) {
+    if (ts + 2 < n_tiles) wait_loads_and_barrier<2 * NLH>();  // tile ts+1 has landed; tile ts+2 may still be in flight
+    else wait_loads_and_barrier<0>();
+    if (ts + 3 < n_tiles) issue();
+    qk(buf_k(ts + 1), s_out);
+    soft_pv(mask_tag, s_in, kv_lo + ts * TT, buf_v(ts));
+  };
   // Steps [t, t_end) with or without the masking code.  Two variants side by side in one loop body (an if / else
   // around the step) make the compiler keep a second copy of every accumulator, so the choice is made per run of
   // steps instead: masked steps at the window's lower edge, unmasked ones, masked ones at the causal edge.
+  // (Unrolling two steps per trip to alternate the score registers instead of copying them was tried: the
+  // compiler then needs 50 more registers and spills.)
   auto run = [&](auto mask_tag, int t_end) __attribute__((always_inline)) {
     for (; t < t_end; ++t) {
-      const int tb = kv_lo + t * TT;
-      if (t + 2 < n_tiles) wait_loads_and_barrier<2 * NLH>();  // tile t+1 has landed; tile t+2 may still be in flight
-      else wait_loads_and_barrier<0>();
-      if (t + 3 < n_tiles) issue();
-      f32x4 s_nxt[RB][NS];
-      qk(buf_k(t + 1), s_nxt);
-      soft_pv(mask_tag, s_cur, tb, buf_v(t));
+      step(mask_tag, s_cur, s_alt, t);
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int st = 0; st < NS; ++st) s_cur[rb][st] = s_nxt[rb][st];
+        for (int st = 0; st < NS; ++st) s_cur[rb][st] = s_alt[rb][st];
     }
   };
   const int t_plain_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT);  // first tile no row of the wave masks from below
@@ -342,8 +407,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   // ---- epilogue -----------------------------------------------------------------------------------------
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 16);
-    l_tot += __shfl_xor(l_tot, 32);
+    const float l_tot = l_acc[rb][0];
     if (row_ok[rb]) {
       if (single) {
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;

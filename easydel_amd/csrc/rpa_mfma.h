@@ -64,6 +64,17 @@ __device__ __forceinline__ int swz_key(int tok) {
 // v_permlane16_swap exchanges the odd 16-lane rows of its first operand with the even rows of its second,
 // v_permlane32_swap the upper half of the first with the lower half of the second.  Fed two copies of v, the
 // results are (own-or-partner, partner-or-own) in every lane.  Pure VALU: no LDS round trip as with ds_bpermute.
+// Swizzle of the V half of a tile, which is read with transposing loads: 16 lanes fetch 32 contiguous bytes of
+// each of 4 consecutive token rows.  With swz_key those four rows share two 32-byte bank groups (a 2-way
+// conflict on every read); XOR-ing the chunk index with twice the row number spreads them over four.
+template <int ROW_BYTES>
+__device__ __forceinline__ int swz_key_v(int tok) {
+  constexpr int NCH = ROW_BYTES / 16;
+  if constexpr (NCH >= 16) return (tok & 7) << 1;
+  else if constexpr (NCH == 8) return (tok & 3) << 1;
+  else return 0;
+}
+
 __device__ __forceinline__ float xor16_max(float v) {
   const uint32_t u = __float_as_uint(v);
   const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);

@@ -165,6 +165,17 @@ def config5_gemma_long_prefill(seed: int = 0, windowed: bool = False, num_pages:
                     softmax_scale=1.0 / 16.0, sliding_window=4096 if windowed else None, logits_soft_cap=50.0)
 
 
+def llama_long_prefill(seed: int = 0, n_seqs: int = 8, q_len: int = 2048, num_pages: int = 6000) -> Workload:
+    """Not one of the five benchmark shapes: a prefill batch large enough to fill the chip at head size 128 (the
+    mixed shape C3 holds only 4 x 512 prefill tokens), used to tune and profile the prefill kernel."""
+    rng = np.random.default_rng(seed)
+    prior = rng.integers(8192, 32769, size=n_seqs)
+    ctx = (prior + q_len).astype(np.int32)
+    return Workload("Llama-3-8B-shaped long-context chunked prefill (tuning shape)", Hq=32, Hkv=8, D=128, page_size=64,
+                    num_pages=num_pages, max_pages_per_seq=576, context_lens=ctx, q_lens=np.full(n_seqs, q_len, dtype=np.int32),
+                    block_tables=_tables(rng, ctx, 64, num_pages, 576), softmax_scale=128.0 ** -0.5)
+
+
 # ---- device side ---------------------------------------------------------------------------------
 
 
