@@ -36,6 +36,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill"])
+    ap.add_argument("--layout", default="interleaved", choices=["interleaved", "unified"],
+                    help="interleaved: one pool [P, page, 2*Hkv, D], scatter fused with the attention call (v3); "
+                         "unified: separate K and V pools [P, page, Hkv, D], two slice scatters then the attention call")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
@@ -163,8 +166,31 @@ def main():
     quant = w.kv_dtype in ("fp8", "int8")
     out = torch.empty_like(tens["query"])
 
+    unified = args.layout == "unified"
+    if unified:
+        from easydel_amd.caching import compute_slot_mapping_v2
+
+        key_cache = tens["kv_pages"][:, :, 0::2].contiguous()
+        value_cache = tens["kv_pages"][:, :, 1::2].contiguous()
+        tens["kv_pages"] = None  # the interleaved pool is not used again: give its memory back
+        torch.cuda.empty_cache()
+        slots_np, n_slices = compute_slot_mapping_v2(num_requests=w.S, scheduled=w.q_lens, num_computed_tokens=w.context_lens - w.q_lens,
+                                                     page_table=w.block_tables, page_size=w.page_size)
+        slots = torch.from_numpy(slots_np).to(dev)
+        n_slices_dev = torch.tensor([n_slices], dtype=torch.int32, device=dev)
+        k_flat, v_flat = key_cache.view(-1, w.Hkv, w.D), value_cache.view(-1, w.Hkv, w.D)
+        args.no_cpu_baseline = True  # the host sample is cut from the interleaved pool
+
     def step():
-        if quant:  # quantised pages are read-only for this path
+        if unified:
+            if not quant:
+                kernels.page_scatter_slices(tens["key"], slots, n_slices_dev, k_flat, page_size=w.page_size)
+                kernels.page_scatter_slices(tens["value"], slots, n_slices_dev, v_flat, page_size=w.page_size)
+            kernels.unified_attention(tens["query"], key_cache, value_cache, tens["context_lens"], tens["block_tables"],
+                                      tens["query_start_loc"], tens["num_seqs"], softmax_scale=w.softmax_scale,
+                                      sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap,
+                                      kv_scales=tens["kv_scales"], out=out)
+        elif quant:  # quantised pages are read-only for this path
             kernels.ragged_paged_attention(tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"],
                                            tens["query_start_loc"], tens["num_seqs"], softmax_scale=w.softmax_scale,
                                            sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap,
@@ -197,10 +223,16 @@ def main():
     # kernel (it reuses the plan left in the workspace) or only the prefill kernel, bracketed by events on the
     # launch stream
     stream = torch.cuda.current_stream(dev)
-    att = lambda: kernels.ragged_paged_attention(  # noqa: E731
-        tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
-        tens["num_seqs"], softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
-        logits_soft_cap=w.logits_soft_cap, kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv, out=out)
+    if unified:
+        att = lambda: kernels.unified_attention(  # noqa: E731
+            tens["query"], key_cache, value_cache, tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
+            tens["num_seqs"], softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
+            logits_soft_cap=w.logits_soft_cap, kv_scales=tens["kv_scales"], out=out)
+    else:
+        att = lambda: kernels.ragged_paged_attention(  # noqa: E731
+            tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"], tens["query_start_loc"],
+            tens["num_seqs"], softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
+            logits_soft_cap=w.logits_soft_cap, kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv, out=out)
 
     def time_stage(mask, reps):
         _lib.set_tunable("stages", mask)
@@ -253,6 +285,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": w.name,
+            "kv_layout": args.layout,
             "sequences": w.S,
             "query_tokens": w.T,
             "q_heads": w.Hq,

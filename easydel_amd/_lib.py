@@ -30,6 +30,10 @@ SIGNATURES = {
         _c_int,
         [_c_vp] * 10 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32],
     ),
+    "rpa_unified_attention": (
+        _c_int,
+        [_c_vp] * 11 + [_c_sz] + [_c_int] * 10 + [_c_f32, _c_int, _c_f32],
+    ),
     "rpa_ragged_paged_attention_v3": (
         _c_int,
         [_c_vp] * 11 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32],

@@ -169,36 +169,39 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
   return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256;
 }
 
-int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages, const float* kv_scales,
-                               const int32_t* context_lens, const int32_t* block_tables,
-                               const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
-                               size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv,
-                               int D, int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
-                               float logits_soft_cap) {
+// Shared body of the attention entry points.  k_pages / v_pages and the strides describe where K and V of
+// (page, token, KV head) lie (sizes are validated here, so the callers' stride arithmetic may see nonsense and
+// must not act on it); C is the row length of kv_scales; num_seqs may be null (every row live) if the caller allows.
+static int attention_impl(const char* who, rpa_stream_t stream, const void* q, const void* k_pages, const void* v_pages,
+                          int64_t token_stride, int64_t head_stride, const float* kv_scales,
+                          const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
+                          const int32_t* num_seqs, bool num_seqs_optional, void* out, void* workspace,
+                          size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
+                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap) {
   if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0)
-    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: bad size (T=%d S=%d M=%d P=%d page_size=%d Hq=%d Hkv=%d D=%d)",
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (T=%d S=%d M=%d P=%d page_size=%d Hq=%d Hkv=%d D=%d)", who,
                 T, S, M, P, page_size, Hq, Hkv, D);
-  if (Hq % Hkv != 0) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
-  if (C < 2 * Hkv) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: C=%d combined heads < 2*Hkv=%d", C, 2 * Hkv);
-  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: q_dtype %d (want f32 or bf16)", q_dtype);
-  if (kv_dtype < RPA_F32 || kv_dtype > RPA_INT8) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: kv_dtype %d", kv_dtype);
-  if (D > 256 || D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention: head_dim %d (want a multiple of 4, <= 256)", D);
+  if (Hq % Hkv != 0) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
+  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16) return fail(RPA_ERR_UNSUPPORTED, "%s: q_dtype %d (want f32 or bf16)", who, q_dtype);
+  if (kv_dtype < RPA_F32 || kv_dtype > RPA_INT8) return fail(RPA_ERR_UNSUPPORTED, "%s: kv_dtype %d", who, kv_dtype);
+  if (D > 256 || D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "%s: head_dim %d (want a multiple of 4, <= 256)", who, D);
   if ((kv_dtype == RPA_FP8_E4M3 || kv_dtype == RPA_INT8) && !kv_scales)
-    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: 8-bit KV pages need kv_scales");
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: 8-bit KV pages need kv_scales", who);
   if (kv_scales && ((uintptr_t)kv_scales & 7))
-    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: kv_scales must be 8-byte aligned");
-  if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: softmax_scale is not finite");
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: kv_scales must be 8-byte aligned", who);
+  if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_scale is not finite", who);
   if (T == 0) return RPA_OK;
-  if (!q || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs || !out)
-    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: null pointer");
+  if (!q || !k_pages || !v_pages || !context_lens || !block_tables || !query_start_loc || (!num_seqs && !num_seqs_optional) || !out)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
 
   rpa::AttnParams p;
   memset(&p, 0, sizeof(p));
-  p.q = q; p.kv_pages = kv_pages; p.kv_scales = kv_scales;
+  p.q = q; p.k_pages = k_pages; p.v_pages = v_pages; p.kv_scales = kv_scales;
   p.context_lens = context_lens; p.block_tables = block_tables; p.qsl = query_start_loc; p.num_seqs = num_seqs;
   p.out = out;
   p.T = T; p.S = S; p.M = M; p.P = P; p.page_size = page_size; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv; p.D = D; p.C = C;
-  p.token_stride = (int64_t)C * D * rpa::elem_bytes(kv_dtype);
+  p.token_stride = token_stride;
+  p.head_stride = head_stride;
   p.page_stride = p.token_stride * page_size;
   p.q_dtype = q_dtype; p.kv_dtype = kv_dtype;
   p.scale = softmax_scale;
@@ -228,7 +231,7 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
     size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (pre_po + pre_pml) : 0;
     size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
     if (!workspace || usable < 2 * (po + pml))
-      return fail(RPA_ERR_WORKSPACE, "rpa_ragged_paged_attention: workspace %zu bytes < %zu needed for two partial slots",
+      return fail(RPA_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu needed for two partial slots", who,
                   workspace_bytes, 2 * (po + pml) + pb + 256);
     if (usable < pre + 2 * (po + pml)) {  // a small workspace: prefill rows are not split over keys
       pre = 0;
@@ -258,6 +261,34 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   }
   if (!(stages & 8)) return RPA_OK;
   return hip_fail(rpa::launch_attn_merge(s, p), "merge kernel launch");
+}
+
+int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages, const float* kv_scales,
+                               const int32_t* context_lens, const int32_t* block_tables,
+                               const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
+                               size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv,
+                               int D, int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
+                               float logits_soft_cap) {
+  if (Hkv > 0 && C < 2 * Hkv)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: C=%d combined heads < 2*Hkv=%d", C, 2 * Hkv);
+  // interleaved pages: K of head h in combined head 2h, V in 2h+1, one row of D elements each
+  const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
+  const void* v_pages = kv_pages ? (const char*)kv_pages + row : nullptr;
+  return attention_impl("rpa_ragged_paged_attention", stream, q, kv_pages, v_pages, (int64_t)C * row, 2 * row, kv_scales,
+                        context_lens, block_tables, query_start_loc, num_seqs, false, out, workspace, workspace_bytes, T, S,
+                        M, P, page_size, Hq, Hkv, D, C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+}
+
+int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_cache, const void* value_cache,
+                          const float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
+                          const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
+                          size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D,
+                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap) {
+  // separate pools [P][page_size][Hkv][D]: heads one row apart, tokens Hkv rows apart
+  const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
+  return attention_impl("rpa_unified_attention", stream, q, key_cache, value_cache, (int64_t)Hkv * row, row, kv_scales,
+                        context_lens, block_tables, query_start_loc, num_seqs, true, out, workspace, workspace_bytes, T, S, M,
+                        P, page_size, Hq, Hkv, D, 2 * Hkv, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
 }
 
 int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void* key, const void* value,

@@ -102,8 +102,9 @@ __global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p
   const int c32 = lane % LPT;
   const bool is_v = c32 >= NCH;
   const int cc = is_v ? c32 - NCH : c32;
-  const char* pages = (const char*)p.kv_pages;
-  const int64_t lane_goff = (int64_t)h * HB + c32 * 16 + (int64_t)sub * p.token_stride;
+  // a lane fetches either K or V chunks, always: its pool and its offset inside a token row are fixed
+  const char* pages = (const char*)(is_v ? p.v_pages : p.k_pages);
+  const int64_t lane_goff = (int64_t)h * p.head_stride + cc * 16 + (int64_t)sub * p.token_stride;
 
   u32x4 stage[DEPTH][NLD];
   u32x2 sc_stage[DEPTH];  // (K scale, V scale) of the staged tile's page: fetched with the tile, in order behind it

@@ -24,7 +24,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
   constexpr int kMaxD = 256;
   __shared__ float q_s[kMaxD];
   const int t = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
-  const int n_live = p.num_seqs[0];
+  const int n_live = live_rows(p);
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) return;
   const int i = find_seq(p.qsl, n_live, t);
   const SeqPlan sp = seq_plan(p, i);
@@ -43,10 +43,11 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
   __syncthreads();
 
   constexpr int eb = ElemBytes<KVT>::v;
-  const char* pages = (const char*)p.kv_pages;
+  const char* k_pages = (const char*)p.k_pages;
+  const char* v_pages = (const char*)p.v_pages;
   const int32_t* bt = p.block_tables + (int64_t)i * p.M;
-  const int64_t k_head_off = (int64_t)(2 * h) * D * eb;
-  const int64_t v_head_off = (int64_t)(2 * h + 1) * D * eb;
+  const int64_t head_off = (int64_t)h * p.head_stride;
+  (void)eb;
 
   float m = -INFINITY, l = 0.f;
   float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -55,11 +56,11 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
     const int j = base + lane;
     float s = -INFINITY;
     float v_scale = 1.f;
-    const char* row = nullptr;
+    int64_t row = 0;  // byte offset of the key's (token, KV head) row inside the K pool; V has the same in its pool
     if (j < k_hi) {
       const int page = min(max(bt[j / p.page_size], 0), p.P - 1);
-      row = pages + (int64_t)page * p.page_stride + (int64_t)(j % p.page_size) * p.token_stride;
-      const void* kp = row + k_head_off;
+      row = (int64_t)page * p.page_stride + (int64_t)(j % p.page_size) * p.token_stride + head_off;
+      const void* kp = k_pages + row;
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(q_s[d], load_elem<KVT>(kp, d), dot);
       if (p.kv_scales) {
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
     const int n_keys = min(64, k_hi - base);
     for (int jj = 0; jj < n_keys; ++jj) {
       const float w = __shfl(pv, jj);
-      const char* vrow = (const char*)__shfl((unsigned long long)row, jj) + v_head_off;
+      const char* vrow = v_pages + (int64_t)__shfl((unsigned long long)row, jj);
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const int d = lane + 64 * k;

@@ -15,7 +15,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);  // (token, head) index
   if (pair >= p.T * p.Hq) return;
   const int t = pair / p.Hq, hq = pair - t * p.Hq;
-  const int n_live = p.num_seqs[0];
+  const int n_live = live_rows(p);
   const int D = p.D;
   bool zero = false;
   int n_pieces = 0, part_row = 0;

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
   const int slot = (blockIdx.x / p.Hkv) % n_slots;
   const int chunk = blockIdx.x / (p.Hkv * n_slots);  // slowest: neighbouring blocks share a key chunk (L2 reuse)
   if (p.plan[2] == 0) return;  // the plan kernel saw no sequence with more than 16 rows per KV head
-  const int n_live = p.num_seqs[0];
+  const int n_live = live_rows(p);
   if (n_live <= 0) return;
   // sequence i starts at slot floor(qsl[i]*G/ROWS) + i; find the last sequence starting at or before `slot`
   int lo_i = 0, hi_i = n_live;
@@ -125,7 +125,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
 
   // ---- staging ---------------------------------------------------------------------------------------
   const int32_t* bt = p.block_tables + (int64_t)i * p.M;
-  const char* pages = (const char*)p.kv_pages;
+  const char* k_pages = (const char*)p.k_pages;
+  const char* v_pages = (const char*)p.v_pages;
   const int pg = p.page_size;
   int st_tok[NLD], st_cc[NLD];
   bool st_v[NLD], st_ok[NLD];
@@ -138,7 +139,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     const int c = idx % LPTG;
     st_v[u] = c >= LPTG / 2;
     st_cc[u] = st_v[u] ? c - LPTG / 2 : c;
-    st_off[u] = (int64_t)st_tok[u] * p.token_stride + (int64_t)h * HBG + c * 16;
+    st_off[u] = (int64_t)st_tok[u] * p.token_stride + (int64_t)h * p.head_stride + st_cc[u] * 16;
   }
   u32x4 stage[NLD];
   auto page_of = [&](int tok) -> int {
@@ -147,10 +148,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     return min(max(pgid, 0), p.P - 1);
   };
   auto issue = [&](int tb, int page) {
-    const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride;
+    const int64_t base = (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride;
 #pragma unroll
     for (int u = 0; u < NLD; ++u)
-      if (FULL || st_ok[u]) stage[u] = *(const u32x4*)(base + st_off[u]);
+      if (FULL || st_ok[u]) stage[u] = *(const u32x4*)((st_v[u] ? v_pages : k_pages) + base + st_off[u]);
   };
   auto commit = [&](int tb, unsigned char* buf) {  // registers -> LDS tile (zeroing keys nobody may see)
     const bool edge = (tb + TT > sp.ctx) || (tb < vis_lo);

@@ -38,7 +38,6 @@ template <int D, int NW, int RB, bool CAP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams p) {
   constexpr int TT = 32;                 // keys per tile
   constexpr int RKL = D * 2;             // bytes of one K (or V) row
-  constexpr int HBG = 2 * RKL;           // K_h | V_h span of one token in global memory
   constexpr int CPR = RKL / 16;          // 16-byte chunks per row
   constexpr int RPI = 64 / CPR;          // rows one DMA instruction covers
   constexpr int NLH = TT / (RPI * NW);   // DMA instructions per wave per tile, for K and again for V
@@ -66,7 +65,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   const int slot = (blockIdx.x / p.Hkv) % n_slots;
   const int chunk = blockIdx.x / (p.Hkv * n_slots);  // slowest: neighbouring blocks share a key chunk (L2 reuse)
   if (p.plan[2] == 0) return;  // the plan kernel saw no sequence with more than 16 rows per KV head
-  const int n_live = p.num_seqs[0];
+  const int n_live = live_rows(p);
   if (n_live <= 0) return;
   // sequence i starts at slot floor(qsl[i]*G/ROWS) + i; find the last sequence starting at or before `slot`
   int lo_i = 0, hi_i = n_live;
@@ -160,7 +159,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   // only so may the compiler keep these loads scalar after the assembly statements above have "written memory".
   typedef const __attribute__((address_space(4))) int32_t* ConstI32;
   ConstI32 bt = (ConstI32)(uintptr_t)(p.block_tables + (int64_t)i * p.M);
-  const char* pages = (const char*)p.kv_pages;
+  const char* k_pages = (const char*)p.k_pages;
+  const char* v_pages = (const char*)p.v_pages;
   const int pg = p.page_size;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
   const int dma_row = wave * RPI + lane / CPR;          // row for u = 0; instruction u adds u * NW * RPI
@@ -186,22 +186,24 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   int cur_page_raw = load_page(cur_idx);
   auto issue = [&]() __attribute__((always_inline)) {  // starts the DMA of the cursor's tile into LDS buffer cur_buf and advances the cursor
     const int cur_page = min(max(cur_page_raw, 0), p.P - 1);
-    const char* base = pages + (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride + (int64_t)h * HBG;
+    const int64_t tile_off = (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride + (int64_t)h * p.head_stride;
+    const char* base_k = k_pages + tile_off;
+    const char* base_v = v_pages + tile_off;
     const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
     const uint32_t buf_lds = lds_base + (uint32_t)cur_buf * TILE_BYTES + dma_wave_lds;
     if (!edge) {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {
-        dma16(buf_lds + u * NW * 1024, voff_k[u], base);                  // K rows
-        dma16(buf_lds + TT * RKL + u * NW * 1024, voff_v[u], base + RKL); // V rows
+        dma16(buf_lds + u * NW * 1024, voff_k[u], base_k);             // K rows
+        dma16(buf_lds + TT * RKL + u * NW * 1024, voff_v[u], base_v);  // V rows
       }
     } else {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {  // keys nobody may see: any visible row's bytes
         const int r = min(max(cur_tb + dma_row + u * NW * RPI, vis_lo), sp.ctx - 1) - cur_tb;
         const uint32_t roff = (uint32_t)r * (uint32_t)p.token_stride;
-        dma16(buf_lds + u * NW * 1024, roff + (uint32_t)(dma_chunk << 4), base);
-        dma16(buf_lds + TT * RKL + u * NW * 1024, roff + (uint32_t)(dma_chunk_v << 4), base + RKL);
+        dma16(buf_lds + u * NW * 1024, roff + (uint32_t)(dma_chunk << 4), base_k);
+        dma16(buf_lds + TT * RKL + u * NW * 1024, roff + (uint32_t)(dma_chunk_v << 4), base_v);
       }
     }
     cur_tb += TT;

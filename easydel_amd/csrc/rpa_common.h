@@ -18,12 +18,14 @@ constexpr int kMaxPrefillChunks = 8; // key chunks one prefill row tile may be s
 // Everything a kernel needs, passed by value.
 struct AttnParams {
   const void* q;
-  const void* kv_pages;
+  const void* k_pages;     // K of KV head h of a token: k_pages + page*page_stride + token*token_stride + h*head_stride
+  const void* v_pages;     // V likewise.  Interleaved pages: v_pages = k_pages + one row, head_stride = two rows;
+                           // separate K and V pools: two allocations, head_stride = one row
   const float* kv_scales;  // [P][C] or null
   const int32_t* context_lens;
   const int32_t* block_tables;
   const int32_t* qsl;
-  const int32_t* num_seqs;
+  const int32_t* num_seqs;  // live rows, or null: every one of the S rows is live
   void* out;
   float* part_o;   // [max_splits][Tdec][Hq][D]   Tdec = t_dec_max: decode-class query tokens, compacted
   float* part_ml;  // [max_splits][Tdec][Hq][2]   (running max in log2 units, running sum)
@@ -36,6 +38,7 @@ struct AttnParams {
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
   int64_t token_stride;  // bytes between consecutive tokens of a page = C*D*elem
   int64_t page_stride;   // bytes between pages
+  int64_t head_stride;   // bytes between KV heads inside a token
   int q_dtype, kv_dtype;
   float scale;       // softmax scale
   float scale_log2;  // softmax scale * log2(e)
@@ -55,6 +58,8 @@ struct AttnParams {
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
 };
 
+__device__ __forceinline__ int live_rows(const AttnParams& p);
+
 // Per-sequence facts.  Every kernel derives them from device metadata with this one function, so the
 // producers (attention kernels) and the consumer (merge) always agree on who wrote what.
 struct SeqPlan {
@@ -66,7 +71,7 @@ struct SeqPlan {
 
 __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
   SeqPlan s;
-  const int n_live = p.num_seqs[0];
+  const int n_live = live_rows(p);
   s.q0 = p.qsl[i];
   s.q_len = p.qsl[i + 1] - s.q0;
   s.ctx = p.context_lens[i];
@@ -81,6 +86,8 @@ __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
   s.small_rows = (s.q_len * p.group <= kRowBlock);
   return s;
 }
+
+__device__ __forceinline__ int live_rows(const AttnParams& p) { return p.num_seqs ? p.num_seqs[0] : p.S; }
 
 // Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + kPrefillRows) of a sequence) must visit, kv_lo
 // rounded down to 64, and the number of split-K chunks the prefill kernel cuts it into.

@@ -161,6 +161,48 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
     return out
 
 
+def unified_attention(query, key_cache, value_cache, context_lens, block_tables, query_start_loc, num_seqs=None, *,
+                      softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_scales=None, out=None):
+    """Ragged paged attention over separate K and V pools ``[P, page_size, Hkv, D]`` (the reference's
+    unified-attention layout).  ``num_seqs`` is optional: without it every row of ``context_lens`` is live."""
+    lib = _lib.load()
+    if key_cache.shape != value_cache.shape or key_cache.dtype != value_cache.dtype:
+        raise ValueError(f"key_cache {tuple(key_cache.shape)} {key_cache.dtype} and value_cache "
+                         f"{tuple(value_cache.shape)} {value_cache.dtype} must match")
+    if key_cache.ndim != 4:
+        raise ValueError(f"key_cache must be [P, page_size, Hkv, D], got {tuple(key_cache.shape)}")
+    T, Hq, D = query.shape
+    P, pg, Hkv, Dk = key_cache.shape
+    if Dk != D:
+        raise NotImplementedError(f"cache head_dim {Dk} != query head_dim {D}")
+    S = context_lens.shape[0]
+    if block_tables.numel() % S:
+        raise ValueError("block_tables size is not a multiple of the number of sequence rows")
+    M = block_tables.numel() // S
+    scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    window = int(sliding_window) if sliding_window else 0
+    cap = float(logits_soft_cap) if logits_soft_cap else 0.0
+    if out is None:
+        out = torch.empty_like(query)
+    if T == 0:
+        return out
+    qd, kd = dtype_tag(query.dtype), dtype_tag(key_cache.dtype)
+    for name, t in (("query", query), ("key_cache", key_cache), ("value_cache", value_cache), ("out", out)):
+        _dev(t, name)
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    scales_ptr = None
+    if kv_scales is not None:
+        if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * 2 * Hkv:
+            raise ValueError(f"kv_scales must be float32 [P={P}, 2*Hkv={2 * Hkv}]")
+        scales_ptr = _dev(kv_scales, "kv_scales")
+    _lib.check(lib.rpa_unified_attention(
+        _stream(query), _dev(query, "query"), _dev(key_cache, "key_cache"), _dev(value_cache, "value_cache"), scales_ptr,
+        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+        None if num_seqs is None else _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+        T, S, M, P, pg, Hq, Hkv, D, qd, kd, scale, window, cap))
+    return out
+
+
 def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_tables, query_start_loc, distribution, *,
                               softmax_scale=None, sliding_window=None, logits_soft_cap=None, num_kv_heads=None, out=None):
     """Fused scatter + attention; updates ``kv_pages`` in place and returns ``(out, kv_pages)``."""

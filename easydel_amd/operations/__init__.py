@@ -1,6 +1,7 @@
 from ._attention_outputs import AttentionOutput
 from ._base_operation import BaseOperation, EasyDeLBackends, OperationImpl, OperationMetadata, OperationRegistry
 from .ragged_page_attention import RaggedPageAttnV2, RaggedPageAttnV3
+from .unified_attention import UnifiedAttn
 from .requirements import (
     CacheRequirements,
     CacheType,
@@ -13,6 +14,6 @@ from .requirements import (
 
 __all__ = [
     "AttentionOutput", "BaseOperation", "EasyDeLBackends", "OperationImpl", "OperationMetadata", "OperationRegistry",
-    "RaggedPageAttnV2", "RaggedPageAttnV3", "CacheRequirements", "CacheType", "ExecutionMode", "MetadataField",
+    "RaggedPageAttnV2", "RaggedPageAttnV3", "UnifiedAttn", "CacheRequirements", "CacheType", "ExecutionMode", "MetadataField",
     "MetadataRequirements", "OperationRequirements", "RequirementsBuilder",
 ]

@@ -125,6 +125,25 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
                                float logits_soft_cap);
 
 /*
+ * The same attention over separate K and V pools: key_cache and value_cache are each
+ * [P][page_size][Hkv][D] (reference: easydel/caching/unified_attention/cache.py:216-218, :492-500).
+ * Replaces ejkernel.modules.unified_attention as called at
+ * easydel/operations/kernels/unified_attention.py:363-388 (and :319-331 for the shard-local form).
+ * The pools are filled by rpa_page_scatter_slices, once for K and once for V, with
+ * row_bytes = Hkv*D*elem (the reference's UnifiedAttentionCacheView.concatenate_to_cache, cache.py:523-610).
+ *
+ *   num_seqs   device, int32 [1], or NULL: the reference passes no row count to this kernel, every one of the
+ *              S rows is live and padded rows are those with an empty query span
+ *   kv_scales  device, float [P][2*Hkv] (K of head h at column 2h, V at 2h+1) or NULL; required for 8-bit pools
+ * Everything else as for rpa_ragged_paged_attention; the workspace size is the same function of the bounds.
+ */
+int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_cache, const void* value_cache,
+                          const float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
+                          const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
+                          size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D,
+                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap);
+
+/*
  * Fused v3 form: rpa_page_scatter_ragged followed by rpa_ragged_paged_attention on the
  * same stream, pages updated in place (the reference returns (out, kv_pages) and the
  * caller stores the pages back, ragged_page_attention.py:747).  key/value must already be

@@ -162,6 +162,24 @@ def run_gpu_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft
     return from_torch(out, b.q_dtype)
 
 
+def run_gpu_unified_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, device="cuda:0",
+                              pass_num_seqs=True):
+    """The same batch with its pages split into separate K and V pools ``[P, pg, Hkv, D]``."""
+    import torch
+
+    from easydel_amd import kernels
+
+    d = device_batch(b, device)
+    key_cache = d["kv_pages"][:, :, 0::2].contiguous()
+    value_cache = d["kv_pages"][:, :, 1::2].contiguous()
+    out = kernels.unified_attention(
+        d["query"], key_cache, value_cache, d["context_lens"], d["block_tables"], d["query_start_loc"],
+        d["num_seqs"] if pass_num_seqs else None, softmax_scale=softmax_scale, sliding_window=sliding_window,
+        logits_soft_cap=logits_soft_cap, kv_scales=d["kv_scales"])
+    torch.cuda.synchronize()
+    return from_torch(out, b.q_dtype)
+
+
 def valid_rows(b) -> slice:
     return slice(0, int(b.query_start_loc[b.n]))
 

@@ -158,3 +158,42 @@ def test_page_geometry_views():
         kernels.page_geometry(torch.empty((5, 16, 4, 2, 128), dtype=torch.bfloat16), 96)
     with pytest.raises(NotImplementedError):
         kernels.dtype_tag(torch.float16)
+
+
+def test_unified_attention_registry_requirements_and_config():
+    from easydel_amd.caching import UnifiedAttentionCacheConfig, UnifiedAttentionCacheView
+    from easydel_amd.operations import UnifiedAttn
+
+    assert OperationRegistry.get("unified_attention") is UnifiedAttn
+    req = UnifiedAttn.get_requirements(ExecutionMode.MIXED)
+    assert req.cache.cache_view_class is UnifiedAttentionCacheView and req.cache.is_compatible_with(CacheType.RAGGED_PAGES)
+    need = (MetadataField.SEQ_LENS | MetadataField.CONTEXT_LENS | MetadataField.POSITIONS | MetadataField.QUERY_START_LOC
+            | MetadataField.PAGES_TABLES | MetadataField.SLOT_MAPPING)
+    assert req.metadata.required == need and req.metadata.optional == MetadataField.LOGITS_INDICES
+    # sizing: K and V pools of all layers share the budget; slices per update page = min(64, pow2 <= 16 MiB / page bytes)
+    cfg = UnifiedAttentionCacheConfig.create(torch.bfloat16, num_hidden_layers=32, num_kv_heads=8, max_model_length=8192,
+                                             head_dim=128, page_size=128, hbm_utilization=0.9, free_hbm_bytes=10 << 30)
+    assert cfg.num_pages == int((10 << 30) * 0.9) // (2 * 32 * 128 * 8 * 128 * 2)
+    assert cfg.version == "v2" and cfg.max_num_pages_per_req == 64 and cfg.num_slices_per_kv_cache_update_page == 32
+    assert cfg.get_max_num_seqs() == 1024 * 1024 // 2 // 64 // 4
+    assert cfg.get_padded_num_slices(2048, 64) == 160  # 2*64 + 2048/128 = 144, rounded up to a multiple of 32
+    assert cfg.get_padded_num_slices(100, 64) == 128   # capped by the token count, then rounded up
+    small = UnifiedAttentionCacheConfig.create(torch.bfloat16, 1, 64, 8192, 256, page_size=128, num_pages=3)
+    assert small.num_slices_per_kv_cache_update_page == 2  # 16 MiB / 8 MiB pages
+    for bad in (dict(num_hidden_layers=0), dict(num_kv_heads=0), dict(head_dim=0), dict(page_size=0), dict(max_model_length=0)):
+        kw = dict(num_hidden_layers=1, num_kv_heads=2, max_model_length=64, head_dim=64, page_size=16, num_pages=4)
+        kw.update(bad)
+        with pytest.raises(ValueError):
+            UnifiedAttentionCacheConfig.create(torch.bfloat16, **kw)
+    with pytest.raises(ValueError, match="non-positive"):
+        UnifiedAttentionCacheConfig.create(torch.bfloat16, 1, 8, 64, 128, free_hbm_bytes=10)
+
+
+def test_unified_product_path_refuses_cpu_tensors():
+    q = torch.zeros((2, 8, 64), dtype=torch.bfloat16)
+    pool = torch.zeros((4, 16, 2, 64), dtype=torch.bfloat16)
+    i32 = lambda *s: torch.zeros(s, dtype=torch.int32)  # noqa: E731
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        kernels.unified_attention(q, pool, pool.clone(), i32(2), i32(2, 4), i32(3))
+    with pytest.raises(ValueError, match="must match"):
+        kernels.unified_attention(q, pool, pool[:, :8].contiguous(), i32(2), i32(2, 4), i32(3))
