@@ -190,11 +190,12 @@ def main():
                                       tens["query_start_loc"], tens["num_seqs"], softmax_scale=w.softmax_scale,
                                       sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap,
                                       kv_scales=tens["kv_scales"], out=out)
-        elif quant:  # quantised pages are read-only for this path
-            kernels.ragged_paged_attention(tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"],
-                                           tens["query_start_loc"], tens["num_seqs"], softmax_scale=w.softmax_scale,
-                                           sliding_window=w.sliding_window, logits_soft_cap=w.logits_soft_cap,
-                                           kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv, out=out)
+        elif quant:  # scaled 8-bit pages: quantising write of the new rows, then the attention
+            kernels.ragged_paged_attention_v3_quantised(tens["query"], tens["key"], tens["value"], tens["kv_pages"],
+                                                        tens["kv_scales"], tens["context_lens"], tens["block_tables"],
+                                                        tens["query_start_loc"], tens["distribution"],
+                                                        softmax_scale=w.softmax_scale, sliding_window=w.sliding_window,
+                                                        logits_soft_cap=w.logits_soft_cap, num_kv_heads=w.Hkv, out=out)
         else:
             kernels.ragged_paged_attention_v3(tens["query"], tens["key"], tens["value"], tens["kv_pages"],
                                               tens["context_lens"], tens["block_tables"], tens["query_start_loc"],

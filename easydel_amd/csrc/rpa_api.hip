@@ -13,6 +13,8 @@ int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_
 int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int);
 int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
+int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
+                                const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int);
 }  // namespace rpa
 
 namespace {
@@ -154,6 +156,29 @@ int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* va
   return hip_fail(rpa::launch_scatter_ragged((hipStream_t)stream, key, value, kv_pages, context_lens, block_tables,
                                              query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C, elem_bytes),
                   "rpa_page_scatter_ragged launch");
+}
+
+int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
+                                      float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
+                                      const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M, int P,
+                                      int page_size, int Hkv, int D, int C, int src_dtype, int kv_dtype) {
+  if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hkv <= 0 || D <= 0 || C < 2 * Hkv)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: bad size (T=%d S=%d M=%d P=%d page_size=%d Hkv=%d D=%d C=%d)",
+                T, S, M, P, page_size, Hkv, D, C);
+  if (D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "rpa_page_scatter_ragged_quantised: head_dim %d is not a multiple of 4", D);
+  if (src_dtype != RPA_F32 && src_dtype != RPA_BF16)
+    return fail(RPA_ERR_UNSUPPORTED, "rpa_page_scatter_ragged_quantised: source dtype %d (want f32 or bf16)", src_dtype);
+  if (kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8)
+    return fail(RPA_ERR_UNSUPPORTED, "rpa_page_scatter_ragged_quantised: page dtype %d (want fp8-e4m3 or int8)", kv_dtype);
+  if (T == 0) return RPA_OK;
+  if (!key || !value || !kv_pages || !kv_scales || !context_lens || !block_tables || !query_start_loc || !num_seqs)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: null pointer");
+  if ((((uintptr_t)key) | ((uintptr_t)value)) & 15 || ((uintptr_t)kv_pages & 3))
+    return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: key/value must be 16-byte and kv_pages 4-byte aligned");
+  return hip_fail(rpa::launch_scatter_ragged_quant((hipStream_t)stream, key, value, kv_pages, kv_scales, context_lens,
+                                                   block_tables, query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C,
+                                                   src_dtype, kv_dtype),
+                  "rpa_page_scatter_ragged_quantised launch");
 }
 
 size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int q_dtype,
@@ -305,6 +330,23 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                     T, S, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
   if (err) return err;
   return rpa_ragged_paged_attention(stream, q, kv_pages, nullptr, context_lens, block_tables, query_start_loc, n_live,
+                                    out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
+                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+}
+
+int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, const void* key, const void* value,
+                                            void* kv_pages, float* kv_scales, const int32_t* context_lens,
+                                            const int32_t* block_tables, const int32_t* query_start_loc,
+                                            const int32_t* distribution, void* out, void* workspace,
+                                            size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq,
+                                            int Hkv, int D, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
+                                            float softmax_scale, int sliding_window, float logits_soft_cap) {
+  if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention_v3_quantised: null distribution");
+  const int32_t* n_live = distribution + 2;
+  int err = rpa_page_scatter_ragged_quantised(stream, key, value, kv_pages, kv_scales, context_lens, block_tables,
+                                              query_start_loc, n_live, T, S, M, P, page_size, Hkv, D, C, kv_src_dtype, kv_dtype);
+  if (err) return err;
+  return rpa_ragged_paged_attention(stream, q, kv_pages, kv_scales, context_lens, block_tables, query_start_loc, n_live,
                                     out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
                                     kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
 }

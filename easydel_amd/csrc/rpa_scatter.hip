@@ -109,6 +109,134 @@ __global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restr
   }
 }
 
+// ---- quantising ragged write ---------------------------------------------------------------------------
+// Four scaled values -> four 8-bit codes in one dword: clamp to the code range, round to nearest even.
+template <int KVT>
+__device__ __forceinline__ uint32_t quant4(float a, float b, float c, float d) {
+  if constexpr (KVT == RPA_FP8_E4M3) {
+    const float q = 448.f;
+    a = fminf(fmaxf(a, -q), q); b = fminf(fmaxf(b, -q), q); c = fminf(fmaxf(c, -q), q); d = fminf(fmaxf(d, -q), q);
+    int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+    return (uint32_t)w;
+  } else {
+    const float q = 127.f;
+    const int ia = (int)rintf(fminf(fmaxf(a, -q), q)), ib = (int)rintf(fminf(fmaxf(b, -q), q));
+    const int ic = (int)rintf(fminf(fmaxf(c, -q), q)), id = (int)rintf(fminf(fmaxf(d, -q), q));
+    return (uint32_t)(ia & 0xff) | ((uint32_t)(ib & 0xff) << 8) | ((uint32_t)(ic & 0xff) << 16) | ((uint32_t)(id & 0xff) << 24);
+  }
+}
+
+template <int KVT>
+__device__ __forceinline__ void decode4_codes(uint32_t w, float* f) {
+  if constexpr (KVT == RPA_FP8_E4M3) {
+    auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = hi[0]; f[3] = hi[1];
+  } else {
+    f[0] = (float)(int8_t)(w & 0xff); f[1] = (float)(int8_t)((w >> 8) & 0xff);
+    f[2] = (float)(int8_t)((w >> 16) & 0xff); f[3] = (float)(int8_t)(w >> 24);
+  }
+}
+
+template <int SRC>
+__device__ __forceinline__ void load4_src(const void* base, int64_t idx, float* f) {  // idx: element index, multiple of 4
+  if constexpr (SRC == RPA_F32) {
+    const float4 v = *(const float4*)((const float*)base + idx);
+    f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+  } else {
+    const uint2 v = *(const uint2*)((const uint16_t*)base + idx);
+    f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+    f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+}
+
+// One wave per (query token, combined head); only the wave of the first new token a sequence writes to a page
+// works, and it handles all of that page's new tokens for its head:
+//   old scale (0 if the page starts with these tokens) -> new scale = max(old, amax / qmax), 1 if that is 0
+//   -> tokens already in the page re-coded if the scale grew -> new tokens coded -> scale stored.
+// All arithmetic in float32, in this order, so that the codes can be checked bit for bit.
+template <int SRC, int KVT>
+__global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __restrict__ key, const void* __restrict__ value,
+                                                                  unsigned char* __restrict__ pages, float* __restrict__ scales,
+                                                                  const int32_t* __restrict__ context_lens,
+                                                                  const int32_t* __restrict__ block_tables,
+                                                                  const int32_t* __restrict__ qsl,
+                                                                  const int32_t* __restrict__ num_seqs, int M, int P,
+                                                                  int page_size, int Hkv, int D, int C) {
+  const int t = blockIdx.x, c = blockIdx.y, lane = threadIdx.x;
+  const int n_live = num_seqs[0];
+  if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
+  const int i = find_seq(qsl, n_live, t);
+  const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
+  const int ctx = context_lens[i];
+  const int pos = ctx - q_len + (t - q0);
+  if (pos < 0) return;
+  const int first_pos = max(ctx - q_len, 0);
+  if (pos != first_pos && pos % page_size != 0) return;  // another token's wave covers this one
+  const int j = pos / page_size;
+  if (j >= M) return;
+  const int page = block_tables[(int64_t)i * M + j];
+  if (page < 0 || page >= P) return;
+  const int first = pos - j * page_size;
+  const int n = min(ctx, (j + 1) * page_size) - pos;
+  const float qmax = KVT == RPA_FP8_E4M3 ? 448.f : 127.f;
+  const int D4 = D >> 2;
+  const void* src = (c & 1) ? value : key;
+  const int64_t src0 = ((int64_t)t * Hkv + (c >> 1)) * D;  // element index of the first new token's head row
+  const int64_t src_row = (int64_t)Hkv * D;
+  unsigned char* dst = pages + ((int64_t)page * page_size * C + c) * D;  // token row r of this head: dst + r*C*D
+  const int64_t dst_row = (int64_t)C * D;
+
+  float amax = 0.f;
+  for (int idx = lane; idx < n * D4; idx += 64) {
+    const int r = idx / D4, c4 = idx - r * D4;
+    float f[4];
+    load4_src<SRC>(src, src0 + r * src_row + c4 * 4, f);
+    amax = fmaxf(amax, fmaxf(fmaxf(fabsf(f[0]), fabsf(f[1])), fmaxf(fabsf(f[2]), fabsf(f[3]))));
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  const float old_scale = first == 0 ? 0.f : scales[(int64_t)page * C + c];
+  float new_scale = fmaxf(old_scale, amax / qmax);
+  if (new_scale == 0.f) new_scale = 1.f;
+
+  if (new_scale > old_scale && first > 0) {
+    for (int idx = lane; idx < first * D4; idx += 64) {
+      const int r = idx / D4, c4 = idx - r * D4;
+      uint32_t* w = (uint32_t*)(dst + r * dst_row + c4 * 4);
+      float f[4];
+      decode4_codes<KVT>(*w, f);
+      *w = quant4<KVT>((f[0] * old_scale) / new_scale, (f[1] * old_scale) / new_scale, (f[2] * old_scale) / new_scale,
+                       (f[3] * old_scale) / new_scale);
+    }
+  }
+  for (int idx = lane; idx < n * D4; idx += 64) {
+    const int r = idx / D4, c4 = idx - r * D4;
+    float f[4];
+    load4_src<SRC>(src, src0 + r * src_row + c4 * 4, f);
+    *(uint32_t*)(dst + (first + r) * dst_row + c4 * 4) = quant4<KVT>(f[0] / new_scale, f[1] / new_scale, f[2] / new_scale, f[3] / new_scale);
+  }
+  if (lane == 0) scales[(int64_t)page * C + c] = new_scale;
+}
+
+int launch_scatter_ragged_quant(hipStream_t stream, const void* key, const void* value, void* pages, float* scales,
+                                const int32_t* context_lens, const int32_t* block_tables, const int32_t* qsl,
+                                const int32_t* num_seqs, int T, int M, int P, int page_size, int Hkv, int D, int C,
+                                int src_dtype, int kv_dtype) {
+  const dim3 grid(T, 2 * Hkv), block(64);
+#define RPA_QSCATTER(SRC, KVT)                                                                                        \
+  hipLaunchKernelGGL((scatter_ragged_quant_kernel<SRC, KVT>), grid, block, 0, stream, key, value, (unsigned char*)pages, \
+                     scales, context_lens, block_tables, qsl, num_seqs, M, P, page_size, Hkv, D, C)
+  if (src_dtype == RPA_F32 && kv_dtype == RPA_FP8_E4M3) RPA_QSCATTER(RPA_F32, RPA_FP8_E4M3);
+  else if (src_dtype == RPA_F32 && kv_dtype == RPA_INT8) RPA_QSCATTER(RPA_F32, RPA_INT8);
+  else if (src_dtype == RPA_BF16 && kv_dtype == RPA_FP8_E4M3) RPA_QSCATTER(RPA_BF16, RPA_FP8_E4M3);
+  else if (src_dtype == RPA_BF16 && kv_dtype == RPA_INT8) RPA_QSCATTER(RPA_BF16, RPA_INT8);
+  else return (int)hipErrorInvalidValue;
+#undef RPA_QSCATTER
+  return (int)hipGetLastError();
+}
+
 // Plain grid-stride copy of 16-byte vectors: the known-size kernel that calibrates HBM traffic counters.
 __global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;

@@ -119,6 +119,30 @@ def page_scatter_ragged(key, value, kv_pages, context_lens, block_tables, query_
     return kv_pages
 
 
+def page_scatter_ragged_quantised(key, value, kv_pages, kv_scales, context_lens, block_tables, query_start_loc, num_seqs):
+    """In-place quantising v3 write into scaled fp8 / int8 pages: per (page, combined head) the scale only grows
+    (``max(old, amax / qmax)``), tokens already in the page are re-coded when it does."""
+    lib = _lib.load()
+    if key.dtype != value.dtype or key.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"key/value must both be float32 or bfloat16, got {key.dtype}/{value.dtype}")
+    if kv_pages.dtype not in (torch.float8_e4m3fn, torch.int8):
+        raise TypeError(f"kv_pages must be float8_e4m3fn or int8 for the quantising write, got {kv_pages.dtype}")
+    T, Hkv, D = key.shape
+    P, pg, C = page_geometry(kv_pages, D)
+    if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
+        raise ValueError(f"kv_scales must be float32 [P={P}, C={C}]")
+    S = context_lens.shape[0]
+    M = block_tables.numel() // S
+    if T == 0:
+        return kv_pages, kv_scales
+    _dev(kv_pages, "kv_pages")
+    _lib.check(lib.rpa_page_scatter_ragged_quantised(
+        _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"), _dev(kv_scales, "kv_scales"),
+        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+        _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, dtype_tag(key.dtype), dtype_tag(kv_pages.dtype)))
+    return kv_pages, kv_scales
+
+
 def _attn_common(query, kv_pages, context_lens, block_tables, num_kv_heads, softmax_scale, sliding_window, logits_soft_cap):
     T, Hq, D = query.shape
     P, pg, C = page_geometry(kv_pages, D)
@@ -226,3 +250,32 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
         _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
         T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap))
     return out, kv_pages
+
+
+def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, context_lens, block_tables,
+                                        query_start_loc, distribution, *, softmax_scale=None, sliding_window=None,
+                                        logits_soft_cap=None, num_kv_heads=None, out=None):
+    """Fused quantising write + attention over scaled 8-bit pages; updates ``kv_pages`` and ``kv_scales`` in place
+    and returns ``(out, kv_pages, kv_scales)``.  ``key`` / ``value`` are float32 or bfloat16."""
+    lib = _lib.load()
+    if key.dtype != value.dtype or key.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError(f"key/value must both be float32 or bfloat16, got {key.dtype}/{value.dtype}")
+    T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+        query, kv_pages, context_lens, block_tables, key.shape[1] if num_kv_heads is None else num_kv_heads,
+        softmax_scale, sliding_window, logits_soft_cap)
+    if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
+        raise ValueError(f"kv_scales must be float32 [P={P}, C={C}]")
+    if out is None:
+        out = torch.empty_like(query)
+    if T == 0:
+        return out, kv_pages, kv_scales
+    qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
+    for name, t in (("query", query), ("key", key), ("value", value), ("kv_pages", kv_pages), ("kv_scales", kv_scales), ("out", out)):
+        _dev(t, name)
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    _lib.check(lib.rpa_ragged_paged_attention_v3_quantised(
+        _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+        _dev(kv_scales, "kv_scales"), _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"),
+        _i32(query_start_loc, "query_start_loc"), _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(),
+        ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap))
+    return out, kv_pages, kv_scales

@@ -63,12 +63,23 @@ class _RaggedPageAttn(OperationImpl):
             raise NotImplementedError("attention sinks (softmax_aux) are not implemented by the ROCm ragged-page kernels")
         kv_pages = cache_view.kv_pages
         if getattr(cache_view, "kv_scales", None) is not None:
-            # quantised pages are read-only for this path: whoever owns the cache wrote codes and scales
-            output = kernels.ragged_paged_attention(
-                query, kv_pages, cache_metadata.context_lens, cache_metadata.pages_tables.reshape(-1),
-                cache_metadata.query_start_loc, cache_metadata.request_distribution[2:3], softmax_scale=softmax_scale,
-                sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, kv_scales=cache_view.kv_scales,
-                num_kv_heads=_num_kv_heads(cache_view))
+            # scaled 8-bit pages: the write quantises (per page and head the scale only grows), then the attention
+            # reads codes and scales
+            if key is None or value is None:  # nothing to write: read the pages as they are
+                output = kernels.ragged_paged_attention(
+                    query, kv_pages, cache_metadata.context_lens, cache_metadata.pages_tables.reshape(-1),
+                    cache_metadata.query_start_loc, cache_metadata.request_distribution[2:3], softmax_scale=softmax_scale,
+                    sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, kv_scales=cache_view.kv_scales,
+                    num_kv_heads=_num_kv_heads(cache_view))
+                return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
+            if key.dtype not in (torch.float32, torch.bfloat16):
+                key, value = key.to(torch.float32), value.to(torch.float32)
+            output, kv_pages, kv_scales = kernels.ragged_paged_attention_v3_quantised(
+                query, key.contiguous(), value.to(key.dtype).contiguous(), kv_pages, cache_view.kv_scales,
+                cache_metadata.context_lens, cache_metadata.pages_tables.reshape(-1), cache_metadata.query_start_loc,
+                cache_metadata.request_distribution, softmax_scale=softmax_scale, sliding_window=sliding_window,
+                logits_soft_cap=logits_soft_cap, num_kv_heads=_num_kv_heads(cache_view))
+            cache_view.kv_pages, cache_view.kv_scales = kv_pages, kv_scales
             return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
         if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
             if kv_pages.element_size() < max(key.element_size(), value.element_size()):

@@ -89,6 +89,24 @@ int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* va
                             int P, int page_size, int Hkv, int D, int C, int elem_bytes);
 
 /*
+ * Page scatter, ragged form, into scaled 8-bit pages (RPA_FP8_E4M3 or RPA_INT8).  No counterpart in the
+ * reference, whose ragged pages carry no scales (its 8-bit page dtypes store unscaled casts,
+ * easydel/caching/ragged_page/cache.py:143-158): this is the write side of the page format the attention entry
+ * points read with kv_scales.  key/value are in src_dtype (RPA_F32 or RPA_BF16), placed as by
+ * rpa_page_scatter_ragged.  Per (sequence, page it writes to, combined head), in float32:
+ *   old   = 0 if the sequence's new tokens start the page, else kv_scales[page][head]
+ *   new   = max(old, amax|new values| / qmax), and 1 if that is 0        (qmax = 448 for fp8, 127 for int8)
+ *   tokens already in the page are re-coded, code <- quant((decode(code) * old) / new), if new > old
+ *   new tokens are coded quant(x / new); kv_scales[page][head] = new
+ * with quant = clamp to the code range, round to nearest even.  Deterministic and bit-exact against that rule.
+ * A page may be written by one sequence per call (pages shared between sequences are full pages).
+ */
+int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
+                                      float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
+                                      const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M, int P,
+                                      int page_size, int Hkv, int D, int C, int src_dtype, int kv_dtype);
+
+/*
  * Bytes of scratch rpa_ragged_paged_attention needs for these static bounds (split-K
  * partial outputs and their running max / sum).  The caller owns the buffer (under XLA it
  * is an extra result of the custom call), 256-byte aligned.
@@ -147,8 +165,8 @@ int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_ca
  * Fused v3 form: rpa_page_scatter_ragged followed by rpa_ragged_paged_attention on the
  * same stream, pages updated in place (the reference returns (out, kv_pages) and the
  * caller stores the pages back, ragged_page_attention.py:747).  key/value must already be
- * in the cache element type (the reference casts them first, :570-580); quantised pages
- * are read-only here, so kv_dtype must be RPA_F32 or RPA_BF16.
+ * in the cache element type (the reference casts them first, :570-580); kv_dtype must be
+ * RPA_F32 or RPA_BF16 (scaled 8-bit pages have rpa_ragged_paged_attention_v3_quantised).
  */
 int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void* key, const void* value,
                                   void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
@@ -156,6 +174,18 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P,
                                   int page_size, int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype,
                                   float softmax_scale, int sliding_window, float logits_soft_cap);
+
+/*
+ * Fused v3 form over scaled 8-bit pages: rpa_page_scatter_ragged_quantised followed by
+ * rpa_ragged_paged_attention on the same stream; pages and scales updated in place.  key/value in kv_src_dtype.
+ */
+int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, const void* key, const void* value,
+                                            void* kv_pages, float* kv_scales, const int32_t* context_lens,
+                                            const int32_t* block_tables, const int32_t* query_start_loc,
+                                            const int32_t* distribution, void* out, void* workspace,
+                                            size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq,
+                                            int Hkv, int D, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
+                                            float softmax_scale, int sliding_window, float logits_soft_cap);
 
 /*
  * Measurement aid with no counterpart in the reference: copies `bytes` (a multiple of 16, both

@@ -37,6 +37,11 @@ Pinning status
   (it runs inside ejkernel); pinned by equivalence with the v2 scatter driven by
   ``slot_mapping_v2_ref`` on the same batch.
 * e4m3fn / bf16 codecs: pinned against ``torch``'s CPU casts over all codes.
+* ``page_scatter_ragged_quantised_ref``: the scaled 8-bit page format has no counterpart in
+  the reference (its ragged pages carry no scales); this function defines it.  Pinned by
+  invariants in ``tests/test_oracle_formats.py`` (round-trip error bounds, monotone scales,
+  equivalence with one-shot quantisation when nothing is re-coded, placement equal to the
+  unquantised ragged write).
 """
 
 from __future__ import annotations
@@ -253,6 +258,77 @@ def page_scatter_ragged_ref(key, value, kv_pages, context_lens, block_tables, qu
             pages[page, pos % pg, 0:2 * hkv:2] = key[q0 + r]
             pages[page, pos % pg, 1:2 * hkv:2] = value[q0 + r]
     return pages
+
+
+QMAX = {FP8_E4M3: 448.0, INT8: 127.0}
+
+
+def quantise_codes(y: np.ndarray, kv_dtype: int) -> np.ndarray:
+    """Scaled values -> 8-bit codes as raw uint8: clamp to the code range, round to nearest even."""
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    q = np.float32(QMAX[kv_dtype])
+    y = np.minimum(np.maximum(y, -q), q)
+    if kv_dtype == FP8_E4M3:
+        return f32_to_e4m3fn_bits(y)
+    return np.rint(y).astype(np.int8).view(np.uint8)
+
+
+def decode_codes(raw: np.ndarray, kv_dtype: int) -> np.ndarray:
+    raw = np.ascontiguousarray(raw).view(np.uint8)
+    if kv_dtype == FP8_E4M3:
+        return e4m3fn_bits_to_f32(raw)
+    return raw.view(np.int8).astype(np.float32)
+
+
+def page_scatter_ragged_quantised_ref(key, value, kv_codes, kv_scales, context_lens, block_tables, query_start_loc,
+                                      num_seqs, *, kv_dtype: int):
+    """Quantising form of the ragged page write.  The scaled 8-bit page format belongs to this build (the
+    reference's ragged pages have no scales), so this function defines it; the kernel must match it bit for bit.
+
+    ``key/value [T, Hkv, D]`` float32 values; ``kv_codes [P, pg, C, D]`` raw uint8 codes; ``kv_scales [P, C]``
+    float32; value = code * scale[page, combined head].  Per (sequence, page it writes to, combined head), with
+    all arithmetic in float32:
+      * the new tokens of the page are ``[first, first + n)`` (token offsets inside the page);
+      * ``old = 0`` if ``first == 0`` (the page starts here: whatever scale it held belonged to an earlier owner),
+        else the stored scale;
+      * ``new = max(old, amax(|new values|) / qmax)``, and 1.0 if that is 0;
+      * if ``new > old`` and ``first > 0`` the tokens already in the page are re-coded:
+        ``code <- quant((decode(code) * old) / new)``;
+      * the new tokens are coded ``quant(x / new)``, and ``new`` is stored.
+    ``quant`` clamps to the code range and rounds to nearest even (``quantise_codes``).
+    Returns ``(codes, scales)``.
+    """
+    codes = np.array(kv_codes, copy=True).view(np.uint8)
+    scales = np.array(kv_scales, dtype=np.float32, copy=True)
+    pg = codes.shape[1]
+    hkv = key.shape[1]
+    qmax = np.float32(QMAX[kv_dtype])
+    bt = np.asarray(block_tables).reshape(len(context_lens), -1)
+    key = np.ascontiguousarray(key, dtype=np.float32)
+    value = np.ascontiguousarray(value, dtype=np.float32)
+    for i in range(int(np.asarray(num_seqs).reshape(-1)[0])):
+        q0, q1 = int(query_start_loc[i]), int(query_start_loc[i + 1])
+        ctx = int(context_lens[i])
+        q_len = q1 - q0
+        pos = max(ctx - q_len, 0)
+        while pos < ctx:
+            j, first = pos // pg, pos % pg
+            n = min(ctx, (j + 1) * pg) - pos
+            page = int(bt[i, j])
+            t0 = q0 + (pos - (ctx - q_len))
+            for c in range(2 * hkv):
+                src = (value if c & 1 else key)[t0:t0 + n, c >> 1]  # [n, D]
+                old = np.float32(0.0) if first == 0 else scales[page, c]
+                new = np.maximum(old, np.float32(np.abs(src).max()) / qmax).astype(np.float32)
+                if new == 0:
+                    new = np.float32(1.0)
+                if new > old and first > 0:
+                    prev = decode_codes(codes[page, :first, c], kv_dtype)
+                    codes[page, :first, c] = quantise_codes((prev * old) / new, kv_dtype)
+                codes[page, first:first + n, c] = quantise_codes(src / new, kv_dtype)
+                scales[page, c] = new
+            pos += n
+    return codes, scales
 
 
 # --------------------------------------------------------------------------------------
