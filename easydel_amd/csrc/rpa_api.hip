@@ -66,10 +66,30 @@ int static_splits(int T, int M, int page_size, int Hq, int D) {
 // Prefill split-K: keys per chunk and number of chunks the partial buffers hold, from the static bounds.
 // A row tile's key range is cut into at most kMaxPrefillChunks chunks of at least 8192 keys; the partial
 // buffers ([chunks][T][Hq][D+2] floats) are kept under ~1 GiB by allowing fewer, longer chunks.
-void prefill_split(int T, int M, int page_size, int Hq, int D, int* chunk_keys, int* max_chunks) {
+// Compute units of the current device (256 on MI355X); 0 if the query fails.
+int device_cus() {
+  static std::atomic<int> cached{-1};
+  int v = cached.load();
+  if (v >= 0) return v;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
+  cached.store(cus);
+  return cus;
+}
+
+// How a prefill row tile's key range is cut into chunks (each a workgroup of its own, merged afterwards).
+// Cutting pays when a batch holds few row tiles (a couple of long prompts): it fills the chip and evens out the
+// workgroups' lengths.  It costs a float32 partial per chunk and row, written and read back by the merge, so a batch
+// whose bounds already allow many times more row tiles than workgroups fit on the chip is not cut at all.
+void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int* chunk_keys, int* max_chunks) {
   const long span = (long)M * page_size;
   int chunks = g_prefill_chunks.load() > 0 ? g_prefill_chunks.load() : rpa::kMaxPrefillChunks;
   if (chunks > rpa::kMaxPrefillChunks) chunks = rpa::kMaxPrefillChunks;
+  if (g_prefill_chunks.load() <= 0 && Hkv > 0) {
+    const long row_tiles = ((long)T * (Hq / Hkv) / rpa::kPrefillRows + S) * Hkv;  // the prefill grid's bound without cutting
+    const int cus = device_cus();
+    if (cus > 0 && row_tiles >= 8L * cus) chunks = 1;
+  }
   const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   long keys = (span + chunks - 1) / chunks;
@@ -189,7 +209,7 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
   const int td = decode_token_bound(T, S, Hq, Hkv);
   const int splits = static_splits(td, M, page_size, Hq, D);
   int pre_keys, pre_chunks;
-  prefill_split(T, M, page_size, Hq, D, &pre_keys, &pre_chunks);
+  prefill_split(T, S, M, page_size, Hq, Hkv, D, &pre_keys, &pre_chunks);
   const size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) : 0;
   return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256;
 }
@@ -251,7 +271,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     const size_t po = part_o_bytes(td, Hq, D), pml = part_ml_bytes(td, Hq), pb = plan_bytes(S);
     int splits = static_splits(td, M, page_size, Hq, D);
     int pre_keys, pre_chunks;
-    prefill_split(T, M, page_size, Hq, D, &pre_keys, &pre_chunks);
+    prefill_split(T, S, M, page_size, Hq, Hkv, D, &pre_keys, &pre_chunks);
     const size_t pre_po = part_o_bytes(T, Hq, D), pre_pml = part_ml_bytes(T, Hq);
     size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (pre_po + pre_pml) : 0;
     size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
