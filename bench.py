@@ -49,8 +49,6 @@ def parse_args():
     ap.add_argument("--sequential-pages", action="store_true", help="experiment: block tables in pool order")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so a counter run shows what a known-size kernel reads")
-    ap.add_argument("--decode-wpb", type=int, default=0)
-    ap.add_argument("--decode-occ", type=int, default=0)
     return ap.parse_args()
 
 
@@ -155,10 +153,6 @@ def main():
         _lib.set_tunable("prefill_chunks", args.prefill_chunks)
     if args.max_splits:
         _lib.set_tunable("max_splits", args.max_splits)
-    if args.decode_wpb:
-        _lib.set_tunable("decode_wpb", args.decode_wpb)
-    if args.decode_occ:
-        _lib.set_tunable("decode_occ", args.decode_occ)
 
     dev = torch.device("cuda:0")
     w = build_workload(args.workload, args.seed, args.sequential_pages)

@@ -25,8 +25,6 @@ std::atomic<int> g_prefill_chunks{0};  // 0 = default (kMaxPrefillChunks)
 std::atomic<int> g_decode_sync{8};  // workgroup barrier every this many decode tiles (power of two, 0 = never)
 std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are resident at once
 std::atomic<int> g_force_generic{0};
-std::atomic<int> g_decode_wpb{0};
-std::atomic<int> g_decode_occ{0};
 std::atomic<int> g_prefill_dma{1};
 std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
 
@@ -134,8 +132,6 @@ int rpa_set_tunable(const char* name, int value) {
   }
   if (!strcmp(name, "decode_wgs")) return g_decode_wgs.exchange(value < 0 ? 0 : value);
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
-  if (!strcmp(name, "decode_wpb")) return g_decode_wpb.exchange(value);
-  if (!strcmp(name, "decode_occ")) return g_decode_occ.exchange(value);
   if (!strcmp(name, "prefill_dma")) return g_prefill_dma.exchange(value != 0);
   if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
   return -1;
@@ -255,8 +251,6 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
   p.decode_wgs = g_decode_wgs.load();
   p.decode_sync = g_decode_sync.load();
-  p.decode_wpb = g_decode_wpb.load();
-  p.decode_occ = g_decode_occ.load();
   p.prefill_dma = g_prefill_dma.load();
   p.max_splits = 2;
   p.pre_chunk = 1 << 30;

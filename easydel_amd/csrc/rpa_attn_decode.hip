@@ -56,8 +56,8 @@ __device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* 
   return pc;
 }
 
-template <int D, int KVT, int TT, int WPB, int OCC, bool CAP>
-__global__ __launch_bounds__(64 * WPB, OCC) void attn_decode_kernel(AttnParams p) {
+template <int D, int KVT, int TT, int WPB, bool CAP>
+__global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
   constexpr int HB = 2 * RK;           // K_h | V_h span of one token
@@ -459,7 +459,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   }
 }
 
-template <int D, int KVT, int TT, int WPB, int OCC, bool CAP>
+template <int D, int KVT, int TT, int WPB, bool CAP>
 static int launch_cap(hipStream_t stream, AttnParams p) {
   // persistent grid: as many workgroups as are resident at once, per KV-head group
   static int resident = 0;
@@ -467,7 +467,7 @@ static int launch_cap(hipStream_t stream, AttnParams p) {
     int dev = 0, cus = 0, per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, OCC, CAP>, 64 * WPB, 0) != hipSuccess)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP>, 64 * WPB, 0) != hipSuccess)
       return (int)hipGetLastError();
     resident = max(1, cus * max(1, per_cu));
   }
@@ -478,33 +478,27 @@ static int launch_cap(hipStream_t stream, AttnParams p) {
   p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2)
-    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, OCC, CAP>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();
 }
 
-template <int D, int KVT, int TT, int WPB, int OCC>
-static int launch_one(hipStream_t stream, const AttnParams& p) {
-  return p.softcap > 0.f ? launch_cap<D, KVT, TT, WPB, OCC, true>(stream, p) : launch_cap<D, KVT, TT, WPB, OCC, false>(stream, p);
-}
-
 template <int D, int KVT, int TT, int WPB>
-static int launch_occ(hipStream_t stream, const AttnParams& p) {
-  // waves per SIMD the register allocator must leave room for; 0 = compiler's choice
-  if (p.decode_occ == 4) return launch_one<D, KVT, TT, WPB, 4>(stream, p);
-  if (p.decode_occ == 3) return launch_one<D, KVT, TT, WPB, 3>(stream, p);
-  return launch_one<D, KVT, TT, WPB, 1>(stream, p);
+static int launch_one(hipStream_t stream, const AttnParams& p) {
+  return p.softcap > 0.f ? launch_cap<D, KVT, TT, WPB, true>(stream, p) : launch_cap<D, KVT, TT, WPB, false>(stream, p);
 }
 
+// Waves (KV heads) per workgroup: as many of 8 / 4 / 2 / 1 as there are heads and as LDS holds tiles for.
+// (Four waves per workgroup with more workgroups per CU, and builds for 3 or 4 waves per SIMD, measured no
+// faster on the Llama-shaped decode batch; the latter spill.)
 template <int D, int KVT, int TT>
 static int launch_wpb(hipStream_t stream, const AttnParams& p) {
   constexpr int tile_bytes = TT * 2 * D * ElemBytes<KVT>::v;
-  const int want = p.decode_wpb > 0 ? p.decode_wpb : 8;
   if constexpr (tile_bytes * 8 <= 65536) {
-    if (p.Hkv >= 8 && want >= 8) return launch_occ<D, KVT, TT, 8>(stream, p);
+    if (p.Hkv >= 8) return launch_one<D, KVT, TT, 8>(stream, p);
   }
-  if (p.Hkv >= 4 && want >= 4) return launch_occ<D, KVT, TT, 4>(stream, p);
-  if (p.Hkv >= 2 && want >= 2) return launch_occ<D, KVT, TT, 2>(stream, p);
-  return launch_occ<D, KVT, TT, 1>(stream, p);
+  if (p.Hkv >= 4) return launch_one<D, KVT, TT, 4>(stream, p);
+  if (p.Hkv >= 2) return launch_one<D, KVT, TT, 2>(stream, p);
+  return launch_one<D, KVT, TT, 1>(stream, p);
 }
 
 template <int KVT>

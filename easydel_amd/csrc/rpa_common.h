@@ -52,8 +52,6 @@ struct AttnParams {
   int pre_max_chunks;  // chunks the prefill partial buffers hold; 1 = never split
   int decode_sync;   // decode workgroups re-align their waves with a barrier every this many tiles (power of two), 0 = never
   int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel
-  int decode_wpb;    // waves (KV heads) per decode workgroup, 0 = default
-  int decode_occ;    // waves per SIMD the decode kernel is compiled for, 0 = compiler's choice
   int prefill_dma;   // 1: bf16 prefill tiles go global -> LDS directly where that kernel applies; 0: always through registers
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
 };
