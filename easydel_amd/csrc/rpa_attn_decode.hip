@@ -14,9 +14,13 @@
 //     O^T[dim][row]  += V^T[dim][token] . P^T[token][row] v_mfma_f32_16x16x16_bf16, k = tokens
 // S^T's accumulator layout (lane = row, 4 tokens per lane) is exactly the B-operand layout of the
 // second product, so probabilities never cross lanes; only the running max does (2 steps).
-// fp8 / int8 pages are widened to bf16 (exactly) after the LDS read; their per-(page, head)
-// scales fold into the score scale (K) and into P (V).
-// No barriers: LDS tiles are wave-private and LDS operations of one wave execute in order.
+// bf16 V operands come from transposing LDS reads (ds_read_b64_tr_b16); fp8 / int8 pages are widened
+// to bf16 (exactly) after the LDS read.  Their per-(page, head) scales travel with the tile: the K scale
+// folds into the score scale, and the accumulators are kept in units of the current page's V scale, so
+// the probabilities stay exact softmax weights.
+// LDS tiles are wave-private and LDS operations of one wave execute in order, so no barrier is needed for
+// correctness; one every few tiles keeps the workgroup's waves on the same token rows, which keeps its
+// outstanding loads inside the same DRAM rows.
 #include <type_traits>
 
 #include "rpa_mfma.h"

@@ -18,7 +18,7 @@ def _check(b, what, **kw):
 
 
 def test_config1_fp32_mixed_batch(gpu):
-    # BASELINE config 1: 4 sequences, ctx [17,64,130,255], q_lens [1,1,8,33], Hq 8, Hkv 2, D 64, page 16, 128 pages
+    # the tiny fp32 configuration: 4 sequences, ctx [17,64,130,255], q_lens [1,1,8,33], Hq 8, Hkv 2, D 64, page 16, 128 pages
     b = tl.make_batch(0, [17, 64, 130, 255], [1, 1, 8, 33], Hq=8, Hkv=2, D=64, page_size=16, num_pages=128,
                       q_dtype=F32, kv_dtype=F32)
     assert list(b.query_start_loc[:5]) == [0, 1, 2, 10, 43]
