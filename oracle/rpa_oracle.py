@@ -29,10 +29,11 @@ Pinning status
   the scatter.
 * ``ragged_paged_attention_ref``: the reference holds no golden vector for the
   attention output (its only test of the call mocks the kernel out); pinned by
-  mathematics only -- see ``tests/test_oracle_attention.py``.  The residual
-  conventions that only an import of ejkernel could confirm (bf16 rounding
-  points, values written to padded rows) are listed in the design notes and are
-  covered by comparing valid rows only, at the stated tolerances.
+  mathematics only -- see ``tests/test_oracle_attention.py`` -- and therefore
+  "parity unpinned" against ejkernel.  The residual conventions that only an
+  import of ejkernel could confirm (where its XLA path rounds to bf16, what it
+  writes to padded rows, the mask value of fully masked rows) are covered by
+  comparing valid rows only, at the stated tolerances.
 * ``page_scatter_ragged_ref`` (the fused v3 write): no reference vector exists
   (it runs inside ejkernel); pinned by equivalence with the v2 scatter driven by
   ``slot_mapping_v2_ref`` on the same batch.
