@@ -68,10 +68,10 @@ def build_workload(name, seed, sequential=False):
     return workloads.config5_gemma_long_prefill(seed, windowed=(name == "c5-window"))
 
 
-def measured_traffic(workload):
-    """HBM bytes per decode-kernel launch from the committed counter runs (FETCH_SIZE and WRITE_SIZE passes,
-    each scaled by what the same counter reads for a 1 GiB copy); None for workloads without such a run."""
-    path = os.path.join(ROOT, "profiles", f"attn_decode_kernel_{workload.replace('-', '_')}_traffic.json")
+def measured_traffic(workload, kernel="attn_decode_kernel"):
+    """HBM bytes per launch of a kernel from the committed counter runs (FETCH_SIZE and WRITE_SIZE passes, each
+    scaled by what the same counter reads for a 1 GiB copy); None for workloads without such a run."""
+    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload.replace('-', '_')}_traffic.json")
     try:
         with open(path) as f:
             return float(json.load(f)["hbm_bytes_per_launch"])
@@ -250,14 +250,15 @@ def main():
         nbytes = w.attention_bytes(small)
         kern["attn_decode_kernel"] = {
             "bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": measured_traffic(args.workload),
+            "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None if unified else measured_traffic(args.workload),
             "algorithmic_bytes_per_launch": nbytes, "kernel_ms": ms}
     if (~small & (w.q_lens > 0)).any():
         ms = time_stage(4, args.steps)
         flops = w.attention_flops(~small)
         kern["attn_prefill_kernel"] = {
             "bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+            "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "traffic": None if unified else measured_traffic(args.workload, "attn_prefill_kernel"),
             "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": w.attention_bytes(~small),
             "kernel_ms": ms}
     _lib.set_tunable("stages", prev)
