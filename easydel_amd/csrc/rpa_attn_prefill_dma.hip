@@ -329,31 +329,40 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     // values of keys 4g4..4g4+3, which is the A operand of the product with k = keys.
     const int tr_key = 4 * g4 + (n >> 2);          // key (within a 16-key sub-tile) this lane addresses
     const int tr_byte = (n & 3) * 8;               // byte offset of its 4 dims inside the 32-byte row-tile span
+    // The V operands are read PD row tiles ahead of the MFMAs that use them: one row tile of MFMAs lasts 32 cycles,
+    // an LDS read under load several times that, so a wave that reads just in time waits at every row tile.
+    constexpr int PD = DPL < 4 ? DPL : 4;
+    auto read_v = [&](int rt) -> u32x4 {
+      const int off = rt * 32 + tr_byte;
+      const unsigned char* lo = lds_v + tr_key * RKL + (((off >> 4) ^ swz_key_v<RKL>(tr_key)) << 4) + (off & 15);
+      const unsigned char* hi = lds_v + (16 + tr_key) * RKL + (((off >> 4) ^ swz_key_v<RKL>(16 + tr_key)) << 4) + (off & 15);
+      const u32x2 a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)lo));
+      const u32x2 a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)hi));
+      return (u32x4){a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
+    };
     __builtin_amdgcn_sched_barrier(0);  // keep the V operand reads out of the softmax: they would only pile up in registers
+    u32x4 av[PD];
+#pragma unroll
+    for (int rt = 0; rt < PD; ++rt) av[rt] = read_v(rt);
 #pragma unroll
     for (int rt = 0; rt < DPL; ++rt) {
-      if (rt > 0 && rt % 4 == 0) __builtin_amdgcn_sched_barrier(0);
-      u32x2 a_lo, a_hi;
-      {
-        const int tk = tr_key;
-        const int off = rt * 32 + tr_byte;
-        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key_v<RKL>(tk)) << 4) + (off & 15);
-        a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
-      }
-      {
-        const int tk = 16 + tr_key;
-        const int off = rt * 32 + tr_byte;
-        const unsigned char* ptr = lds_v + tk * RKL + (((off >> 4) ^ swz_key_v<RKL>(tk)) << 4) + (off & 15);
-        a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr));
-      }
-      const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
+      const u32x4 a4 = av[rt % PD];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
         o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
                                                                 o_acc[rb][rt], 0, 0, 0);
       }
+      if (rt + PD < DPL) av[rt % PD] = read_v(rt + PD);
     }
+    // The order the scheduler must keep: PD row tiles of reads first, then a row tile of MFMAs and the next reads in turn.
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * PD, 0);
+#pragma unroll
+    for (int rt = 0; rt + PD < DPL; ++rt) {
+      __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, RB * PD, 0);
   };
   auto needs_mask = [&](int tb) { return !((tb >= wave_lo) && (tb + TT <= wave_hi)); };
   auto buf_k = [&](int t) -> const unsigned char* { return lds_all + (t & (NBUF - 1)) * TILE_BYTES; };
