@@ -47,11 +47,14 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   constexpr int DPL = D / 16;            // 16-dim row tiles of O^T
   constexpr int NKK = D / 32;            // k-steps of the score MFMA
   constexpr int ROWS = NW * RB * 16;
+  constexpr float kMaxSlack = 8.f;       // how far a score may exceed the softmax reference before it is raised
   static_assert(ROWS == kPrefillRows, "merge kernel assumes this row-tile height");
-  constexpr int TILE_BYTES = TT * 2 * RKL;
-  constexpr int NBUF = 4;
+  constexpr int HALF = TT * RKL;         // bytes of the K (or V) rows of one tile
+  // K of a tile is needed a step before its V (see the pipeline below), so the two halves live in rings of their
+  // own: three K slots and five V slots hold everything between a tile's issue and its last read.
+  constexpr int KN = 3, VN = 5;
 
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[NBUF * TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[(KN + VN) * HALF];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -171,7 +174,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   int cur_idx = kv_lo / pg;
   int cur_off = kv_lo - cur_idx * pg;
   int cur_tb = kv_lo;
-  int cur_buf = 0;
+  int cur_ks = 0, cur_vs = 0;  // ring slots of the tile the cursor is at
   // Lane offsets of an ordinary tile, loop-invariant; only a tile that holds keys nobody may see recomputes them.
   uint32_t voff_k[NLH], voff_v[NLH];
 #pragma unroll
@@ -184,26 +187,27 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   // waits for the scalar load it has just made.
   auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
   int cur_page_raw = load_page(cur_idx);
-  auto issue = [&]() __attribute__((always_inline)) {  // starts the DMA of the cursor's tile into LDS buffer cur_buf and advances the cursor
+  auto issue = [&]() __attribute__((always_inline)) {  // starts the DMA of the cursor's tile into its ring slots and advances the cursor
     const int cur_page = min(max(cur_page_raw, 0), p.P - 1);
     const int64_t tile_off = (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride + (int64_t)h * p.head_stride;
     const char* base_k = k_pages + tile_off;
     const char* base_v = v_pages + tile_off;
     const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
-    const uint32_t buf_lds = lds_base + (uint32_t)cur_buf * TILE_BYTES + dma_wave_lds;
+    const uint32_t k_lds = lds_base + (uint32_t)cur_ks * HALF + dma_wave_lds;
+    const uint32_t v_lds = lds_base + (uint32_t)(KN + cur_vs) * HALF + dma_wave_lds;
     if (!edge) {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {
-        dma16(buf_lds + u * NW * 1024, voff_k[u], base_k);             // K rows
-        dma16(buf_lds + TT * RKL + u * NW * 1024, voff_v[u], base_v);  // V rows
+        dma16(k_lds + u * NW * 1024, voff_k[u], base_k);  // K rows
+        dma16(v_lds + u * NW * 1024, voff_v[u], base_v);  // V rows
       }
     } else {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {  // keys nobody may see: any visible row's bytes
         const int r = min(max(cur_tb + dma_row + u * NW * RPI, vis_lo), sp.ctx - 1) - cur_tb;
         const uint32_t roff = (uint32_t)r * (uint32_t)p.token_stride;
-        dma16(buf_lds + u * NW * 1024, roff + (uint32_t)(dma_chunk << 4), base_k);
-        dma16(buf_lds + TT * RKL + u * NW * 1024, roff + (uint32_t)(dma_chunk_v << 4), base_v);
+        dma16(k_lds + u * NW * 1024, roff + (uint32_t)(dma_chunk << 4), base_k);
+        dma16(v_lds + u * NW * 1024, roff + (uint32_t)(dma_chunk_v << 4), base_v);
       }
     }
     cur_tb += TT;
@@ -212,7 +216,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       cur_off -= pg;
       ++cur_idx;
     }
-    cur_buf = (cur_buf + 1) & (NBUF - 1);
+    cur_ks = (cur_ks == KN - 1) ? 0 : cur_ks + 1;
+    cur_vs = (cur_vs == VN - 1) ? 0 : cur_vs + 1;
     cur_page_raw = load_page(cur_idx);
   };
 
@@ -231,30 +236,36 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   }
 
   // ---- S^T = K . Q^T for every row block (K operands shared) ------------------------------------------
-  auto qk = [&](const unsigned char* lds_k, f32x4 (&sa)[RB][NS]) __attribute__((always_inline)) {
+  // K operand i = (16-key sub-tile i / NKK, k-step i % NKK).  The first KPD operands of a tile are read a phase
+  // early (k_prefetch, behind the PV MFMAs of the tile before), the rest KPD operands ahead of their MFMAs.
+  constexpr int NKO = NS * NKK;
+  constexpr int KPD = NKO < 4 ? NKO : 4;
+  auto read_k = [&](const unsigned char* lds_k, int i) __attribute__((always_inline)) -> u32x4 {
+    const int tk = (i / NKK) * 16 + n;
+    return *(const u32x4*)(lds_k + tk * RKL + ((((i % NKK) * 4 + g4) ^ swz_key<RKL>(tk)) << 4));
+  };
+  auto k_prefetch = [&](const unsigned char* lds_k, u32x4 (&kp)[KPD]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < KPD; ++i) kp[i] = read_k(lds_k, i);
+  };
+  auto qk = [&](const unsigned char* lds_k, u32x4 (&kp)[KPD], f32x4 (&sa)[RB][NS]) __attribute__((always_inline)) {
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int st = 0; st < NS; ++st) sa[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int st = 0; st < NS; ++st) {
-      const int tk = st * 16 + n;
-      const unsigned char* krow = lds_k + tk * RKL;
-      const int key = swz_key<RKL>(tk);
+    for (int i = 0; i < NKO; ++i) {
+      const u32x4 a = kp[i % KPD];
 #pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) {
-        const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
-          sa[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], sa[rb][st], 0, 0, 0);
-      }
+      for (int rb = 0; rb < RB; ++rb)
+        sa[rb][i / NKK] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][i % NKK], sa[rb][i / NKK], 0, 0, 0);
+      if (i + KPD < NKO) kp[i % KPD] = read_k(lds_k, i + KPD);
     }
   };
-  // ---- online softmax of the scores of tile tb, then O^T += V^T . P^T ---------------------------------
-  auto soft_pv = [&](auto mask_tag, f32x4 (&sa)[RB][NS], int tb, const unsigned char* lds_v) __attribute__((always_inline)) {
+  // ---- online softmax of the scores of tile tb ----------------------------------------------------------
+  auto softmax = [&](auto mask_tag, f32x4 (&sa)[RB][NS], int tb, uint32_t (&pfrag)[RB][NS][2]) __attribute__((always_inline)) {
     constexpr bool MASK = decltype(mask_tag)::value;
     const float sc_mul = CAP ? cap_out : p.scale_log2;
-    uint32_t pfrag[RB][NS][2];
     // Soft cap and mask in place; each lane's maximum over its own 8 keys of the row.
     float lmx[RB];
     bool grow = false;
@@ -275,11 +286,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
           lmx[rb] = fmaxf(lmx[rb], sv);
         }
       lmx[rb] *= sc_mul;  // sc_mul > 0: scaling commutes with the maximum
-      grow |= lmx[rb] > m_run[rb];
+      grow |= lmx[rb] > m_run[rb] + kMaxSlack;
     }
-    // The running maximum is the reference every probability of a row is taken against.  Only when some key of
-    // the tile exceeds it (rare once a few tiles are behind) is it raised: the lanes of a row then agree on the new
-    // maximum and everything accumulated so far is scaled down.  Otherwise the tile costs neither the lane
+    // The reference every probability of a row is taken against need not be the exact running maximum: any common
+    // value works as long as exp2 stays in range, the quotient of the two accumulated sums does not depend on it.
+    // It is raised -- the lanes of a row agree on the new maximum and everything accumulated so far is scaled down --
+    // only when some key of the tile exceeds it by more than kMaxSlack (in log2 units, so probabilities stay below
+    // 2^kMaxSlack).  After the first tiles of a sequence that is rare, and a tile then costs neither the lane
     // exchange nor a rescale.
     if (__any(grow)) {
 #pragma unroll
@@ -313,6 +326,9 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
         pfrag[rb][st][1] = pack_bf16(pr[2], pr[3]);
       }
     }
+  };
+  // ---- O^T += V^T . P^T, and the row sums ------------------------------------------------------------------
+  auto pv = [&](uint32_t (&pfrag)[RB][NS][2], const unsigned char* lds_v) __attribute__((always_inline)) {
     // The row sums come from the matrix cores as well: a V^T tile of ones times P^T leaves, in every accumulator
     // element of column n, the sum of row n's probabilities over all 32 keys (as rounded to bf16, i.e. exactly the
     // weights the PV product uses).  Two MFMAs replace 16 additions per lane and the cross-lane sum at the end.
@@ -364,54 +380,76 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     }
     __builtin_amdgcn_sched_group_barrier(0x008, RB * PD, 0);
   };
-  auto needs_mask = [&](int tb) { return !((tb >= wave_lo) && (tb + TT <= wave_hi)); };
-  auto buf_k = [&](int t) -> const unsigned char* { return lds_all + (t & (NBUF - 1)) * TILE_BYTES; };
-  auto buf_v = [&](int t) -> const unsigned char* { return lds_all + (t & (NBUF - 1)) * TILE_BYTES + TT * RKL; };
-
   // ---- pipeline ----------------------------------------------------------------------------------------
-  // Step t: the matrix cores compute the scores of tile t+1 while the vector ALU does the softmax of tile t,
-  // then the PV product of tile t runs.  Four LDS buffers: during step t tiles t (V) and t+1 (K) are read and
-  // tiles t+2 and t+3 are in flight; tile t+3 goes where tile t-1 lay, whose last reader finished before the
-  // barrier that opens step t.
+  // Step t: (A) the matrix cores compute the scores of tile t+1 while the vector ALU does the softmax of tile t;
+  // (B) the workgroup meets at the step's barrier, behind which tile t+2 is visible and the slots of K(t+1) and
+  // V(t-1) are free: tile t+4 is issued into them and the first K operands of tile t+2 are read; (C) the PV product
+  // of tile t runs, hiding the latency of those reads, so that the next step starts on the matrix cores at once.
+  // (With the barrier at the head of the step every wave of the CU asked LDS for its K operands at the same moment
+  // and waited for them with nothing else to do: a quarter of the kernel's time.)
+  auto k_slot = [&](int sl) -> const unsigned char* { return lds_all + sl * HALF; };
+  auto v_slot = [&](int sl) -> const unsigned char* { return lds_all + (KN + sl) * HALF; };
+  const std::true_type masked{};
+  f32x4 s_cur[RB][NS], s_nxt[RB][NS];
+  uint32_t pf[RB][NS][2];
+  u32x4 kp[KPD];
   issue();                   // tile 0
   if (n_tiles > 1) issue();  // tile 1
   if (n_tiles > 2) issue();  // tile 2
   if (n_tiles > 2) wait_loads_and_barrier<4 * NLH>();
   else if (n_tiles > 1) wait_loads_and_barrier<2 * NLH>();
   else wait_loads_and_barrier<0>();
-  // (A wave whose rows all lie past the sequence's end computes like the others, on zero queries: its rows are
-  // never stored, and the loop stays free of a branch around every step.)
-  f32x4 s_cur[RB][NS], s_alt[RB][NS];
-  qk(buf_k(0), s_cur);
-  int t = 0;
-  auto step = [&](auto mask_tag, f32x4 (&s_in)[RB][NS], f32x4 (&s_out)[RB][NS], int ts) __attribute__((always_inline)) {
-    if (ts + 2 < n_tiles) wait_loads_and_barrier<2 * NLH>();  // tile ts+1 has landed; tile ts+2 may still be in flight
+  k_prefetch(k_slot(0), kp);
+  qk(k_slot(0), kp, s_cur);
+  if (n_tiles > 1) {
+    if (n_tiles > 2) wait_loads_and_barrier<2 * NLH>();  // tile 1 has landed, and every wave is done with K slot 0
     else wait_loads_and_barrier<0>();
-    if (ts + 3 < n_tiles) issue();
-    qk(buf_k(ts + 1), s_out);
-    soft_pv(mask_tag, s_in, kv_lo + ts * TT, buf_v(ts));
-  };
+    if (n_tiles > 3) issue();  // tile 3
+    k_prefetch(k_slot(1), kp);
+  }
+  int t = 0;
+  int rd_k = 1, rd_v = 0;  // ring slots of K(t+1) and V(t)
+  auto next_k = [&](int sl) { return sl == KN - 1 ? 0 : sl + 1; };
   // Steps [t, t_end) with or without the masking code.  Two variants side by side in one loop body (an if / else
   // around the step) make the compiler keep a second copy of every accumulator, so the choice is made per run of
   // steps instead: masked steps at the window's lower edge, unmasked ones, masked ones at the causal edge.
   // (Unrolling two steps per trip to alternate the score registers instead of copying them was tried: the
   // compiler then needs 50 more registers and spills.)
   auto run = [&](auto mask_tag, int t_end) __attribute__((always_inline)) {
-    for (; t < t_end; ++t) {
-      step(mask_tag, s_cur, s_alt, t);
+    for (; t < t_end; ++t) {  // t + 2 < n_tiles
+      qk(k_slot(rd_k), kp, s_nxt);
+      softmax(mask_tag, s_cur, kv_lo + t * TT, pf);
+      if (t + 3 < n_tiles) wait_loads_and_barrier<2 * NLH>();  // tile t+2 has landed; tile t+3 may still be in flight
+      else wait_loads_and_barrier<0>();
+      if (t + 4 < n_tiles) issue();
+      rd_k = next_k(rd_k);
+      k_prefetch(k_slot(rd_k), kp);
+      pv(pf, v_slot(rd_v));
+      rd_v = (rd_v == VN - 1) ? 0 : rd_v + 1;
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-        for (int st = 0; st < NS; ++st) s_cur[rb][st] = s_alt[rb][st];
+        for (int st = 0; st < NS; ++st) s_cur[rb][st] = s_nxt[rb][st];
     }
   };
   const int t_plain_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT);  // first tile no row of the wave masks from below
   const int t_plain_hi = (wave_hi - kv_lo) / TT;                   // first tile some row of the wave masks from above
-  run(std::true_type{}, min(t_plain_lo, n_tiles - 1));
-  run(std::false_type{}, min(t_plain_hi, n_tiles - 1));
-  run(std::true_type{}, n_tiles - 1);
-  soft_pv(std::true_type{}, s_cur, kv_lo + t * TT, buf_v(t));  // last tile: nothing left to overlap with
-  (void)needs_mask;
+  run(masked, min(t_plain_lo, n_tiles - 2));
+  run(std::false_type{}, min(t_plain_hi, n_tiles - 2));
+  run(masked, n_tiles - 2);
+  if (n_tiles > 1) {  // t = n_tiles - 2: the last scores; every tile has landed and is visible
+    qk(k_slot(rd_k), kp, s_nxt);
+    softmax(masked, s_cur, kv_lo + t * TT, pf);
+    pv(pf, v_slot(rd_v));
+    rd_v = (rd_v == VN - 1) ? 0 : rd_v + 1;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int st = 0; st < NS; ++st) s_cur[rb][st] = s_nxt[rb][st];
+    ++t;
+  }
+  softmax(masked, s_cur, kv_lo + t * TT, pf);  // the last tile
+  pv(pf, v_slot(rd_v));
   (void)wave_active;
   (void)wave_lo_min; (void)wave_hi_max;
 
