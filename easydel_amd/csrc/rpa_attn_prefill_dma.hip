@@ -1,15 +1,17 @@
 // MFMA prefill / chunked-prefill attention for bf16 pages, K/V tiles moved global -> LDS by the
-// load unit itself (global_load_lds_dwordx4), three tiles deep.
+// load unit itself (global_load_lds_dwordx4) and the loop software-pipelined inside every wave.
 //
 // Same work split and arithmetic as attn_prefill_kernel (rpa_attn_prefill.hip): a workgroup owns 128
 // query rows of one (sequence, KV head), each wave keeps RB 16-row blocks in registers and every wave
-// reads the shared K/V tile in MFMA operand order.  What differs is how a tile reaches LDS.  There the
-// tile passes through registers (load, wait, ds_write), which costs staging registers, address and
-// write instructions, and leaves one tile of prefetch.  Here every lane hands the load unit one 16-byte
-// global address and the unit writes the 64 lanes' chunks to 1 KiB of LDS in lane order; the XOR swizzle
-// of the tile is applied on the global side (lane for LDS chunk c' of row r fetches global chunk
-// c' ^ key(r)).  No registers are held while a tile is in flight, so tiles t+1 and t+2 are on their way
-// while tile t is computed, and the compute loop holds no global-memory instructions of its own.
+// reads the shared K/V tile in MFMA operand order.  What differs is how a tile reaches LDS and how a
+// step is scheduled.  There the tile passes through registers (load, wait, ds_write), which costs
+// staging registers, address and write instructions, and leaves one tile of prefetch; scores, softmax
+// and PV product run one after the other.  Here every lane hands the load unit one 16-byte global
+// address and the unit writes the 64 lanes' chunks to 1 KiB of LDS in lane order; the XOR swizzle of
+// the tile is applied on the global side (lane for LDS chunk c' of row r fetches global chunk
+// c' ^ key(r)).  No registers are held while a tile is in flight, so a tile is issued four steps before
+// its last read, and the compute loop holds no global-memory instructions of its own.  Inside a step the
+// scores of the next tile run on the matrix cores while the vector ALU does the softmax of this one.
 //
 // The loads are issued through inline assembly: the compiler then neither tracks them nor orders its
 // own waits around them, and the kernel states its waits itself (s_waitcnt vmcnt(n) + s_barrier before a
