@@ -28,20 +28,20 @@ SIGNATURES = {
     "rpa_attention_workspace_bytes": (_c_sz, [_c_int] * 9),
     "rpa_ragged_paged_attention": (
         _c_int,
-        [_c_vp] * 10 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32],
+        [_c_vp] * 10 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
     "rpa_page_scatter_ragged_quantised": (_c_int, [_c_vp] * 9 + [_c_int] * 10),
     "rpa_ragged_paged_attention_v3_quantised": (
         _c_int,
-        [_c_vp] * 12 + [_c_sz] + [_c_int] * 12 + [_c_f32, _c_int, _c_f32],
+        [_c_vp] * 12 + [_c_sz] + [_c_int] * 12 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
     "rpa_unified_attention": (
         _c_int,
-        [_c_vp] * 11 + [_c_sz] + [_c_int] * 10 + [_c_f32, _c_int, _c_f32],
+        [_c_vp] * 11 + [_c_sz] + [_c_int] * 10 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
     "rpa_ragged_paged_attention_v3": (
         _c_int,
-        [_c_vp] * 11 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32],
+        [_c_vp] * 11 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
 }
 

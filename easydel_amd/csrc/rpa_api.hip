@@ -218,7 +218,8 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
                           const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
                           const int32_t* num_seqs, bool num_seqs_optional, void* out, void* workspace,
                           size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
-                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap) {
+                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
+                          const float* softmax_aux) {
   if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (T=%d S=%d M=%d P=%d page_size=%d Hq=%d Hkv=%d D=%d)", who,
                 T, S, M, P, page_size, Hq, Hkv, D);
@@ -231,13 +232,15 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   if (kv_scales && ((uintptr_t)kv_scales & 7))
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: kv_scales must be 8-byte aligned", who);
   if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_scale is not finite", who);
+  if (softmax_aux && ((uintptr_t)softmax_aux & 3))
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_aux must be 4-byte aligned", who);
   if (T == 0) return RPA_OK;
   if (!q || !k_pages || !v_pages || !context_lens || !block_tables || !query_start_loc || (!num_seqs && !num_seqs_optional) || !out)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
 
   rpa::AttnParams p;
   memset(&p, 0, sizeof(p));
-  p.q = q; p.k_pages = k_pages; p.v_pages = v_pages; p.kv_scales = kv_scales;
+  p.q = q; p.k_pages = k_pages; p.v_pages = v_pages; p.kv_scales = kv_scales; p.sinks = softmax_aux;
   p.context_lens = context_lens; p.block_tables = block_tables; p.qsl = query_start_loc; p.num_seqs = num_seqs;
   p.out = out;
   p.T = T; p.S = S; p.M = M; p.P = P; p.page_size = page_size; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv; p.D = D; p.C = C;
@@ -307,7 +310,7 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
                                const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
                                size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv,
                                int D, int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
-                               float logits_soft_cap) {
+                               float logits_soft_cap, const float* softmax_aux) {
   if (Hkv > 0 && C < 2 * Hkv)
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: C=%d combined heads < 2*Hkv=%d", C, 2 * Hkv);
   // interleaved pages: K of head h in combined head 2h, V in 2h+1, one row of D elements each
@@ -315,19 +318,22 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
   const void* v_pages = kv_pages ? (const char*)kv_pages + row : nullptr;
   return attention_impl("rpa_ragged_paged_attention", stream, q, kv_pages, v_pages, (int64_t)C * row, 2 * row, kv_scales,
                         context_lens, block_tables, query_start_loc, num_seqs, false, out, workspace, workspace_bytes, T, S,
-                        M, P, page_size, Hq, Hkv, D, C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+                        M, P, page_size, Hq, Hkv, D, C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap,
+                        softmax_aux);
 }
 
 int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_cache, const void* value_cache,
                           const float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
                           const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
                           size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D,
-                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap) {
+                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
+                          const float* softmax_aux) {
   // separate pools [P][page_size][Hkv][D]: heads one row apart, tokens Hkv rows apart
   const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
   return attention_impl("rpa_unified_attention", stream, q, key_cache, value_cache, (int64_t)Hkv * row, row, kv_scales,
                         context_lens, block_tables, query_start_loc, num_seqs, true, out, workspace, workspace_bytes, T, S, M,
-                        P, page_size, Hq, Hkv, D, 2 * Hkv, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+                        P, page_size, Hq, Hkv, D, 2 * Hkv, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap,
+                        softmax_aux);
 }
 
 int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void* key, const void* value,
@@ -335,7 +341,7 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   const int32_t* query_start_loc, const int32_t* distribution, void* out,
                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P, int page_size,
                                   int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype, float softmax_scale,
-                                  int sliding_window, float logits_soft_cap) {
+                                  int sliding_window, float logits_soft_cap, const float* softmax_aux) {
   if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16)
     return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention_v3: quantised pages are read-only (kv_dtype %d)", kv_dtype);
   if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention_v3: null distribution");
@@ -345,7 +351,7 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
   if (err) return err;
   return rpa_ragged_paged_attention(stream, q, kv_pages, nullptr, context_lens, block_tables, query_start_loc, n_live,
                                     out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
-                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux);
 }
 
 int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, const void* key, const void* value,
@@ -354,7 +360,8 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
                                             const int32_t* distribution, void* out, void* workspace,
                                             size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq,
                                             int Hkv, int D, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
-                                            float softmax_scale, int sliding_window, float logits_soft_cap) {
+                                            float softmax_scale, int sliding_window, float logits_soft_cap,
+                                            const float* softmax_aux) {
   if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention_v3_quantised: null distribution");
   const int32_t* n_live = distribution + 2;
   int err = rpa_page_scatter_ragged_quantised(stream, key, value, kv_pages, kv_scales, context_lens, block_tables,
@@ -362,7 +369,7 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
   if (err) return err;
   return rpa_ragged_paged_attention(stream, q, kv_pages, kv_scales, context_lens, block_tables, query_start_loc, n_live,
                                     out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
-                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap);
+                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux);
 }
 
 }  // extern "C"

@@ -353,7 +353,8 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     const int tok_out = cur.q0 + r_tok;
     const int head_out = h * G + r_head;
     if (cur.single) {
-      const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
+      const float l_fin = with_sink(p, head_out, m_run, l_tot);
+      const float inv = (l_fin > 0.f ? 1.f / l_fin : 0.f) * v_unit;
       uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D;
       if constexpr (EB == 2) {
 #pragma unroll

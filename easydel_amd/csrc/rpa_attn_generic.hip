@@ -90,6 +90,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
       }
     }
   }
+  if (p.sinks && l > 0.f) l += expf(p.sinks[hq] - m);  // attention sink: one more logit in the denominator only
   const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
   for (int k = 0; k < 4; ++k) {

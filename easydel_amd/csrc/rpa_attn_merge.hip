@@ -74,6 +74,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    l = with_sink(p, hq, m_use, l);  // the pieces carry key sums only; the sink joins the denominator once, here
     inv = l > 0.f ? 1.f / l : 0.f;
   }
 #pragma unroll

@@ -303,7 +303,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
     l_tot += __shfl_xor(l_tot, 32);
     if (row_ok[rb]) {
       if (single) {
-        const float inv = (l_tot > 0.f ? 1.f / l_tot : 0.f) * v_unit;
+        const float l_fin = with_sink(p, out_head[rb], m_run[rb], l_tot);
+        const float inv = (l_fin > 0.f ? 1.f / l_fin : 0.f) * v_unit;
         uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j

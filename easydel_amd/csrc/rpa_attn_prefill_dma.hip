@@ -461,7 +461,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     const float l_tot = l_acc[rb][0];
     if (row_ok[rb]) {
       if (single) {
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        const float l_fin = with_sink(p, out_head[rb], m_run[rb], l_tot);
+        const float inv = l_fin > 0.f ? 1.f / l_fin : 0.f;
         uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j

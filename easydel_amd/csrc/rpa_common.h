@@ -22,6 +22,7 @@ struct AttnParams {
   const void* v_pages;     // V likewise.  Interleaved pages: v_pages = k_pages + one row, head_stride = two rows;
                            // separate K and V pools: two allocations, head_stride = one row
   const float* kv_scales;  // [P][C] or null
+  const float* sinks;      // [Hq] attention-sink logits (natural-log units, not scaled, not soft-capped) or null
   const int32_t* context_lens;
   const int32_t* block_tables;
   const int32_t* qsl;
@@ -86,6 +87,15 @@ __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
 }
 
 __device__ __forceinline__ int live_rows(const AttnParams& p) { return p.num_seqs ? p.num_seqs[0] : p.S; }
+
+// Attention sinks: the softmax of query head hq runs over the keys and one more logit, sinks[hq], whose
+// probability is then dropped -- a key with that score and a zero value row.  Only the denominator changes:
+// given l = sum over keys of exp2(score - m_log2), for any reference m_log2 common to the row (log2 units),
+// this returns l + exp2(sinks[hq]*log2(e) - m_log2).  Rows that see no key (l == 0) keep their zero output.
+__device__ __forceinline__ float with_sink(const AttnParams& p, int hq, float m_log2, float l) {
+  if (p.sinks == nullptr || !(l > 0.f)) return l;
+  return l + __builtin_amdgcn_exp2f(__builtin_fmaf(p.sinks[hq], 1.4426950408889634f, -m_log2));
+}
 
 // Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + kPrefillRows) of a sequence) must visit, kv_lo
 // rounded down to 64, and the number of split-K chunks the prefill kernel cuts it into.

@@ -143,6 +143,21 @@ def page_scatter_ragged_quantised(key, value, kv_pages, kv_scales, context_lens,
     return kv_pages, kv_scales
 
 
+def _sinks(softmax_aux, num_q_heads: int, device):
+    """Attention-sink logits as the library takes them: float32 ``[Hq]`` on the query's device (the reference
+    casts them to float32 and shards them by head, easydel/operations/kernels/ragged_page_attention.py:469-471).
+    Returns ``(tensor kept alive by the caller, pointer)``; ``(None, None)`` without sinks."""
+    if softmax_aux is None:
+        return None, None
+    if softmax_aux.ndim != 1 or softmax_aux.shape[0] != num_q_heads:
+        raise NotImplementedError(f"softmax_aux must hold one sink logit per query head, shape [{num_q_heads}]; "
+                                  f"got {tuple(softmax_aux.shape)}")
+    if softmax_aux.device != device:
+        raise ValueError(f"softmax_aux is on {softmax_aux.device}, the query on {device}")
+    aux = softmax_aux.detach().to(torch.float32).contiguous()
+    return aux, _dev(aux, "softmax_aux")
+
+
 def _attn_common(query, kv_pages, context_lens, block_tables, num_kv_heads, softmax_scale, sliding_window, logits_soft_cap):
     T, Hq, D = query.shape
     P, pg, C = page_geometry(kv_pages, D)
@@ -159,7 +174,7 @@ def _attn_common(query, kv_pages, context_lens, block_tables, num_kv_heads, soft
 
 def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *,
                            softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_scales=None,
-                           num_kv_heads=None, out=None):
+                           num_kv_heads=None, softmax_aux=None, out=None):
     """Read-only ragged paged attention; returns ``[T, Hq, D]`` in the query dtype."""
     lib = _lib.load()
     T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
@@ -171,6 +186,7 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
     qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
     for name, t in (("query", query), ("kv_pages", kv_pages), ("out", out)):
         _dev(t, name)
+    aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
     scales_ptr = None
     if kv_scales is not None:
@@ -181,12 +197,13 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
         _stream(query), _dev(query, "query"), _dev(kv_pages, "kv_pages"), scales_ptr,
         _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
         _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap))
+        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
     return out
 
 
 def unified_attention(query, key_cache, value_cache, context_lens, block_tables, query_start_loc, num_seqs=None, *,
-                      softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_scales=None, out=None):
+                      softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_scales=None, softmax_aux=None,
+                      out=None):
     """Ragged paged attention over separate K and V pools ``[P, page_size, Hkv, D]`` (the reference's
     unified-attention layout).  ``num_seqs`` is optional: without it every row of ``context_lens`` is live."""
     lib = _lib.load()
@@ -213,6 +230,7 @@ def unified_attention(query, key_cache, value_cache, context_lens, block_tables,
     qd, kd = dtype_tag(query.dtype), dtype_tag(key_cache.dtype)
     for name, t in (("query", query), ("key_cache", key_cache), ("value_cache", value_cache), ("out", out)):
         _dev(t, name)
+    aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
     scales_ptr = None
     if kv_scales is not None:
@@ -223,12 +241,13 @@ def unified_attention(query, key_cache, value_cache, context_lens, block_tables,
         _stream(query), _dev(query, "query"), _dev(key_cache, "key_cache"), _dev(value_cache, "value_cache"), scales_ptr,
         _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
         None if num_seqs is None else _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-        T, S, M, P, pg, Hq, Hkv, D, qd, kd, scale, window, cap))
+        T, S, M, P, pg, Hq, Hkv, D, qd, kd, scale, window, cap, aux_ptr))
     return out
 
 
 def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_tables, query_start_loc, distribution, *,
-                              softmax_scale=None, sliding_window=None, logits_soft_cap=None, num_kv_heads=None, out=None):
+                              softmax_scale=None, sliding_window=None, logits_soft_cap=None, num_kv_heads=None,
+                              softmax_aux=None, out=None):
     """Fused scatter + attention; updates ``kv_pages`` in place and returns ``(out, kv_pages)``."""
     lib = _lib.load()
     if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
@@ -243,18 +262,19 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
     qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
     for name, t in (("query", query), ("key", key), ("value", value), ("kv_pages", kv_pages), ("out", out)):
         _dev(t, name)
+    aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
     _lib.check(lib.rpa_ragged_paged_attention_v3(
         _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
         _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
         _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap))
+        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
     return out, kv_pages
 
 
 def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, context_lens, block_tables,
                                         query_start_loc, distribution, *, softmax_scale=None, sliding_window=None,
-                                        logits_soft_cap=None, num_kv_heads=None, out=None):
+                                        logits_soft_cap=None, num_kv_heads=None, softmax_aux=None, out=None):
     """Fused quantising write + attention over scaled 8-bit pages; updates ``kv_pages`` and ``kv_scales`` in place
     and returns ``(out, kv_pages, kv_scales)``.  ``key`` / ``value`` are float32 or bfloat16."""
     lib = _lib.load()
@@ -272,10 +292,11 @@ def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, 
     qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
     for name, t in (("query", query), ("key", key), ("value", value), ("kv_pages", kv_pages), ("kv_scales", kv_scales), ("out", out)):
         _dev(t, name)
+    aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
     _lib.check(lib.rpa_ragged_paged_attention_v3_quantised(
         _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
         _dev(kv_scales, "kv_scales"), _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"),
         _i32(query_start_loc, "query_start_loc"), _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(),
-        ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap))
+        ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap, aux_ptr))
     return out, kv_pages, kv_scales

@@ -4,7 +4,8 @@ Drop-in for the reference's ``easydel/operations/kernels/ragged_page_attention.p
 registry names, call signature (``query, key, value, cache_view, cache_metadata, softmax_scale,
 logits_soft_cap, sliding_window`` plus swallowed extras), 4-D <-> ragged reshape (:881-918), cast of K/V to
 the cache dtype with a warning when it narrows (:570-580), write-back of the updated pages into the view
-(:747) and ``AttentionOutput`` result.  Where the reference hands the arrays to ``ejkernel`` (:281-313,
+(:747), ``softmax_aux`` attention sinks (one logit per query head, cast to float32 as at :469-471) and
+``AttentionOutput`` result.  Where the reference hands the arrays to ``ejkernel`` (:281-313,
 :732-746), this module hands device pointers to ``librpa_hip.so`` through ``easydel_amd.kernels``.
 """
 
@@ -46,21 +47,18 @@ class _RaggedPageAttn(OperationImpl):
                    softmax_scale: float | None = None, logits_soft_cap: float | None = None, compute_dtype=None,
                    optimized: bool = False, sliding_window: int | None = None, softmax_aux=None,
                    mask_value: float | None = None, vmem_limit_bytes: int | None = None, **ignore) -> AttentionOutput:
-        if softmax_aux is not None:
-            raise NotImplementedError("attention sinks (softmax_aux) are not implemented by the ROCm ragged-page kernels")
         output = kernels.ragged_paged_attention(
             query, cache_view.kv_pages, cache_metadata.context_lens, cache_metadata.pages_tables,
             cache_metadata.query_start_loc, cache_metadata.num_seqs.reshape(-1), softmax_scale=softmax_scale,
             sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
-            kv_scales=getattr(cache_view, "kv_scales", None), num_kv_heads=_num_kv_heads(cache_view))
+            kv_scales=getattr(cache_view, "kv_scales", None), num_kv_heads=_num_kv_heads(cache_view),
+            softmax_aux=softmax_aux)
         return AttentionOutput(attention_weights=None, attention_outputs=output)
 
     # -- v3: fused page write + attention ------------------------------------------------------------------
     def forward_v3(self, query, key, value, cache_view: RaggedPagesCacheView, cache_metadata: RaggedPagesMetadata,
                    softmax_scale: float | None = None, logits_soft_cap: float | None = None,
                    sliding_window: int | None = None, softmax_aux=None, **ignore) -> AttentionOutput:
-        if softmax_aux is not None:
-            raise NotImplementedError("attention sinks (softmax_aux) are not implemented by the ROCm ragged-page kernels")
         kv_pages = cache_view.kv_pages
         if getattr(cache_view, "kv_scales", None) is not None:
             # scaled 8-bit pages: the write quantises (per page and head the scale only grows), then the attention
@@ -70,7 +68,7 @@ class _RaggedPageAttn(OperationImpl):
                     query, kv_pages, cache_metadata.context_lens, cache_metadata.pages_tables.reshape(-1),
                     cache_metadata.query_start_loc, cache_metadata.request_distribution[2:3], softmax_scale=softmax_scale,
                     sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, kv_scales=cache_view.kv_scales,
-                    num_kv_heads=_num_kv_heads(cache_view))
+                    num_kv_heads=_num_kv_heads(cache_view), softmax_aux=softmax_aux)
                 return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
             if key.dtype not in (torch.float32, torch.bfloat16):
                 key, value = key.to(torch.float32), value.to(torch.float32)
@@ -78,7 +76,7 @@ class _RaggedPageAttn(OperationImpl):
                 query, key.contiguous(), value.to(key.dtype).contiguous(), kv_pages, cache_view.kv_scales,
                 cache_metadata.context_lens, cache_metadata.pages_tables.reshape(-1), cache_metadata.query_start_loc,
                 cache_metadata.request_distribution, softmax_scale=softmax_scale, sliding_window=sliding_window,
-                logits_soft_cap=logits_soft_cap, num_kv_heads=_num_kv_heads(cache_view))
+                logits_soft_cap=logits_soft_cap, num_kv_heads=_num_kv_heads(cache_view), softmax_aux=softmax_aux)
             cache_view.kv_pages, cache_view.kv_scales = kv_pages, kv_scales
             return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
         if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
@@ -90,7 +88,8 @@ class _RaggedPageAttn(OperationImpl):
         output, kv_pages = kernels.ragged_paged_attention_v3(
             query, key.contiguous(), value.contiguous(), kv_pages, cache_metadata.context_lens,
             cache_metadata.pages_tables.reshape(-1), cache_metadata.query_start_loc, cache_metadata.request_distribution,
-            softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap)
+            softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
+            softmax_aux=softmax_aux)
         cache_view.kv_pages = kv_pages
         return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
 

@@ -43,8 +43,6 @@ class UnifiedAttn(OperationImpl):
             raise ValueError("UnifiedAttn requires `cache_view` (paged KV cache).")
         if not causal:
             raise NotImplementedError("the paged attention kernels are causal-only, as the reference's kernel is")
-        if softmax_aux is not None:
-            raise NotImplementedError("attention sinks (softmax_aux) are not implemented by the ROCm paged-attention kernels")
         is_4d = query.ndim == 4
         shape4 = tuple(query.shape) if is_4d else None
         query_ragged = query.reshape(-1, *query.shape[-2:]).contiguous()
@@ -53,7 +51,7 @@ class UnifiedAttn(OperationImpl):
         out = kernels.unified_attention(
             query_ragged, cache_view.key_cache, cache_view.value_cache, cache_metadata.context_lens,
             cache_metadata.pages_tables, cache_metadata.query_start_loc, None, softmax_scale=softmax_scale,
-            sliding_window=sliding_window, logits_soft_cap=logits_soft_cap)
+            sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, softmax_aux=softmax_aux)
         if is_4d:
             out = out.reshape(shape4)
         return AttentionOutput(attention_weights=None, attention_outputs=out, cache_view=cache_view)

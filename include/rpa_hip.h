@@ -132,6 +132,12 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
  *   softmax_scale                            multiplies q.k before the soft cap
  *   sliding_window                           <= 0: none; W: key j visible iff pos-W < j <= pos
  *   logits_soft_cap                          <= 0: none; cap: s = cap*tanh(s/cap)
+ *   softmax_aux   device, float [Hq] or NULL: attention sinks, the reference's softmax_aux
+ *                 (ragged_page_attention.py:469-471, :590-592: one float32 logit per query head).  The softmax of
+ *                 head hq runs over the visible keys and the extra logit softmax_aux[hq] (taken as is: no
+ *                 softmax_scale, no soft cap), whose probability is then dropped, so the weights of a row sum to
+ *                 less than one: out = sum_j exp(s_j) v_j / (sum_j exp(s_j) + exp(softmax_aux[hq])).  This is the
+ *                 GPT-OSS definition the reference's model file feeds (modules/gpt_oss/modeling_gpt_oss.py:436-442).
  * Query row r of sequence i sits at position ctx_i - q_len_i + r and attends causally.
  */
 int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages,
@@ -140,7 +146,7 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
                                const int32_t* num_seqs, void* out, void* workspace, size_t workspace_bytes,
                                int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
                                int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
-                               float logits_soft_cap);
+                               float logits_soft_cap, const float* softmax_aux);
 
 /*
  * The same attention over separate K and V pools: key_cache and value_cache are each
@@ -159,7 +165,8 @@ int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_ca
                           const float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
                           const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
                           size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D,
-                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap);
+                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
+                          const float* softmax_aux);
 
 /*
  * Fused v3 form: rpa_page_scatter_ragged followed by rpa_ragged_paged_attention on the
@@ -173,7 +180,8 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   const int32_t* query_start_loc, const int32_t* distribution, void* out,
                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P,
                                   int page_size, int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype,
-                                  float softmax_scale, int sliding_window, float logits_soft_cap);
+                                  float softmax_scale, int sliding_window, float logits_soft_cap,
+                                  const float* softmax_aux);
 
 /*
  * Fused v3 form over scaled 8-bit pages: rpa_page_scatter_ragged_quantised followed by
@@ -185,7 +193,8 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
                                             const int32_t* distribution, void* out, void* workspace,
                                             size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq,
                                             int Hkv, int D, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
-                                            float softmax_scale, int sliding_window, float logits_soft_cap);
+                                            float softmax_scale, int sliding_window, float logits_soft_cap,
+                                  const float* softmax_aux);
 
 /*
  * Measurement aid with no counterpart in the reference: copies `bytes` (a multiple of 16, both

@@ -33,7 +33,10 @@ Pinning status
   "parity unpinned" against ejkernel.  The residual conventions that only an
   import of ejkernel could confirm (where its XLA path rounds to bf16, what it
   writes to padded rows, the mask value of fully masked rows) are covered by
-  comparing valid rows only, at the stated tolerances.
+  comparing valid rows only, at the stated tolerances.  Its ``softmax_aux`` (attention sinks) arm is
+  likewise unpinned against ejkernel; it is pinned to the published GPT-OSS attention (the
+  ``transformers`` library's eager implementation, run on dense inputs) and to the closed form
+  ``out = out_without_sink * sigmoid(logsumexp(scores) - sink)``.
 * ``page_scatter_ragged_ref`` (the fused v3 write): no reference vector exists
   (it runs inside ejkernel); pinned by equivalence with the v2 scatter driven by
   ``slot_mapping_v2_ref`` on the same batch.
@@ -339,7 +342,7 @@ def page_scatter_ragged_quantised_ref(key, value, kv_codes, kv_scales, context_l
 
 def ragged_paged_attention_ref(query, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *,
                                softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_scales=None,
-                               num_kv_heads=None) -> np.ndarray:
+                               num_kv_heads=None, softmax_aux=None) -> np.ndarray:
     """Ragged paged attention in float64 (operation called at ragged_page_attention.py:281-313 / 732-746).
 
     ``query [T, Hq, D]`` and ``kv_pages [P, pg, C, D]`` are *decoded values* (float arrays).  Conventions, each
@@ -352,6 +355,11 @@ def ragged_paged_attention_ref(query, kv_pages, context_lens, block_tables, quer
         (``W`` keys including self; single_type_cache_manager.py:497)
       * ``softmax_scale=None`` means ``D**-0.5``                                       (ragged_page_attention.py:784)
       * ``kv_scales [P, C]`` (this build's quantised-page format): value = code * scale[page, combined head].
+      * ``softmax_aux [Hq]``: attention sinks, one logit per query head, float32
+        (ragged_page_attention.py:469-471, fed by modules/gpt_oss/modeling_gpt_oss.py:436-442).  The sink
+        arithmetic lives in ejkernel; restated here is the published GPT-OSS definition that parameter belongs
+        to: the softmax runs over ``[scores, sink]`` and the sink's column is dropped, so the sink enters the
+        denominator only, as is (no scale, no soft cap, never masked).
     Rows of padded tokens (``t >= qsl[num_seqs]``) and of sequences with ``q_len == 0`` are returned as zeros.
     """
     q = np.asarray(query, dtype=np.float64)
@@ -363,6 +371,11 @@ def ragged_paged_attention_ref(query, kv_pages, context_lens, block_tables, quer
     scale = float(d) ** -0.5 if softmax_scale is None else float(softmax_scale)
     bt = np.asarray(block_tables).reshape(len(context_lens), -1)
     out = np.zeros((n_tok, hq, d), dtype=np.float64)
+    sinks = None
+    if softmax_aux is not None:
+        sinks = np.asarray(softmax_aux, dtype=np.float64).reshape(-1)
+        if sinks.shape[0] != hq:
+            raise ValueError(f"softmax_aux must hold one logit per query head ({hq}), got {sinks.shape[0]}")
     for i in range(int(np.asarray(num_seqs).reshape(-1)[0])):
         q0, q1 = int(query_start_loc[i]), int(query_start_loc[i + 1])
         ctx, q_len = int(context_lens[i]), q1 - q0
@@ -387,8 +400,12 @@ def ragged_paged_attention_ref(query, kv_pages, context_lens, block_tables, quer
                 s = float(logits_soft_cap) * np.tanh(s / float(logits_soft_cap))
             s = np.where(visible, s, -np.inf)
             m = s.max(axis=1, keepdims=True)
+            if sinks is not None:
+                m = np.maximum(m, sinks[h])
             m = np.where(np.isfinite(m), m, 0.0)
             p = np.exp(s - m)
             denom = p.sum(axis=1, keepdims=True)
+            if sinks is not None:
+                denom = denom + np.exp(sinks[h] - m)
             out[q0:q1, h, :] = (p @ v) / np.where(denom > 0, denom, 1.0)
     return out

@@ -102,11 +102,11 @@ def make_batch(seed, ctx_lens, q_lens, *, Hq, Hkv, D, page_size, num_pages=None,
     return b
 
 
-def oracle_out(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_val=None):
+def oracle_out(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_val=None, softmax_aux=None):
     return orc.ragged_paged_attention_ref(
         b.q_val, b.kv_val if kv_val is None else kv_val, b.context_lens, b.block_tables, b.query_start_loc, b.num_seqs,
         softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
-        kv_scales=b.kv_scales, num_kv_heads=b.Hkv)
+        kv_scales=b.kv_scales, num_kv_heads=b.Hkv, softmax_aux=softmax_aux)
 
 
 # ---- torch plumbing (imported lazily so the CPU-only tests need no GPU) ---------------------------
@@ -148,14 +148,21 @@ def device_batch(b, device="cuda:0"):
     return d
 
 
-def run_gpu_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, device="cuda:0"):
+def _aux_to_device(softmax_aux, device):
+    import torch
+
+    return None if softmax_aux is None else torch.from_numpy(np.asarray(softmax_aux, dtype=np.float32)).to(device)
+
+
+def run_gpu_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, device="cuda:0",
+                      softmax_aux=None):
     from easydel_amd import kernels
 
     d = device_batch(b, device)
     out = kernels.ragged_paged_attention(
         d["query"], d["kv_pages"], d["context_lens"], d["block_tables"], d["query_start_loc"], d["num_seqs"],
         softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap,
-        kv_scales=d["kv_scales"], num_kv_heads=b.Hkv)
+        kv_scales=d["kv_scales"], num_kv_heads=b.Hkv, softmax_aux=_aux_to_device(softmax_aux, device))
     import torch
 
     torch.cuda.synchronize()
@@ -163,7 +170,7 @@ def run_gpu_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft
 
 
 def run_gpu_unified_attention(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, device="cuda:0",
-                              pass_num_seqs=True):
+                              pass_num_seqs=True, softmax_aux=None):
     """The same batch with its pages split into separate K and V pools ``[P, pg, Hkv, D]``."""
     import torch
 
@@ -175,7 +182,7 @@ def run_gpu_unified_attention(b, *, softmax_scale=None, sliding_window=None, log
     out = kernels.unified_attention(
         d["query"], key_cache, value_cache, d["context_lens"], d["block_tables"], d["query_start_loc"],
         d["num_seqs"] if pass_num_seqs else None, softmax_scale=softmax_scale, sliding_window=sliding_window,
-        logits_soft_cap=logits_soft_cap, kv_scales=d["kv_scales"])
+        logits_soft_cap=logits_soft_cap, kv_scales=d["kv_scales"], softmax_aux=_aux_to_device(softmax_aux, device))
     torch.cuda.synchronize()
     return from_torch(out, b.q_dtype)
 

@@ -33,13 +33,13 @@ def test_host_only_entry_points():
     assert re.fullmatch(r"\d+\.\d+\.\d+", lib.rpa_version().decode())
     # argument validation happens before any device work
     rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
-                                        4, 1, 1, 1, 16, 8, 3, 64, 6, 1, 1, 1.0, 0, 0.0)
+                                        4, 1, 1, 1, 16, 8, 3, 64, 6, 1, 1, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"multiple of Hkv" in lib.rpa_last_error()
     rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
-                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 5, 1, 1.0, 0, 0.0)
+                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 5, 1, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_UNSUPPORTED
     rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
-                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 2, 1.0, 0, 0.0)
+                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 2, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"kv_scales" in lib.rpa_last_error()
     with pytest.raises(_lib.RpaError):
         _lib.check(rc)

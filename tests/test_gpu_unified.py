@@ -118,7 +118,7 @@ def test_unified_operation_rejects_what_the_kernels_do_not_cover(gpu):
     cfg = UnifiedAttentionCacheConfig.create(torch.bfloat16, 1, 2, 64, 64, page_size=16, num_pages=4)
     view = UnifiedAttentionCacheView.init(cfg, device=gpu)
     meta = RaggedPagesMetadata.create_empty(2, 2, 4, page_size=16, version="v2", device=gpu)
-    with pytest.raises(NotImplementedError):
-        op(q, view, meta, softmax_aux=torch.zeros(2, device=gpu))
+    with pytest.raises(NotImplementedError, match="one sink logit per query head"):
+        op(q, view, meta, softmax_aux=torch.zeros(2, device=gpu))  # 8 query heads
     with pytest.raises(NotImplementedError):
         op(q, view, meta, causal=False)

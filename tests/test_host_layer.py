@@ -146,8 +146,14 @@ def test_product_path_refuses_cpu_tensors():
                                request_distribution=i32(0, 1, 1))
     with pytest.raises(RuntimeError, match="GPU memory"):
         RaggedPageAttnV3(OperationMetadata())(q[None], q[None, :, :2], q[None, :, :2], view, meta)
-    with pytest.raises(NotImplementedError, match="sinks"):
+    with pytest.raises(RuntimeError, match="GPU memory"):
         RaggedPageAttnV3(OperationMetadata())(q[None], q[None, :, :2], q[None, :, :2], view, meta, softmax_aux=torch.zeros(4))
+    # attention sinks: one logit per query head, anything else is refused by name
+    assert kernels._sinks(None, 4, torch.device("cpu")) == (None, None)
+    with pytest.raises(NotImplementedError, match="one sink logit per query head"):
+        kernels._sinks(torch.zeros(4, 2), 4, torch.device("cpu"))
+    with pytest.raises(NotImplementedError, match="one sink logit per query head"):
+        kernels._sinks(torch.zeros(8), 4, torch.device("cpu"))
 
 
 def test_page_geometry_views():

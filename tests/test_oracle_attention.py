@@ -173,3 +173,72 @@ def test_brute_force_scalar_loops_match():
                 for w, vv in ws:
                     acc += w / z * vv
                 np.testing.assert_allclose(got[t, h], acc, rtol=1e-12)
+
+
+# ---- attention sinks (softmax_aux) ------------------------------------------------------------------------------
+# The sink arithmetic is ejkernel's; the reference fixes only where the parameter comes from (the GPT-OSS model's
+# per-head `sinks`, modules/gpt_oss/modeling_gpt_oss.py:436-442) and how it is passed (float32, one logit per query
+# head, operations/kernels/ragged_page_attention.py:469-471).  These tests pin the oracle's restatement to the
+# published GPT-OSS attention and to what the mathematics fixes.
+
+
+def test_sinks_closed_form_scales_each_row_by_a_sigmoid():
+    # softmax over [scores, sink] with the sink column dropped = plain softmax times sigmoid(logsumexp(scores) - sink)
+    from scipy.special import expit, logsumexp
+    rng = np.random.default_rng(21)
+    n, hq, hkv, d = 11, 4, 2, 8
+    q = rng.standard_normal((n, hq, d)); k = rng.standard_normal((n, hkv, d)); v = rng.standard_normal((n, hkv, d))
+    sinks = rng.standard_normal(hq) * 2.0
+    pages = _dense_pages(k, v, 4, [5, 2, 7])
+    bt = np.array([[5, 2, 7]])
+    plain = orc.ragged_paged_attention_ref(q, pages, [n], bt, [0, n], [1], softmax_scale=0.4, sliding_window=6)
+    got = orc.ragged_paged_attention_ref(q, pages, [n], bt, [0, n], [1], softmax_scale=0.4, sliding_window=6, softmax_aux=sinks)
+    i, j = np.arange(n)[:, None], np.arange(n)[None, :]
+    vis = (j <= i) & (j > i - 6)
+    for h in range(hq):
+        s = np.where(vis, 0.4 * q[:, h] @ k[:, h // 2].T, -np.inf)
+        np.testing.assert_allclose(got[:, h], plain[:, h] * expit(logsumexp(s, axis=1) - sinks[h])[:, None], rtol=1e-12, atol=1e-14)
+
+
+def test_sinks_limits_and_row_weight():
+    b = tl.make_batch(22, [9, 30], [3, 1], Hq=4, Hkv=2, D=8, page_size=8, q_dtype=F32, kv_dtype=F32, pad_rows=1, pad_tokens=2)
+    plain = tl.oracle_out(b)
+    # a sink at -inf is no sink; a huge sink takes all the weight; padded rows stay zero
+    np.testing.assert_array_equal(tl.oracle_out(b, softmax_aux=np.full(4, -np.inf)), plain)
+    assert np.abs(tl.oracle_out(b, softmax_aux=np.full(4, 80.0))).max() < 1e-25
+    got = tl.oracle_out(b, softmax_aux=np.array([0.0, 1.0, -1.0, 3.0]))
+    assert (got[int(b.query_start_loc[b.n]):] == 0).all()
+    # with all values equal to one, a row's output is the weight its keys keep: 1 - P(sink) < 1, per head
+    ones = tl.make_batch(22, [9, 30], [3, 1], Hq=4, Hkv=2, D=8, page_size=8, q_dtype=F32, kv_dtype=F32, fill=1.0)
+    w = tl.oracle_out(ones, softmax_aux=np.array([0.0, 1.0, -1.0, 3.0]))[tl.valid_rows(ones)]
+    # equal keys: every score is the same s0, so the kept weight is n*e^s0 / (n*e^s0 + e^sink)
+    s0 = (ones.q_val.sum(axis=2) * 8 ** -0.5)[tl.valid_rows(ones)]
+    n_vis = np.array([7, 8, 9, 30])[:, None]
+    want = n_vis * np.exp(s0) / (n_vis * np.exp(s0) + np.exp(np.array([0.0, 1.0, -1.0, 3.0]))[None, :])
+    np.testing.assert_allclose(w[:, :, 0], want, rtol=1e-12)
+
+
+def test_sinks_match_the_published_gpt_oss_attention():
+    """Dense restatement through the `transformers` library's GPT-OSS eager attention (an installed third-party
+    package, the published definition of the parameter the reference's GPT-OSS module feeds into softmax_aux)."""
+    torch = pytest.importorskip("torch")
+    gpt_oss = pytest.importorskip("transformers.models.gpt_oss.modeling_gpt_oss")
+    from types import SimpleNamespace
+    rng = np.random.default_rng(23)
+    ctx, q_len, hq, hkv, d, window = 37, 9, 8, 2, 16, 12
+    k = rng.standard_normal((ctx, hkv, d)); v = rng.standard_normal((ctx, hkv, d)); q = rng.standard_normal((q_len, hq, d))
+    sinks = rng.standard_normal(hq) * 1.5
+    table = [4, 9, 1, 6, 3]
+    pages = _dense_pages(k, v, 8, table)
+    for win in (None, window):
+        got = orc.ragged_paged_attention_ref(q, pages, [ctx], np.array([table]), [0, q_len], [1], softmax_scale=0.25,
+                                             sliding_window=win, softmax_aux=sinks)
+        pos = ctx - q_len + np.arange(q_len)[:, None]
+        j = np.arange(ctx)[None, :]
+        vis = (j <= pos) & ((j > pos - win) if win else True)
+        mask = torch.from_numpy(np.where(vis, 0.0, -np.inf))[None, None]
+        module = SimpleNamespace(num_key_value_groups=hq // hkv, sinks=torch.from_numpy(sinks), training=False)
+        want, _ = gpt_oss.eager_attention_forward(
+            module, torch.from_numpy(q).permute(1, 0, 2)[None], torch.from_numpy(k).permute(1, 0, 2)[None],
+            torch.from_numpy(v).permute(1, 0, 2)[None], mask, scaling=0.25)
+        np.testing.assert_allclose(got, want[0].numpy(), rtol=1e-10, atol=1e-12)
