@@ -219,7 +219,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
                           const int32_t* num_seqs, bool num_seqs_optional, void* out, void* workspace,
                           size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
                           int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
-                          const float* softmax_aux) {
+                          const float* softmax_aux, const void* new_key = nullptr, const void* new_value = nullptr) {
   if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (T=%d S=%d M=%d P=%d page_size=%d Hq=%d Hkv=%d D=%d)", who,
                 T, S, M, P, page_size, Hq, Hkv, D);
@@ -262,6 +262,16 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
 
   hipStream_t s = (hipStream_t)stream;
   const int stages = g_stages.load();
+  if (new_key) {  // fused write + attention: the new rows go into the pages before any kernel reads them
+    if (p.mfma_path && (stages & 1)) {
+      p.new_k = new_key;  // copied by extra blocks of the decode plan kernel's launch
+      p.new_v = new_value;
+    } else {
+      const int err = rpa::launch_scatter_ragged(s, new_key, new_value, const_cast<void*>(k_pages), context_lens, block_tables,
+                                                 query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
+      if (err) return hip_fail(err, "page scatter launch");
+    }
+  }
   if (p.mfma_path) {
     const int td = decode_token_bound(T, S, Hq, Hkv);
     p.t_dec_max = td;
@@ -342,16 +352,18 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P, int page_size,
                                   int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype, float softmax_scale,
                                   int sliding_window, float logits_soft_cap, const float* softmax_aux) {
+  const char* who = "rpa_ragged_paged_attention_v3";
   if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16)
-    return fail(RPA_ERR_UNSUPPORTED, "rpa_ragged_paged_attention_v3: quantised pages are read-only (kv_dtype %d)", kv_dtype);
-  if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention_v3: null distribution");
+    return fail(RPA_ERR_UNSUPPORTED, "%s: quantised pages are read-only (kv_dtype %d)", who, kv_dtype);
+  if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null distribution", who);
+  if (Hkv > 0 && C < 2 * Hkv) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: C=%d combined heads < 2*Hkv=%d", who, C, 2 * Hkv);
+  if (T > 0 && (!key || !value)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null key / value", who);
   const int32_t* n_live = distribution + 2;
-  int err = rpa_page_scatter_ragged(stream, key, value, kv_pages, context_lens, block_tables, query_start_loc, n_live,
-                                    T, S, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
-  if (err) return err;
-  return rpa_ragged_paged_attention(stream, q, kv_pages, nullptr, context_lens, block_tables, query_start_loc, n_live,
-                                    out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
-                                    kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux);
+  const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
+  const void* v_pages = kv_pages ? (const char*)kv_pages + row : nullptr;
+  return attention_impl(who, stream, q, kv_pages, v_pages, (int64_t)C * row, 2 * row, nullptr, context_lens, block_tables,
+                        query_start_loc, n_live, false, out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C,
+                        q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux, key, value);
 }
 
 int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, const void* key, const void* value,

@@ -26,7 +26,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
   const int t = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
   const int n_live = live_rows(p);
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) return;
-  const int i = find_seq(p.qsl, n_live, t);
+  const int i = find_seq_wave(p.qsl, n_live, t);
   const SeqPlan sp = seq_plan(p, i);
   if (!sp.live) return;
   if (p.mfma_path && sp.small_rows) return;  // the MFMA decode kernel owns these rows

@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) {
     zero = true;
   } else {
-    const int i = find_seq(p.qsl, n_live, t);
+    const int i = find_seq_wave(p.qsl, n_live, t);  // one wave per (token, head): t is the same in all its lanes
     const SeqPlan sp = seq_plan(p, i);
     if (!sp.live) zero = true;
     else if (p.mfma_path && sp.small_rows) {

@@ -23,6 +23,8 @@ struct AttnParams {
                            // separate K and V pools: two allocations, head_stride = one row
   const float* kv_scales;  // [P][C] or null
   const float* sinks;      // [Hq] attention-sink logits (natural-log units, not scaled, not soft-capped) or null
+  const void* new_k;       // [T][Hkv][D] rows the decode plan kernel's launch also writes into the pages (fused v3
+  const void* new_v;       // call on the MFMA path), or null: the pages are read as they are
   const int32_t* context_lens;
   const int32_t* block_tables;
   const int32_t* qsl;
@@ -134,6 +136,65 @@ __device__ __forceinline__ int find_seq(const int32_t* qsl, int n, int t) {
   return lo;
 }
 
+// The same search by a whole wavefront whose 64 lanes (all active) ask for the same t: every round reads 64
+// entries spread evenly over what is left of the range with one load and keeps the sixty-fourth that holds the
+// answer, so up to 4096 sequences cost two dependent loads where the scalar search costs twelve.
+__device__ __forceinline__ int find_seq_wave(const int32_t* qsl, int n, int t) {
+  const int lane = threadIdx.x & 63;
+  int lo = 0, hi = n;  // invariant: qsl[lo] <= t < qsl[hi]
+  while (hi - lo > 1) {
+    const int stride = (hi - lo + 63) >> 6;
+    const int idx = lo + lane * stride;
+    const bool le = idx < hi && qsl[idx] <= t;  // true for a prefix of the lanes (lane 0 by the invariant)
+    const int last = __popcll(__ballot(le)) - 1;
+    lo += last * stride;
+    hi = min(lo + stride, hi);
+  }
+  return lo;
+}
+
+// New K/V rows of query token t into their page slot (the write half of the fused v3 operation): the token's
+// sequence i and position ctx_i - q_len_i + (t - q0_i) give the page and slot; K of head h goes to k_pages' row of
+// head h, V to v_pages'.  Called by every thread of a block with the same t; bit-exact copy of whole rows.
+__device__ __forceinline__ void scatter_token(const char* __restrict__ key, const char* __restrict__ value,
+                                              char* k_pages, char* v_pages, const int32_t* __restrict__ context_lens,
+                                              const int32_t* __restrict__ block_tables, const int32_t* __restrict__ qsl,
+                                              int n_live, int M, int P, int page_size, int Hkv, int head_bytes,
+                                              int64_t head_stride, int64_t token_stride, int64_t page_stride, int t) {
+  if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
+  const int i = find_seq_wave(qsl, n_live, t);
+  const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
+  const int pos = context_lens[i] - q_len + (t - q0);
+  if (pos < 0) return;
+  const int page_idx = pos / page_size;
+  if (page_idx >= M) return;
+  const int page = block_tables[(int64_t)i * M + page_idx];
+  if (page < 0 || page >= P) return;
+  const int64_t row = (int64_t)page * page_stride + (int64_t)(pos % page_size) * token_stride;
+  const char* ksrc = key + (int64_t)t * Hkv * head_bytes;
+  const char* vsrc = value + (int64_t)t * Hkv * head_bytes;
+  char* kdst = k_pages + row;
+  char* vdst = v_pages + row;
+  if ((head_bytes & 15) == 0 && ((((uintptr_t)kdst) | ((uintptr_t)vdst) | ((uintptr_t)ksrc) | ((uintptr_t)vsrc) | (uintptr_t)head_stride) & 15) == 0) {
+    const int vec_per_head = head_bytes >> 4;
+    const int n = 2 * Hkv * vec_per_head;
+    for (int k = threadIdx.x; k < n; k += blockDim.x) {
+      const int ch = k / vec_per_head, w = k - ch * vec_per_head;  // (head, K or V), vector within the row
+      const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
+      char* dst = ((ch & 1) ? vdst : kdst) + (int64_t)(ch >> 1) * head_stride;
+      ((uint4*)dst)[w] = ((const uint4*)src)[w];
+    }
+  } else {
+    const int n = 2 * Hkv * head_bytes;
+    for (int k = threadIdx.x; k < n; k += blockDim.x) {
+      const int ch = k / head_bytes, w = k - ch * head_bytes;
+      const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
+      char* dst = ((ch & 1) ? vdst : kdst) + (int64_t)(ch >> 1) * head_stride;
+      dst[w] = src[w];
+    }
+  }
+}
+
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
 
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {  // round to nearest even, NaN kept quiet
@@ -154,6 +215,7 @@ template <> struct ElemBytes<RPA_FP8_E4M3> { static constexpr int v = 1; };
 template <> struct ElemBytes<RPA_INT8> { static constexpr int v = 1; };
 
 inline int elem_bytes(int dt) { return dt == RPA_F32 ? 4 : dt == RPA_BF16 ? 2 : 1; }
+__device__ __forceinline__ int elem_bytes_dev(int dt) { return dt == RPA_F32 ? 4 : dt == RPA_BF16 ? 2 : 1; }
 
 template <int DT>
 __device__ __forceinline__ float load_elem(const void* base, int64_t idx) {

@@ -77,36 +77,9 @@ __global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restr
                                                              const int32_t* __restrict__ num_seqs, int M, int P,
                                                              int page_size, int Hkv, int head_bytes,
                                                              int64_t token_stride, int64_t page_stride) {
-  const int t = blockIdx.x;
-  const int n_live = num_seqs[0];
-  if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
-  const int i = find_seq(qsl, n_live, t);
-  const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
-  const int pos = context_lens[i] - q_len + (t - q0);
-  if (pos < 0) return;
-  const int page_idx = pos / page_size;
-  if (page_idx >= M) return;
-  const int page = block_tables[(int64_t)i * M + page_idx];
-  if (page < 0 || page >= P) return;
-  char* row = pages + (int64_t)page * page_stride + (int64_t)(pos % page_size) * token_stride;
-  const char* ksrc = key + (int64_t)t * Hkv * head_bytes;
-  const char* vsrc = value + (int64_t)t * Hkv * head_bytes;
-  if ((head_bytes & 15) == 0 && ((((uintptr_t)row) | ((uintptr_t)ksrc) | ((uintptr_t)vsrc)) & 15) == 0) {
-    const int vec_per_head = head_bytes >> 4;
-    const int n = 2 * Hkv * vec_per_head;
-    for (int k = threadIdx.x; k < n; k += blockDim.x) {
-      const int ch = k / vec_per_head, w = k - ch * vec_per_head;  // combined head, vector within head
-      const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
-      ((uint4*)(row + (int64_t)ch * head_bytes))[w] = ((const uint4*)src)[w];
-    }
-  } else {
-    const int n = 2 * Hkv * head_bytes;
-    for (int k = threadIdx.x; k < n; k += blockDim.x) {
-      const int ch = k / head_bytes, w = k - ch * head_bytes;
-      const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
-      row[(int64_t)ch * head_bytes + w] = src[w];
-    }
-  }
+  // interleaved pages: V of a head one row behind its K, heads two rows apart
+  scatter_token(key, value, pages, pages + head_bytes, context_lens, block_tables, qsl, num_seqs[0], M, P, page_size, Hkv,
+                head_bytes, 2 * (int64_t)head_bytes, token_stride, page_stride, blockIdx.x);
 }
 
 // ---- quantising ragged write ---------------------------------------------------------------------------
@@ -167,7 +140,7 @@ __global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __
   const int t = blockIdx.x, c = blockIdx.y, lane = threadIdx.x;
   const int n_live = num_seqs[0];
   if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
-  const int i = find_seq(qsl, n_live, t);
+  const int i = find_seq_wave(qsl, n_live, t);
   const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
   const int ctx = context_lens[i];
   const int pos = ctx - q_len + (t - q0);
