@@ -48,13 +48,15 @@ size_t part_o_bytes(int T, int Hq, int D) { return align256((size_t)T * Hq * D *
 size_t part_ml_bytes(int T, int Hq) { return align256((size_t)T * Hq * 2 * 4); }
 
 // Partial slots per sequence the workspace is sized for: enough to spread one maximal sequence over
-// 256-token pieces, capped so the partial buffers stay within ~256 MiB, never fewer than 2.
+// 256-token pieces, capped so the partial buffers stay within ~1 GiB, never fewer than 2.  (Too few slots force
+// long spans on every workgroup, so that one long sequence in a batch of short ones leaves most of the chip idle:
+// with a 256 MiB cap a 100k-token sequence among 255 short ones ran on 40 % of the workgroups.)
 int static_splits(int T, int M, int page_size, int Hq, int D) {
   const int forced = g_max_splits.load();
   if (forced > 0) return forced < 2 ? 2 : forced;
   long want = ((long)M * page_size + 255) / 256 + 1;
   const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
-  long cap = (long)(((size_t)256 << 20) / per);
+  long cap = (long)(((size_t)1 << 30) / per);
   if (cap > rpa::kMaxSplitsCap) cap = rpa::kMaxSplitsCap;
   if (want > cap) want = cap;
   if (want < 2) want = 2;
@@ -237,6 +239,8 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   if (T == 0) return RPA_OK;
   if (!q || !k_pages || !v_pages || !context_lens || !block_tables || !query_start_loc || (!num_seqs && !num_seqs_optional) || !out)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if ((((uintptr_t)q) | ((uintptr_t)out) | ((uintptr_t)k_pages) | ((uintptr_t)v_pages)) & 15)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: q, out and the page pools must be 16-byte aligned", who);
 
   rpa::AttnParams p;
   memset(&p, 0, sizeof(p));

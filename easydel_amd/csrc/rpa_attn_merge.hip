@@ -9,8 +9,12 @@
 
 namespace rpa {
 
-template <int QT>
-__global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
+
+// NK: output dims per lane (D <= 64 * NK)
+template <int QT, int NK>
+__global__ __launch_bounds__(256, 8) void attn_merge_kernel(AttnParams p) {
+  // partial rows in flight per wave: as many as leave the kernel within 64 registers, i.e. eight waves per SIMD
+  constexpr int kUnroll = NK == 4 ? 2 : 4;
   const int lane = threadIdx.x & 63;
   const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);  // (token, head) index
   if (pair >= p.T * p.Hq) return;
@@ -43,7 +47,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   const bool merge = n_pieces > 1;
   if (!zero && !merge) return;
 
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};  // dims lane, lane+64, lane+128, lane+192
+  float acc[NK];  // dims lane, lane+64, ...
+#pragma unroll
+  for (int k = 0; k < NK; ++k) acc[k] = 0.f;
   float inv = 0.f;
   if (merge) {
     const int64_t slot0 = (int64_t)part_row * p.Hq + hq;
@@ -62,11 +68,32 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
         l += w_c * ml.y;
       }
       const int cnt = min(64, n_pieces - base);
-      for (int c = 0; c < cnt; ++c) {
+      int c = 0;
+      // A row with hundreds of pieces (one long sequence spread over the whole chip leaves a piece per workgroup) is
+      // bound by the latency of these reads: kUnroll rows in flight at a time, accumulated in piece order as below.
+      for (; c + kUnroll <= cnt; c += kUnroll) {
+        float v[kUnroll][NK];
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const float* row = part_o + (slot0 + (base + c + u) * stride) * D;
+#pragma unroll
+          for (int k = 0; k < NK; ++k) {
+            const int d = lane + 64 * k;
+            v[u][k] = (d < D) ? row[d] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kUnroll; ++u) {
+          const float w = __shfl(w_c, c + u);
+#pragma unroll
+          for (int k = 0; k < NK; ++k) acc[k] = fmaf(w, v[u][k], acc[k]);
+        }
+      }
+      for (; c < cnt; ++c) {
         const float w = __shfl(w_c, c);
         const float* row = part_o + (slot0 + (base + c) * stride) * D;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
+        for (int k = 0; k < NK; ++k) {
           const int d = lane + 64 * k;
           if (d < D) acc[k] = fmaf(w, row[d], acc[k]);
         }
@@ -78,7 +105,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
     inv = l > 0.f ? 1.f / l : 0.f;
   }
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < NK; ++k) {
     const int d = lane + 64 * k;
     if (d < D) {
       const int64_t o = ((int64_t)t * p.Hq + hq) * D + d;
@@ -89,10 +116,17 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   }
 }
 
+template <int QT>
+static void launch_merge_q(hipStream_t stream, const AttnParams& p, int blocks) {
+  if (p.D <= 64) hipLaunchKernelGGL((attn_merge_kernel<QT, 1>), dim3(blocks), dim3(256), 0, stream, p);
+  else if (p.D <= 128) hipLaunchKernelGGL((attn_merge_kernel<QT, 2>), dim3(blocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((attn_merge_kernel<QT, 4>), dim3(blocks), dim3(256), 0, stream, p);
+}
+
 int launch_attn_merge(hipStream_t stream, const AttnParams& p) {
   const int blocks = (p.T * p.Hq + 3) / 4;
-  if (p.q_dtype == RPA_F32) hipLaunchKernelGGL((attn_merge_kernel<RPA_F32>), dim3(blocks), dim3(256), 0, stream, p);
-  else hipLaunchKernelGGL((attn_merge_kernel<RPA_BF16>), dim3(blocks), dim3(256), 0, stream, p);
+  if (p.q_dtype == RPA_F32) launch_merge_q<RPA_F32>(stream, p, blocks);
+  else launch_merge_q<RPA_BF16>(stream, p, blocks);
   return (int)hipGetLastError();
 }
 
