@@ -394,14 +394,17 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 
 // One block: exclusive prefix sum of the 64-token-rounded key spans of the decode-class sequences
 // (the flattened key stream), the per-workgroup span length Q, and each workgroup's first sequence.
-// With new_k / new_v set (the fused write + attention call), blocks 1 .. T of the same launch each copy one new
-// token's K/V rows into its page slot: the two jobs do not depend on each other, and the attention kernels that
-// follow on the stream see both.
+// With new_k / new_v set (the fused write + attention call), the blocks after the first copy the new tokens' K/V
+// rows into their page slots, one token per wavefront (16 per block): the two jobs do not depend on each other,
+// and the attention kernels that follow on the stream see both.
+constexpr int kScatterTokensPerBlock = 16;
 __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   if (blockIdx.x > 0) {
-    scatter_token((const char*)p.new_k, (const char*)p.new_v, (char*)p.k_pages, (char*)p.v_pages, p.context_lens,
-                  p.block_tables, p.qsl, live_rows(p), p.M, p.P, p.page_size, p.Hkv, p.D * elem_bytes_dev(p.kv_dtype),
-                  p.head_stride, p.token_stride, p.page_stride, (int)blockIdx.x - 1);
+    const int t = ((int)blockIdx.x - 1) * kScatterTokensPerBlock + (int)(threadIdx.x >> 6);
+    if (t < p.T)
+      scatter_token((const char*)p.new_k, (const char*)p.new_v, (char*)p.k_pages, (char*)p.v_pages, p.context_lens,
+                    p.block_tables, p.qsl, live_rows(p), p.M, p.P, p.page_size, p.Hkv, p.D * elem_bytes_dev(p.kv_dtype),
+                    p.head_stride, p.token_stride, p.page_stride, t, threadIdx.x & 63, 64);
     return;
   }
   __shared__ int part[1024], part2[1024];
@@ -490,7 +493,7 @@ static int launch_cap(hipStream_t stream, AttnParams p) {
   if (p.decode_wgs > 0) n_wg = p.decode_wgs;
   n_wg = max(1, min(n_wg, kMaxDecodeWgs));
   p.n_wg = n_wg;
-  if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + p.T : 1), dim3(1024), 0, stream, p);
+  if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + (p.T + kScatterTokensPerBlock - 1) / kScatterTokensPerBlock : 1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2)
     hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();

@@ -155,12 +155,14 @@ __device__ __forceinline__ int find_seq_wave(const int32_t* qsl, int n, int t) {
 
 // New K/V rows of query token t into their page slot (the write half of the fused v3 operation): the token's
 // sequence i and position ctx_i - q_len_i + (t - q0_i) give the page and slot; K of head h goes to k_pages' row of
-// head h, V to v_pages'.  Called by every thread of a block with the same t; bit-exact copy of whole rows.
+// head h, V to v_pages'.  Called with the same t by nthreads threads (whole wavefronts) numbered tid = 0 .. nthreads-1,
+// which share the copy; bit-exact copy of whole rows.
 __device__ __forceinline__ void scatter_token(const char* __restrict__ key, const char* __restrict__ value,
                                               char* k_pages, char* v_pages, const int32_t* __restrict__ context_lens,
                                               const int32_t* __restrict__ block_tables, const int32_t* __restrict__ qsl,
                                               int n_live, int M, int P, int page_size, int Hkv, int head_bytes,
-                                              int64_t head_stride, int64_t token_stride, int64_t page_stride, int t) {
+                                              int64_t head_stride, int64_t token_stride, int64_t page_stride, int t,
+                                              int tid, int nthreads) {
   if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
   const int i = find_seq_wave(qsl, n_live, t);
   const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
@@ -178,7 +180,7 @@ __device__ __forceinline__ void scatter_token(const char* __restrict__ key, cons
   if ((head_bytes & 15) == 0 && ((((uintptr_t)kdst) | ((uintptr_t)vdst) | ((uintptr_t)ksrc) | ((uintptr_t)vsrc) | (uintptr_t)head_stride) & 15) == 0) {
     const int vec_per_head = head_bytes >> 4;
     const int n = 2 * Hkv * vec_per_head;
-    for (int k = threadIdx.x; k < n; k += blockDim.x) {
+    for (int k = tid; k < n; k += nthreads) {
       const int ch = k / vec_per_head, w = k - ch * vec_per_head;  // (head, K or V), vector within the row
       const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
       char* dst = ((ch & 1) ? vdst : kdst) + (int64_t)(ch >> 1) * head_stride;
@@ -186,7 +188,7 @@ __device__ __forceinline__ void scatter_token(const char* __restrict__ key, cons
     }
   } else {
     const int n = 2 * Hkv * head_bytes;
-    for (int k = threadIdx.x; k < n; k += blockDim.x) {
+    for (int k = tid; k < n; k += nthreads) {
       const int ch = k / head_bytes, w = k - ch * head_bytes;
       const char* src = ((ch & 1) ? vsrc : ksrc) + (int64_t)(ch >> 1) * head_bytes;
       char* dst = ((ch & 1) ? vdst : kdst) + (int64_t)(ch >> 1) * head_stride;

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restr
                                                              int64_t token_stride, int64_t page_stride) {
   // interleaved pages: V of a head one row behind its K, heads two rows apart
   scatter_token(key, value, pages, pages + head_bytes, context_lens, block_tables, qsl, num_seqs[0], M, P, page_size, Hkv,
-                head_bytes, 2 * (int64_t)head_bytes, token_stride, page_stride, blockIdx.x);
+                head_bytes, 2 * (int64_t)head_bytes, token_stride, page_stride, blockIdx.x, threadIdx.x, blockDim.x);
 }
 
 // ---- quantising ragged write ---------------------------------------------------------------------------
