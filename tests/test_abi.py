@@ -43,6 +43,17 @@ def test_host_only_entry_points():
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"kv_scales" in lib.rpa_last_error()
     with pytest.raises(_lib.RpaError):
         _lib.check(rc)
+    # pointers are checked for null and alignment before anything is launched (the values below are never dereferenced)
+    a = 0x7000_0000_0000
+    rc = lib.rpa_ragged_paged_attention(None, a + 8, a, None, a, a, a, a, a, a, 1 << 20,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"16-byte aligned" in lib.rpa_last_error()
+    rc = lib.rpa_ragged_paged_attention(None, a, a, None, a, a, a, a, a, a, 1 << 20,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 1, 1.0, 0, 0.0, a + 2)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"softmax_aux" in lib.rpa_last_error()
+    rc = lib.rpa_ragged_paged_attention_v3(None, a, None, a, a, a, a, a, a, a, a, 1 << 20,
+                                           4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"null key" in lib.rpa_last_error()
     assert lib.rpa_page_scatter_slices(None, None, None, None, None, 0, 0, 0, 4, 16, 0) == 0  # empty input is a no-op
     assert lib.rpa_page_scatter_slices(None, None, None, None, None, 4, 4, 64, 0, 16, 0) == _lib.RPA_ERR_INVALID_ARGUMENT
     n = lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1)
