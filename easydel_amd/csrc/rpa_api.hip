@@ -103,11 +103,11 @@ void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, i
 
 size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + 2 * ((size_t)S + 1) + rpa::kMaxDecodeWgs) * 4); }
 
-// Static bound on query tokens the decode kernel can own: sequences with at most 16 rows per KV head.
-int decode_token_bound(int T, int S, int Hq, int Hkv) {
+// Static bound on query tokens the decode kernel can own: sequences with at most dec_rows rows per KV head.
+int decode_token_bound(int T, int S, int Hq, int Hkv, int dec_rows) {
   const int group = Hq / Hkv;
-  if (group > 16) return 1;
-  const long bound = (long)S * (16 / group);
+  if (group > dec_rows) return 1;
+  const long bound = (long)S * (dec_rows / group);
   return (int)(bound < T ? bound : T);
 }
 
@@ -201,10 +201,10 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
 
 size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int q_dtype,
                                      int kv_dtype) {
-  (void)q_dtype; (void)kv_dtype;
+  (void)q_dtype;
   if (T <= 0 || S <= 0 || M <= 0 || page_size <= 0 || Hq <= 0 || D <= 0) return 256;
   if (Hkv <= 0 || Hq % Hkv != 0) return 256;
-  const int td = decode_token_bound(T, S, Hq, Hkv);
+  const int td = decode_token_bound(T, S, Hq, Hkv, rpa::decode_row_limit(T, S, D, kv_dtype));
   const int splits = static_splits(td, M, page_size, Hq, D);
   int pre_keys, pre_chunks;
   prefill_split(T, S, M, page_size, Hq, Hkv, D, &pre_keys, &pre_chunks);
@@ -260,6 +260,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.decode_sync = g_decode_sync.load();
   p.prefill_dma = g_prefill_dma.load();
   p.max_splits = 2;
+  p.dec_rows = rpa::decode_row_limit(T, S, D, kv_dtype);
   p.pre_chunk = 1 << 30;
   p.pre_max_chunks = 1;
   p.mfma_path = (!g_force_generic.load() && rpa::decode_supported(p)) ? 1 : 0;
@@ -277,7 +278,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     }
   }
   if (p.mfma_path) {
-    const int td = decode_token_bound(T, S, Hq, Hkv);
+    const int td = decode_token_bound(T, S, Hq, Hkv, p.dec_rows);
     p.t_dec_max = td;
     const size_t po = part_o_bytes(td, Hq, D), pml = part_ml_bytes(td, Hq), pb = plan_bytes(S);
     int splits = static_splits(td, M, page_size, Hq, D);

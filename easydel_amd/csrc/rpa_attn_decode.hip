@@ -1,6 +1,6 @@
 // Split-K decode attention on MFMA, persistent and evenly split: one wavefront per KV head.
 //
-// Serves sequences whose query rows for one KV head (q_len * group) fit one 16-row MFMA block:
+// Serves sequences whose query rows for one KV head (q_len * group) fit one or two 16-row MFMA blocks:
 // plain decode (q_len = 1) and short speculative / multi-token rows.  The keys of all such
 // sequences are laid end to end (a small plan kernel computes the prefix sums on the device); each
 // of the resident workgroups takes one equal span of that stream, whatever sequence boundaries fall
@@ -60,7 +60,9 @@ __device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* 
   return pc;
 }
 
-template <int D, int KVT, int TT, int WPB, bool CAP>
+// RB: 16-row blocks of query rows one wave carries (rows of a sequence for one KV head: q_len * group <= 16 * RB).
+// Every K and V operand read from LDS feeds the MFMAs of all RB blocks.
+template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
@@ -141,28 +143,34 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   const int n_tiles = (cur.t_end - t_begin + TT - 1) / TT;
 
   // ---- per-lane row limits -------------------------------------------------------------
-  const int r_tok = (n < rows) ? n / G : 0;           // padded rows shadow row 0 and are never stored
-  const int r_head = (n < rows) ? n - r_tok * G : 0;
-  const int pos = cur.ctx - cur.q_len + r_tok;
-  const int row_hi = min(pos + 1, cur.ctx);            // exclusive
-  const int row_lo = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+  int r_tok[RB], r_head[RB], row_hi[RB], row_lo[RB];  // this lane's row of block rb is row n + 16 rb of the sequence
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int nr = n + 16 * rb;
+    r_tok[rb] = (nr < rows) ? nr / G : 0;               // padded rows shadow row 0 and are never stored
+    r_head[rb] = (nr < rows) ? nr - r_tok[rb] * G : 0;
+    const int pos = cur.ctx - cur.q_len + r_tok[rb];
+    row_hi[rb] = min(pos + 1, cur.ctx);                 // exclusive
+    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+  }
   const int vis_lo = (p.window > 0) ? max(cur.ctx - cur.q_len - p.window + 1, 0) : 0;  // lowest key any row sees
   // keys every row sees: from the last row's window start to the first row's causal limit
   const int all_lo = (p.window > 0) ? max(cur.ctx - p.window, 0) : 0;
   const int all_hi = cur.ctx - cur.q_len + 1;
 
   // ---- Q as B operands -----------------------------------------------------------------
-  bf16x8 qf[NKK];
-  {
-    const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok) * p.Hq + (h * G + r_head)) * D * 2;
+  bf16x8 qf[RB][NKK];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok[rb]) * p.Hq + (h * G + r_head[rb])) * D * 2;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
       // bf16 pages: step kk covers dims 32kk + 8g4 + e.  8-bit pages: a 16-byte K chunk holds 16
       // dims, so steps (2j, 2j+1) cover dims 64j + 16g4 + 8b + e.
       const int d0 = (EB == 2) ? (kk * 32 + 8 * g4) : ((kk >> 1) * 64 + 16 * g4 + 8 * (kk & 1));
       u32x4 v = {0u, 0u, 0u, 0u};
-      if (n < rows) v = *(const u32x4*)(qrow + d0 * 2);
-      qf[kk] = __builtin_bit_cast(bf16x8, v);
+      if (n + 16 * rb < rows) v = *(const u32x4*)(qrow + d0 * 2);
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
     }
   }
 
@@ -175,11 +183,16 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     page_nxt = page_of(nxt.i, nxt.t_begin);
   }
 
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run[RB], l_run[RB];
   float v_unit = 1.f;  // V scale the accumulators are currently expressed in (8-bit pages)
-  f32x4 o_acc[DPL];
+  f32x4 o_acc[RB][DPL];
 #pragma unroll
-  for (int rt = 0; rt < DPL; ++rt) o_acc[rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RB; ++rb) {
+    m_run[rb] = -INFINITY;
+    l_run[rb] = 0.f;
+#pragma unroll
+    for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
 
   // ---- registers -> LDS (zero rows past the context end or left of every row's window, so stale or
   //      null-page bytes cannot reach P.V as 0 * NaN)
@@ -205,10 +218,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     __builtin_amdgcn_wave_barrier();
 
     // ---- S^T = K . Q^T ----------------------------------------------------------------------
-    f32x4 s_acc[NS];
+    f32x4 s_acc[RB][NS];
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-      s_acc[st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) s_acc[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
       const int tk = st * 16 + n;  // this lane's A-operand row (token)
       const unsigned char* krow = lds_k + tk * RK;
       const int key = swz_key<RK>(tk);
@@ -216,36 +230,47 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 #pragma unroll
         for (int kk = 0; kk < NKK; ++kk) {
           const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
-          s_acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[kk], s_acc[st], 0, 0, 0);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < NKK / 2; ++j) {
           const u32x4 a = *(const u32x4*)(krow + (((j * 4 + g4) ^ key) << 4));
-          s_acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(codes8_to_bf16x8<KVT>(a[0], a[1]), qf[2 * j], s_acc[st], 0, 0, 0);
-          s_acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(codes8_to_bf16x8<KVT>(a[2], a[3]), qf[2 * j + 1], s_acc[st], 0, 0, 0);
+          const bf16x8 a_lo = codes8_to_bf16x8<KVT>(a[0], a[1]), a_hi = codes8_to_bf16x8<KVT>(a[2], a[3]);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, qf[rb][2 * j], s_acc[rb][st], 0, 0, 0);
+            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, qf[rb][2 * j + 1], s_acc[rb][st], 0, 0, 0);
+          }
         }
       }
     }
 
     // ---- online softmax (log2 domain) -------------------------------------------------------
     const float sc_mul = CAP ? cap_out : p.scale_log2 * k_scale;
-    uint32_t pfrag[NS][2];
-    float alpha;
-    if (tb >= all_lo && tb + TT <= all_hi)
-      alpha = softmax_step<false, CAP, NS>(s_acc, sc_mul, cap_in * k_scale, tb, g4, row_lo, row_hi, m_run, l_run, pfrag);
-    else
-      alpha = softmax_step<true, CAP, NS>(s_acc, sc_mul, cap_in * k_scale, tb, g4, row_lo, row_hi, m_run, l_run, pfrag);
+    uint32_t pfrag[RB][NS][2];
     // The accumulators hold sum(p * v_code) in units of the current page's V scale, so P stays an exact
     // softmax weight in bf16; when the scale changes (a new page) they are converted once.
-    float o_mul = alpha;
+    float unit_mul = 1.f;
     if constexpr (EB == 1) {
-      if (v_unit != v_scale) o_mul = alpha * (v_unit * __builtin_amdgcn_rcpf(v_scale));
+      if (v_unit != v_scale) unit_mul = v_unit * __builtin_amdgcn_rcpf(v_scale);
       v_unit = v_scale;
     }
-    if (__any(o_mul != 1.f)) {
+    const bool inside = tb >= all_lo && tb + TT <= all_hi;
 #pragma unroll
-      for (int rt = 0; rt < DPL; ++rt) o_acc[rt] *= o_mul;
+    for (int rb = 0; rb < RB; ++rb) {
+      float alpha;
+      if (inside)
+        alpha = softmax_step<false, CAP, NS>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+      else
+        alpha = softmax_step<true, CAP, NS>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+      const float o_mul = (EB == 1) ? alpha * unit_mul : alpha;
+      if (__any(o_mul != 1.f)) {
+#pragma unroll
+        for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] *= o_mul;
+      }
     }
 
     // ---- O^T += V^T . P^T ---------------------------------------------------------------------
@@ -254,8 +279,12 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     // 8-bit pages: each lane reads 4 keys x 4 consecutive dims of codes and widens them while transposing.
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-      const u32x2 pb2 = {pfrag[st][0], pfrag[st][1]};
-      const s16x4 pb = __builtin_bit_cast(s16x4, pb2);
+      s16x4 pb[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const u32x2 pb2 = {pfrag[rb][st][0], pfrag[rb][st][1]};
+        pb[rb] = __builtin_bit_cast(s16x4, pb2);
+      }
       if constexpr (EB == 2) {
         const int tk = st * 16 + 4 * g4 + (n >> 2);
         const unsigned char* vrow = lds_v + tk * RK;
@@ -265,7 +294,8 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
           const int off = rt * 32 + (n & 3) * 8;
           const unsigned char* ptr = vrow + (((off >> 4) ^ key) << 4) + (off & 15);
           const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr);
-          o_acc[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb, o_acc[rt], 0, 0, 0);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[rb], o_acc[rb][rt], 0, 0, 0);
         }
       } else {
         // lane (n, g4) reads DPL consecutive dims (DPL*n ..) of keys 4g4..4g4+3 and widens them; row tile rt
@@ -295,7 +325,9 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) {
           const u32x2 a2 = {pack_bf16(vf[0][rt], vf[1][rt]), pack_bf16(vf[2][rt], vf[3][rt])};
-          o_acc[rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), pb, o_acc[rt], 0, 0, 0);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb)
+            o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), pb[rb], o_acc[rb][rt], 0, 0, 0);
         }
       }
     }
@@ -347,43 +379,47 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 
   // ---- epilogue ---------------------------------------------------------------------------------
   // accumulator column j of row tile rt is dim 16rt + 4g4 + j (bf16 pages) or DPL*(4g4 + j) + rt (8-bit pages)
-  float l_tot = l_run + __shfl_xor(l_run, 16);
-  l_tot += __shfl_xor(l_tot, 32);
-  if (n < rows) {
-    const int tok_out = cur.q0 + r_tok;
-    const int head_out = h * G + r_head;
-    if (cur.single) {
-      const float l_fin = with_sink(p, head_out, m_run, l_tot);
-      const float inv = (l_fin > 0.f ? 1.f / l_fin : 0.f) * v_unit;
-      uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D;
-      if constexpr (EB == 2) {
 #pragma unroll
-        for (int rt = 0; rt < DPL; ++rt) {
-          const u32x2 w = {pack_bf16(o_acc[rt][0] * inv, o_acc[rt][1] * inv), pack_bf16(o_acc[rt][2] * inv, o_acc[rt][3] * inv)};
-          *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
+  for (int rb = 0; rb < RB; ++rb) {
+    float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    if (n + 16 * rb < rows) {
+      const int tok_out = cur.q0 + r_tok[rb];
+      const int head_out = h * G + r_head[rb];
+      if (cur.single) {
+        const float l_fin = with_sink(p, head_out, m_run[rb], l_tot);
+        const float inv = (l_fin > 0.f ? 1.f / l_fin : 0.f) * v_unit;
+        uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D;
+        if constexpr (EB == 2) {
+#pragma unroll
+          for (int rt = 0; rt < DPL; ++rt) {
+            const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                             pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+            *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int rt = 0; rt < DPL; rt += 2)
+              *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
         }
       } else {
+        const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok[rb]) * p.Hq + head_out;
+        float* prow = p.part_o + slot * D;
+        if constexpr (EB == 2) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+          for (int rt = 0; rt < DPL; ++rt) *(f32x4*)(prow + 16 * rt + 4 * g4) = o_acc[rb][rt];
+        } else {
 #pragma unroll
-          for (int rt = 0; rt < DPL; rt += 2)
-            *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rt][j] * inv, o_acc[rt + 1][j] * inv);
-      }
-    } else {
-      const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok) * p.Hq + head_out;
-      float* prow = p.part_o + slot * D;
-      if constexpr (EB == 2) {
+          for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int rt = 0; rt < DPL; ++rt) *(f32x4*)(prow + 16 * rt + 4 * g4) = o_acc[rt];
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int rt = 0; rt < DPL; ++rt) prow[DPL * (4 * g4 + j) + rt] = o_acc[rt][j] * v_unit;
-      }
-      if (g4 == 0) {
-        p.part_ml[slot * 2 + 0] = m_run;
-        p.part_ml[slot * 2 + 1] = l_tot;
+            for (int rt = 0; rt < DPL; ++rt) prow[DPL * (4 * g4 + j) + rt] = o_acc[rb][rt][j] * v_unit;
+        }
+        if (g4 == 0) {
+          p.part_ml[slot * 2 + 0] = m_run[rb];
+          p.part_ml[slot * 2 + 1] = l_tot;
+        }
       }
     }
   }
@@ -476,15 +512,15 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   }
 }
 
-template <int D, int KVT, int TT, int WPB, bool CAP>
-static int launch_cap(hipStream_t stream, AttnParams p) {
+template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
+static int launch_rb(hipStream_t stream, AttnParams p) {
   // persistent grid: as many workgroups as are resident at once, per KV-head group
   static int resident = 0;
   if (resident == 0) {
     int dev = 0, cus = 0, per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP>, 64 * WPB, 0) != hipSuccess)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP, RB>, 64 * WPB, 0) != hipSuccess)
       return (int)hipGetLastError();
     resident = max(1, cus * max(1, per_cu));
   }
@@ -495,8 +531,18 @@ static int launch_cap(hipStream_t stream, AttnParams p) {
   p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + (p.T + kScatterTokensPerBlock - 1) / kScatterTokensPerBlock : 1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2)
-    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP, RB>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();
+}
+
+// Two row blocks per wave exist for bf16 pages up to head size 128 (beyond that the accumulators of the second block do
+// not fit the registers of two waves per SIMD); decode_row_limit() below tells the callers which limit applies.
+template <int D, int KVT, int TT, int WPB, bool CAP>
+static int launch_cap(hipStream_t stream, const AttnParams& p) {
+  if constexpr (ElemBytes<KVT>::v == 2 && D <= 128) {
+    if (p.dec_rows > kRowBlock) return launch_rb<D, KVT, TT, WPB, CAP, 2>(stream, p);
+  }
+  return launch_rb<D, KVT, TT, WPB, CAP, 1>(stream, p);
 }
 
 template <int D, int KVT, int TT, int WPB>
@@ -533,6 +579,14 @@ static int launch_kvt(hipStream_t stream, const AttnParams& p) {
     default:
       return (int)hipErrorInvalidValue;
   }
+}
+
+// Most query rows per KV head (q_len * group) a sequence may have and still be served by the decode kernel, for a
+// call with T query tokens over S sequence rows.  A call that cannot hold a multi-token row (T <= S leaves no room
+// for one unless other rows are empty) keeps the one-block kernel, which is the faster one on single-token rows.
+int decode_row_limit(int T, int S, int D, int kv_dtype) {
+  if (kv_dtype == RPA_BF16 && D <= 128 && T > S) return 2 * kRowBlock;
+  return kRowBlock;
 }
 
 bool decode_supported(const AttnParams& p) {

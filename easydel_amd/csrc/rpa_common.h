@@ -48,6 +48,7 @@ struct AttnParams {
   int window;        // <= 0: none
   float softcap;     // <= 0: none
   int max_splits;    // >= 2: most partial slots one sequence may use
+  int dec_rows;      // most query rows per KV head (q_len * group) of a sequence the decode kernel serves: 16 or 32
   int t_dec_max;     // static bound on decode-class query tokens = rows of one partial slot
   int n_wg;          // persistent decode workgroups per KV-head group
   int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
@@ -67,7 +68,7 @@ struct SeqPlan {
   int q0, q_len, ctx;
   int lo, hi;       // key range any row of the sequence may see, lo rounded down to 64 tokens
   bool live;        // has queries and keys
-  bool small_rows;  // q_len * group <= 16: served by the split-K decode kernel
+  bool small_rows;  // q_len * group <= dec_rows (16 or 32): served by the split-K decode kernel
 };
 
 __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
@@ -84,7 +85,7 @@ __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
     int first = s.ctx - s.q_len - p.window + 1;  // lowest key visible to the first query row
     s.lo = first > 0 ? (first & ~63) : 0;
   }
-  s.small_rows = (s.q_len * p.group <= kRowBlock);
+  s.small_rows = (s.q_len * p.group <= p.dec_rows);
   return s;
 }
 
@@ -234,6 +235,7 @@ int launch_attn_prefill(hipStream_t stream, const AttnParams& p);
 int launch_attn_prefill_dma(hipStream_t stream, const AttnParams& p);  // bf16 pages, tiles loaded straight into LDS
 int launch_attn_merge(hipStream_t stream, const AttnParams& p);
 bool decode_supported(const AttnParams& p);
+int decode_row_limit(int T, int S, int D, int kv_dtype);
 bool prefill_supported(const AttnParams& p);
 bool prefill_dma_supported(const AttnParams& p);
 

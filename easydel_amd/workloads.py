@@ -70,9 +70,15 @@ class Workload:
             return np.minimum(ctx, self.sliding_window + self.q_lens.astype(np.int64) - 1)
         return ctx
 
+    def decode_row_limit(self) -> int:
+        """Most (token, group-head) rows per KV head of a sequence the split-K decode kernel serves in a call on this
+        workload: 32 for bf16 pages up to head size 128 when the batch has more query tokens than sequence rows
+        (only then can a row hold several tokens), else 16 (mirrors ``decode_row_limit`` of the library)."""
+        return 32 if (self.kv_dtype == "bf16" and self.D <= 128 and int(self.q_lens.sum()) > len(self.q_lens)) else 16
+
     def small_row_mask(self) -> np.ndarray:
-        """Sequences the split-K decode kernel serves: at most 16 (token, group-head) rows per KV head."""
-        return (self.q_lens > 0) & (self.q_lens * (self.Hq // self.Hkv) <= 16)
+        """Sequences the split-K decode kernel serves."""
+        return (self.q_lens > 0) & (self.q_lens * (self.Hq // self.Hkv) <= self.decode_row_limit())
 
     def attention_bytes(self, select: np.ndarray | None = None) -> int:
         """Algorithmic HBM bytes of one attention call: every visible K/V element once per sequence,

@@ -52,6 +52,37 @@ def test_small_multi_token_rows(gpu):
     _check(b, "bf16 multi-token small rows")
 
 
+@pytest.mark.parametrize("D,page_size,Hq,Hkv", [(128, 64, 32, 8), (64, 32, 64, 8), (128, 16, 40, 8), (64, 16, 16, 1)])
+def test_multi_token_rows_of_17_to_32(gpu, D, page_size, Hq, Hkv):
+    # speculative-decoding verification steps: 17..32 rows per KV head ride the decode kernel with two row blocks per
+    # wave (bf16 pages, head size <= 128, a batch with more tokens than sequence rows); long contexts are cut into
+    # spans and merged, every row has its own causal limit
+    G = Hq // Hkv
+    q_max = 32 // G
+    ctx = [5, 64, 300, 1100, 777, 40, 33, 3000, 9]
+    q_lens = [min(q, c) for q, c in zip([q_max, q_max - 1, q_max, 17 // G + 1, q_max, 1, q_max, q_max, q_max], ctx)]
+    b = tl.make_batch(15 + D, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, max_pages=-(-3000 // page_size))
+    assert b.T > b.S and max(q * G for q in q_lens) > 16
+    _check(b, f"bf16 rows up to 32, D{D} pg{page_size} {Hq}/{Hkv}")
+    _check(b, f"bf16 rows up to 32 + window, D{D}", sliding_window=70)
+    s = np.random.default_rng(D).uniform(-1.0, 6.0, size=Hq).astype(np.float32)
+    got = tl.run_gpu_attention(b, softmax_aux=s, logits_soft_cap=30.0)
+    tl.assert_close(got, tl.oracle_out(b, softmax_aux=s, logits_soft_cap=30.0), b, "rows up to 32 + sinks + soft cap")
+
+
+def test_row_class_limit_follows_the_static_bounds(gpu):
+    # the same sequences in a call whose bounds leave no room for multi-token rows (T <= S through padded sequence
+    # rows) are served by the large-row kernel instead: both routes must agree with the oracle and with each other
+    ctx = [300, 1100, 64, 2000]
+    q_lens = [6, 8, 5, 7]
+    wide = tl.make_batch(16, ctx, q_lens, Hq=32, Hkv=8, D=128, page_size=64, max_pages=32)
+    padded = tl.make_batch(16, ctx, q_lens, Hq=32, Hkv=8, D=128, page_size=64, max_pages=32, pad_rows=40)
+    assert wide.T > wide.S and padded.T <= padded.S
+    a = _check(wide, "rows 20..32, decode kernel")
+    c = _check(padded, "rows 20..32, large-row kernel")
+    assert np.abs(a[tl.valid_rows(wide)] - c[tl.valid_rows(padded)]).max() <= 2e-2
+
+
 @pytest.mark.parametrize("window", [1, 64, 100, 1000])
 def test_sliding_window_decode(gpu, window):
     ctx = [1, window, window + 1, window + 2, 900, 1500, 65, 129]
