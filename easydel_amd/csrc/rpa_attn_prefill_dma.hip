@@ -103,7 +103,6 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   int out_tok[RB], out_head[RB];
   bf16x8 qf[RB][NKK];
   int wave_lo, wave_hi;          // keys every row of the wave sees: [max row_lo, min row_hi)
-  int wave_lo_min, wave_hi_max;  // keys some row of the wave sees: [min row_lo, max row_hi)
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = R0 + (wave * RB + rb) * 16 + n;
@@ -134,28 +133,20 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
     }
   {
-    int lo_max = 0, hi_min = 0x7fffffff, lo_min = 0x7fffffff, hi_max = 0;
+    int lo_max = 0, hi_min = 0x7fffffff;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       lo_max = max(lo_max, row_lo[rb]);
       hi_min = min(hi_min, row_hi[rb]);
-      lo_min = min(lo_min, row_lo[rb]);
-      hi_max = max(hi_max, row_hi[rb]);
     }
 #pragma unroll
     for (int o = 1; o < 16; o <<= 1) {
       lo_max = max(lo_max, __shfl_xor(lo_max, o));
       hi_min = min(hi_min, __shfl_xor(hi_min, o));
-      lo_min = min(lo_min, __shfl_xor(lo_min, o));
-      hi_max = max(hi_max, __shfl_xor(hi_max, o));
     }
     wave_lo = __builtin_amdgcn_readfirstlane(lo_max);
     wave_hi = __builtin_amdgcn_readfirstlane(hi_min);
-    wave_lo_min = __builtin_amdgcn_readfirstlane(lo_min);
-    wave_hi_max = __builtin_amdgcn_readfirstlane(hi_max);
   }
-  // a wave whose row blocks all lie past the sequence's rows only helps with the loads
-  const bool wave_active = (R0 + wave * RB * 16) < rows_total;
 
   // ---- tile loads ------------------------------------------------------------------------------------
   // DMA instruction u of wave w fills LDS rows (u NW + w) RPI .. + RPI - 1 of the K half, and again of the V
@@ -452,8 +443,6 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   }
   softmax(masked, s_cur, kv_lo + t * TT, pf);  // the last tile
   pv(pf, v_slot(rd_v));
-  (void)wave_active;
-  (void)wave_lo_min; (void)wave_hi_max;
 
   // ---- epilogue -----------------------------------------------------------------------------------------
 #pragma unroll
