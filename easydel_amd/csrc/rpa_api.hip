@@ -11,10 +11,10 @@ namespace rpa {
 int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_t*, void*, int, int, int64_t, int,
                           int64_t, int);
 int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
-                          const int32_t*, const int32_t*, int, int, int, int, int, int, int, int);
+                          const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int);
 int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
 int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
-                                const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int);
+                                const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int);
 }  // namespace rpa
 
 namespace {
@@ -172,7 +172,7 @@ int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* va
   if (!key || !value || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs)
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged: null pointer");
   return hip_fail(rpa::launch_scatter_ragged((hipStream_t)stream, key, value, kv_pages, context_lens, block_tables,
-                                             query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C, elem_bytes),
+                                             query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, elem_bytes),
                   "rpa_page_scatter_ragged launch");
 }
 
@@ -194,7 +194,7 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
   if ((((uintptr_t)key) | ((uintptr_t)value)) & 15 || ((uintptr_t)kv_pages & 3))
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: key/value must be 16-byte and kv_pages 4-byte aligned");
   return hip_fail(rpa::launch_scatter_ragged_quant((hipStream_t)stream, key, value, kv_pages, kv_scales, context_lens,
-                                                   block_tables, query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C,
+                                                   block_tables, query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C,
                                                    src_dtype, kv_dtype),
                   "rpa_page_scatter_ragged_quantised launch");
 }
@@ -273,7 +273,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
       p.new_v = new_value;
     } else {
       const int err = rpa::launch_scatter_ragged(s, new_key, new_value, const_cast<void*>(k_pages), context_lens, block_tables,
-                                                 query_start_loc, num_seqs, T, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
+                                                 query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
       if (err) return hip_fail(err, "page scatter launch");
     }
   }

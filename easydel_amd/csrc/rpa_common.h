@@ -89,7 +89,8 @@ __device__ __forceinline__ SeqPlan seq_plan(const AttnParams& p, int i) {
   return s;
 }
 
-__device__ __forceinline__ int live_rows(const AttnParams& p) { return p.num_seqs ? p.num_seqs[0] : p.S; }
+// never more than the S rows the metadata arrays hold, whatever the device value says
+__device__ __forceinline__ int live_rows(const AttnParams& p) { return p.num_seqs ? min(p.num_seqs[0], p.S) : p.S; }
 
 // Attention sinks: the softmax of query head hq runs over the keys and one more logit, sinks[hq], whose
 // probability is then dropped -- a key with that score and a zero value row.  Only the denominator changes:

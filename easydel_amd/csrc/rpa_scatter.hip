@@ -74,11 +74,11 @@ __global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restr
                                                              const int32_t* __restrict__ context_lens,
                                                              const int32_t* __restrict__ block_tables,
                                                              const int32_t* __restrict__ qsl,
-                                                             const int32_t* __restrict__ num_seqs, int M, int P,
+                                                             const int32_t* __restrict__ num_seqs, int S, int M, int P,
                                                              int page_size, int Hkv, int head_bytes,
                                                              int64_t token_stride, int64_t page_stride) {
   // interleaved pages: V of a head one row behind its K, heads two rows apart
-  scatter_token(key, value, pages, pages + head_bytes, context_lens, block_tables, qsl, num_seqs[0], M, P, page_size, Hkv,
+  scatter_token(key, value, pages, pages + head_bytes, context_lens, block_tables, qsl, min(num_seqs[0], S), M, P, page_size, Hkv,
                 head_bytes, 2 * (int64_t)head_bytes, token_stride, page_stride, blockIdx.x, threadIdx.x, blockDim.x);
 }
 
@@ -135,10 +135,10 @@ __global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __
                                                                   const int32_t* __restrict__ context_lens,
                                                                   const int32_t* __restrict__ block_tables,
                                                                   const int32_t* __restrict__ qsl,
-                                                                  const int32_t* __restrict__ num_seqs, int M, int P,
+                                                                  const int32_t* __restrict__ num_seqs, int S, int M, int P,
                                                                   int page_size, int Hkv, int D, int C) {
   const int t = blockIdx.x, c = blockIdx.y, lane = threadIdx.x;
-  const int n_live = num_seqs[0];
+  const int n_live = min(num_seqs[0], S);  // never more than the rows the metadata arrays hold
   if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
   const int i = find_seq_wave(qsl, n_live, t);
   const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
@@ -195,12 +195,12 @@ __global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __
 
 int launch_scatter_ragged_quant(hipStream_t stream, const void* key, const void* value, void* pages, float* scales,
                                 const int32_t* context_lens, const int32_t* block_tables, const int32_t* qsl,
-                                const int32_t* num_seqs, int T, int M, int P, int page_size, int Hkv, int D, int C,
+                                const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int Hkv, int D, int C,
                                 int src_dtype, int kv_dtype) {
   const dim3 grid(T, 2 * Hkv), block(64);
 #define RPA_QSCATTER(SRC, KVT)                                                                                        \
   hipLaunchKernelGGL((scatter_ragged_quant_kernel<SRC, KVT>), grid, block, 0, stream, key, value, (unsigned char*)pages, \
-                     scales, context_lens, block_tables, qsl, num_seqs, M, P, page_size, Hkv, D, C)
+                     scales, context_lens, block_tables, qsl, num_seqs, S, M, P, page_size, Hkv, D, C)
   if (src_dtype == RPA_F32 && kv_dtype == RPA_FP8_E4M3) RPA_QSCATTER(RPA_F32, RPA_FP8_E4M3);
   else if (src_dtype == RPA_F32 && kv_dtype == RPA_INT8) RPA_QSCATTER(RPA_F32, RPA_INT8);
   else if (src_dtype == RPA_BF16 && kv_dtype == RPA_FP8_E4M3) RPA_QSCATTER(RPA_BF16, RPA_FP8_E4M3);
@@ -231,12 +231,12 @@ int launch_scatter_slices(hipStream_t stream, const void* new_kv, const int32_t*
 
 int launch_scatter_ragged(hipStream_t stream, const void* key, const void* value, void* pages,
                           const int32_t* context_lens, const int32_t* block_tables, const int32_t* qsl,
-                          const int32_t* num_seqs, int T, int M, int P, int page_size, int Hkv, int D, int C,
+                          const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int Hkv, int D, int C,
                           int elem_bytes) {
   const int head_bytes = D * elem_bytes;
   const int64_t token_stride = (int64_t)C * head_bytes;
   hipLaunchKernelGGL(scatter_ragged_kernel, dim3(T), dim3(256), 0, stream, (const char*)key, (const char*)value,
-                     (char*)pages, context_lens, block_tables, qsl, num_seqs, M, P, page_size, Hkv, head_bytes,
+                     (char*)pages, context_lens, block_tables, qsl, num_seqs, S, M, P, page_size, Hkv, head_bytes,
                      token_stride, token_stride * page_size);
   return (int)hipGetLastError();
 }

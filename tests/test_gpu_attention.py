@@ -123,6 +123,15 @@ def test_padding_rows_tokens_and_zero_length_rows(gpu):
     assert np.all(got[int(b.query_start_loc[b.n]):] == 0.0), "padded token rows must be written as zeros"
 
 
+def test_live_row_count_beyond_the_metadata_is_clamped(gpu):
+    # a row count larger than the metadata arrays (a caller's mistake) must not index past them: it counts as "all rows"
+    b = tl.make_batch(17, [100, 257, 64, 900], [1, 3, 1, 40], Hq=32, Hkv=8, D=128, page_size=64, max_pages=16)
+    want = tl.oracle_out(b)
+    b.num_seqs = np.array([b.S + 1000], dtype=np.int32)
+    got = tl.run_gpu_attention(b)
+    tl.assert_close(got, want, b, "row count beyond S")
+
+
 def test_shared_prefix_pages(gpu):
     # prefix caching: the same physical pages appear in several block-table rows
     ctx = [640, 700, 1000, 650]
