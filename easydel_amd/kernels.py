@@ -93,10 +93,11 @@ def page_scatter_slices(new_kv, slice_indices, num_slices, kv_cache_pages, *, pa
         return kv_cache_pages
     row_bytes = math.prod(new_kv.shape[1:]) * new_kv.element_size()
     _dev(kv_cache_pages, "kv_cache_pages")
-    _lib.check(lib.rpa_page_scatter_slices(
-        _stream(kv_cache_pages), _dev(new_kv, "new_kv"), _i32(slice_indices, "slice_indices"),
-        _i32(num_slices, "num_slices"), _dev(kv_cache_pages, "kv_cache_pages"), T, N, n_pos, int(page_size), row_bytes,
-        int(page_shard_index)))
+    with torch.cuda.device(kv_cache_pages.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_page_scatter_slices(
+            _stream(kv_cache_pages), _dev(new_kv, "new_kv"), _i32(slice_indices, "slice_indices"),
+            _i32(num_slices, "num_slices"), _dev(kv_cache_pages, "kv_cache_pages"), T, N, n_pos, int(page_size), row_bytes,
+            int(page_shard_index)))
     return kv_cache_pages
 
 
@@ -112,10 +113,11 @@ def page_scatter_ragged(key, value, kv_pages, context_lens, block_tables, query_
     if T == 0:
         return kv_pages
     _dev(kv_pages, "kv_pages")
-    _lib.check(lib.rpa_page_scatter_ragged(
-        _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
-        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-        _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, key.element_size()))
+    with torch.cuda.device(kv_pages.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_page_scatter_ragged(
+            _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, key.element_size()))
     return kv_pages
 
 
@@ -136,10 +138,11 @@ def page_scatter_ragged_quantised(key, value, kv_pages, kv_scales, context_lens,
     if T == 0:
         return kv_pages, kv_scales
     _dev(kv_pages, "kv_pages")
-    _lib.check(lib.rpa_page_scatter_ragged_quantised(
-        _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"), _dev(kv_scales, "kv_scales"),
-        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-        _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, dtype_tag(key.dtype), dtype_tag(kv_pages.dtype)))
+    with torch.cuda.device(kv_pages.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_page_scatter_ragged_quantised(
+            _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"), _dev(kv_scales, "kv_scales"),
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, dtype_tag(key.dtype), dtype_tag(kv_pages.dtype)))
     return kv_pages, kv_scales
 
 
@@ -193,11 +196,12 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
         if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
             raise ValueError(f"kv_scales must be float32 [P={P}, C={C}]")
         scales_ptr = _dev(kv_scales, "kv_scales")
-    _lib.check(lib.rpa_ragged_paged_attention(
-        _stream(query), _dev(query, "query"), _dev(kv_pages, "kv_pages"), scales_ptr,
-        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-        _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
+    with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_ragged_paged_attention(
+            _stream(query), _dev(query, "query"), _dev(kv_pages, "kv_pages"), scales_ptr,
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+            T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
     return out
 
 
@@ -237,11 +241,12 @@ def unified_attention(query, key_cache, value_cache, context_lens, block_tables,
         if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * 2 * Hkv:
             raise ValueError(f"kv_scales must be float32 [P={P}, 2*Hkv={2 * Hkv}]")
         scales_ptr = _dev(kv_scales, "kv_scales")
-    _lib.check(lib.rpa_unified_attention(
-        _stream(query), _dev(query, "query"), _dev(key_cache, "key_cache"), _dev(value_cache, "value_cache"), scales_ptr,
-        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-        None if num_seqs is None else _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-        T, S, M, P, pg, Hq, Hkv, D, qd, kd, scale, window, cap, aux_ptr))
+    with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_unified_attention(
+            _stream(query), _dev(query, "query"), _dev(key_cache, "key_cache"), _dev(value_cache, "value_cache"), scales_ptr,
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            None if num_seqs is None else _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+            T, S, M, P, pg, Hq, Hkv, D, qd, kd, scale, window, cap, aux_ptr))
     return out
 
 
@@ -264,11 +269,12 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
         _dev(t, name)
     aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
-    _lib.check(lib.rpa_ragged_paged_attention_v3(
-        _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
-        _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-        _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-        T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
+    with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_ragged_paged_attention_v3(
+            _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+            T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
     return out, kv_pages
 
 
@@ -294,9 +300,10 @@ def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, 
         _dev(t, name)
     aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
     ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
-    _lib.check(lib.rpa_ragged_paged_attention_v3_quantised(
-        _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
-        _dev(kv_scales, "kv_scales"), _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"),
-        _i32(query_start_loc, "query_start_loc"), _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(),
-        ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap, aux_ptr))
+    with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_ragged_paged_attention_v3_quantised(
+            _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+            _dev(kv_scales, "kv_scales"), _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"),
+            _i32(query_start_loc, "query_start_loc"), _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(),
+            ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap, aux_ptr))
     return out, kv_pages, kv_scales
