@@ -68,6 +68,11 @@ def load() -> ctypes.CDLL:
                     f"{LIB_PATH} is missing: build it with `python -m easydel_amd.build` "
                     "(there is no CPU or PyTorch fallback for this path)"
                 )
+            # PyTorch owns the device memory and streams this library is handed, so its HIP runtime must be the one
+            # in the process: loaded first here, the system's copy of the runtime would take its place and the
+            # library's first launch would find no device.
+            import torch  # noqa: F401
+
             lib = ctypes.CDLL(str(LIB_PATH))
             for name, (restype, argtypes) in SIGNATURES.items():
                 fn = getattr(lib, name)

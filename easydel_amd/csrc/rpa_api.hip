@@ -26,6 +26,7 @@ std::atomic<int> g_decode_sync{8};  // workgroup barrier every this many decode 
 std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are resident at once
 std::atomic<int> g_force_generic{0};
 std::atomic<int> g_prefill_dma{1};
+std::atomic<int> g_decode_pace{1};
 std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
 
 int fail(int code, const char* fmt, ...) {
@@ -135,6 +136,7 @@ int rpa_set_tunable(const char* name, int value) {
   if (!strcmp(name, "decode_wgs")) return g_decode_wgs.exchange(value < 0 ? 0 : value);
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
   if (!strcmp(name, "prefill_dma")) return g_prefill_dma.exchange(value != 0);
+  if (!strcmp(name, "decode_pace")) return g_decode_pace.exchange(value != 0);
   if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
   return -1;
 }
@@ -259,6 +261,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.decode_wgs = g_decode_wgs.load();
   p.decode_sync = g_decode_sync.load();
   p.prefill_dma = g_prefill_dma.load();
+  p.decode_pace = g_decode_pace.load();
   p.max_splits = 2;
   p.dec_rows = rpa::decode_row_limit(T, S, D, kv_dtype);
   p.pre_chunk = 1 << 30;

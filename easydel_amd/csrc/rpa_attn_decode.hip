@@ -62,7 +62,14 @@ __device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* 
 
 // RB: 16-row blocks of query rows one wave carries (rows of a sequence for one KV head: q_len * group <= 16 * RB).
 // Every K and V operand read from LDS feeds the MFMAs of all RB blocks.
-template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
+// PACE: the workgroup counts its waves that have a tile's loads in flight (an LDS counter: up by one before a wave
+// issues, down by one when its data has arrived), and a wave that finds kPaceCrowd or more of them pauses once, for
+// kPacePause x 64 clocks, before it adds its own.  This memory system delivers more a little below saturation than
+// with every wave pressing on it: bounding the requests in flight this way is worth 2 % on long bf16 streams
+// (742 -> 727 us on the Llama-shaped decode batch; 8-bit pages and four-wave workgroups lose by it, so they are
+// built without).  There is no loop and no waiting on another wave: the delay of a tile is bounded by the pause.
+constexpr int kPaceCrowd = 5, kPacePause = 16;
+template <int D, int KVT, int TT, int WPB, bool CAP, int RB, bool PACE>
 __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
@@ -82,6 +89,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   static_assert(LPT <= 64 && TT % TPI == 0 && TT % 16 == 0, "tile shape");
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_all[WPB * TT * HB];
+  __shared__ int s_inflight;  // PACE: waves of this workgroup with a tile's loads in flight
+  if constexpr (PACE) {
+    if (threadIdx.x == 0) s_inflight = 0;
+    __syncthreads();
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -133,8 +145,30 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   const float cap_out = p.softcap * 1.4426950408889634f;
   const float cap_in = CAP ? p.scale / p.softcap : 0.f;
 
+  // short spans (small batches) are latency-bound from start to end: no pacing there
+  const bool pace = PACE && p.decode_pace != 0 && Q >= 512;
+  bool counted = false;
+  auto enter = [&]() {
+    if constexpr (PACE) {
+      if (!pace) return;
+      int seen = 0;
+      if (lane == 0) seen = atomicAdd(&s_inflight, 1);
+      seen = __builtin_amdgcn_readfirstlane(seen);
+      counted = true;
+      if (seen >= kPaceCrowd) __builtin_amdgcn_s_sleep(kPacePause);
+    }
+  };
+  auto leave = [&]() {
+    if constexpr (PACE) {
+      if (!counted) return;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the tile has arrived
+      if (lane == 0) atomicSub(&s_inflight, 1);
+      counted = false;
+    }
+  };
   Piece cur = make_piece(p, P, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
   int page_a = page_of(cur.i, cur.t_begin), page_b = 0;  // pages of the tiles in staging buffers 0 and 1
+  enter();
   issue(Buf0{}, cur.t_begin, page_a);  // first tile in flight before anything else is set up
 
   for (;;) {
@@ -345,6 +379,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     // The waves of a workgroup read adjacent 512-byte spans of the same token rows; a barrier every few tiles
     // keeps them in step so each DRAM row is opened once (740 vs 764 us).  All waves of a workgroup walk the
     // same pieces and tiles, so every live wave reaches every barrier.
+    leave();
     if (p.decode_sync > 0 && (tile & (p.decode_sync - 1)) == 0) __builtin_amdgcn_s_barrier();
     commit(Buf0{}, tb);
     float ks = 1.f, vs = 1.f;
@@ -354,9 +389,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     }
     if (tile + DEPTH < n_tiles) {
       page_a = page_of(cur.i, tb + DEPTH * TT);
+      enter();
       issue(Buf0{}, tb + DEPTH * TT, page_a);
     } else if (has_next) {
       page_a = page_nxt;
+      enter();
       issue(Buf0{}, nxt.t_begin, page_nxt);
     }
     compute(tb, ks, vs);
@@ -514,13 +551,14 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
 
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 static int launch_rb(hipStream_t stream, AttnParams p) {
+  constexpr bool PACE = ElemBytes<KVT>::v == 2 && WPB == 8;
   // persistent grid: as many workgroups as are resident at once, per KV-head group
   static int resident = 0;
   if (resident == 0) {
     int dev = 0, cus = 0, per_cu = 0;
     if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP, RB>, 64 * WPB, 0) != hipSuccess)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP, RB, PACE>, 64 * WPB, 0) != hipSuccess)
       return (int)hipGetLastError();
     resident = max(1, cus * max(1, per_cu));
   }
@@ -531,7 +569,7 @@ static int launch_rb(hipStream_t stream, AttnParams p) {
   p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + (p.T + kScatterTokensPerBlock - 1) / kScatterTokensPerBlock : 1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2)
-    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP, RB>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+    hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP, RB, PACE>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
   return (int)hipGetLastError();
 }
 
