@@ -65,10 +65,11 @@ __device__ __forceinline__ Piece make_piece(const AttnParams& p, const int32_t* 
 // PACE: the workgroup counts its waves that have a tile's loads in flight (an LDS counter: up by one before a wave
 // issues, down by one when its data has arrived), and a wave that finds kPaceCrowd or more of them pauses once, for
 // kPacePause x 64 clocks, before it adds its own.  This memory system delivers more a little below saturation than
-// with every wave pressing on it: bounding the requests in flight this way is worth 2 % on long bf16 streams
-// (742 -> 727 us on the Llama-shaped decode batch; 8-bit pages and four-wave workgroups lose by it, so they are
+// with every wave pressing on it: bounding the requests in flight this way is worth 2.4 % on long bf16 streams
+// (738.5 -> 721 us on the Llama-shaped decode batch, both builds run in one process; crowds of 3 to 5 and pauses
+// of 512 to 1024 clocks all lie within 1 % of that; 8-bit pages and four-wave workgroups lose by it, so they are
 // built without).  There is no loop and no waiting on another wave: the delay of a tile is bounded by the pause.
-constexpr int kPaceCrowd = 5, kPacePause = 16;
+constexpr int kPaceCrowd = 4, kPacePause = 8;
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB, bool PACE>
 __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;

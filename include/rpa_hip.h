@@ -209,8 +209,8 @@ int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t
  *                    from the shapes); set it before sizing the workspace
  *   "decode_wgs"     persistent decode workgroups per KV-head group (0 = as many as are resident at once)
  *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
- *   "decode_pace"    1 (default): in the bf16 eight-wave decode kernel a wave that finds five or more of its workgroup's
- *                    tiles in flight pauses once (1 024 clocks) before issuing its own; 0: never
+ *   "decode_pace"    1 (default): in the bf16 eight-wave decode kernel a wave that finds four or more of its workgroup's
+ *                    tiles in flight pauses once (512 clocks) before issuing its own; 0: never
  *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
  *                    set it before sizing the workspace
  *   "prefill_dma"    1 (default): bf16 prefill tiles are loaded global -> LDS by the load unit where that kernel
