@@ -43,6 +43,12 @@ SIGNATURES = {
         _c_int,
         [_c_vp] * 11 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
+    "rpa_mla_ragged_paged_attention": (
+        _c_int,
+        [_c_vp] * 12 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],
+    ),
+    "rpa_mla_workspace_bytes": (_c_sz, [_c_int] * 8),
+    "rpa_mla_page_scatter": (_c_int, [_c_vp] * 8 + [_c_int] * 9),
 }
 
 

@@ -26,6 +26,7 @@ SOURCES = [
     "rpa_attn_prefill.hip",
     "rpa_attn_prefill_dma.hip",
     "rpa_attn_merge.hip",
+    "rpa_mla.hip",
 ]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from scalar float code on this target.

@@ -6,6 +6,7 @@
 #include <cstring>
 
 #include "rpa_common.h"
+#include "rpa_mla.h"
 
 namespace rpa {
 int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_t*, void*, int, int, int64_t, int,
@@ -27,6 +28,7 @@ std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are 
 std::atomic<int> g_force_generic{0};
 std::atomic<int> g_prefill_dma{1};
 std::atomic<int> g_decode_pace{1};
+std::atomic<int> g_mla_chunks{0};  // 0 = sized from the shapes
 std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
 
 int fail(int code, const char* fmt, ...) {
@@ -112,6 +114,25 @@ int decode_token_bound(int T, int S, int Hq, int Hkv, int dec_rows) {
   return (int)(bound < T ? bound : T);
 }
 
+// MLA: how many key chunks a row tile may be cut into, and the shortest chunk.  Cutting fills the chip when the batch
+// holds few row tiles and evens out sequences of different lengths; every chunk of a row costs a float32 partial
+// row (lkv + 2 floats) written and read back, which with many heads per token is comparable to the keys themselves,
+// hence the longer minimum there.  The partial buffers stay under ~1 GiB.
+void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* min_chunk) {
+  const long slots = (long)T * Hq / rpa::kMlaRows + S;
+  long chunks = g_mla_chunks.load() > 0 ? g_mla_chunks.load() : (768 + slots - 1) / slots;
+  if (chunks > rpa::kMlaMaxChunks) chunks = rpa::kMlaMaxChunks;
+  if (chunks < 1) chunks = 1;
+  const size_t per = part_o_bytes(T, Hq, lkv) + part_ml_bytes(T, Hq);
+  while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
+  *max_chunks = (int)chunks;
+  *min_chunk = Hq >= 64 ? 2048 : 512;
+}
+
+bool mla_shape_on_mfma(int page_size, int lkv, int rope, int row_elems, int q_dtype, int kv_dtype) {
+  return q_dtype == RPA_BF16 && kv_dtype == RPA_BF16 && lkv == 512 && rope == 64 && page_size % 32 == 0 && row_elems % 8 == 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -137,6 +158,7 @@ int rpa_set_tunable(const char* name, int value) {
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
   if (!strcmp(name, "prefill_dma")) return g_prefill_dma.exchange(value != 0);
   if (!strcmp(name, "decode_pace")) return g_decode_pace.exchange(value != 0);
+  if (!strcmp(name, "mla_chunks")) return g_mla_chunks.exchange(value < 0 ? 0 : (value > rpa::kMlaMaxChunks ? rpa::kMlaMaxChunks : value));
   if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
   return -1;
 }
@@ -390,6 +412,114 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
   return rpa_ragged_paged_attention(stream, q, kv_pages, kv_scales, context_lens, block_tables, query_start_loc, n_live,
                                     out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
                                     kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux);
+}
+
+size_t rpa_mla_workspace_bytes(int T, int S, int M, int page_size, int Hq, int kv_lora_rank, int q_dtype, int kv_dtype) {
+  (void)M; (void)page_size; (void)q_dtype; (void)kv_dtype;
+  if (T <= 0 || S <= 0 || Hq <= 0 || kv_lora_rank <= 0) return 256;
+  int chunks, min_chunk;
+  mla_split(T, S, Hq, kv_lora_rank, &chunks, &min_chunk);
+  return (chunks > 1 ? (size_t)chunks * (part_o_bytes(T, Hq, kv_lora_rank) + part_ml_bytes(T, Hq)) : 0) + 512;
+}
+
+static int mla_fill(const char* who, rpa::MlaParams& p, const void* keys_values, const void* keys_pe, void* kv_pages,
+                    const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
+                    const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int lkv, int rope, int row_elems,
+                    int kv_dtype) {
+  if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || lkv <= 0 || rope < 0 || row_elems <= 0)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (T=%d S=%d M=%d P=%d page_size=%d kv_lora_rank=%d rope=%d row_elems=%d)",
+                who, T, S, M, P, page_size, lkv, rope, row_elems);
+  if (lkv > 512 || rope > 256 || lkv % 8 != 0 || rope % 8 != 0)
+    return fail(RPA_ERR_UNSUPPORTED, "%s: kv_lora_rank %d / qk_rope_head_dim %d (want multiples of 8, <= 512 / <= 256)", who, lkv, rope);
+  const int rope_off = (lkv + 127) / 128 * 128;
+  if (row_elems < rope_off + rope)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: row_elems=%d < %d (latent part padded to 128, then the rope key)", who, row_elems, rope_off + rope);
+  if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16)
+    return fail(RPA_ERR_UNSUPPORTED, "%s: kv_dtype %d (want f32 or bf16)", who, kv_dtype);
+  memset(&p, 0, sizeof(p));
+  p.new_kv = keys_values; p.new_pe = keys_pe; p.pages = kv_pages;
+  p.context_lens = context_lens; p.block_tables = block_tables; p.qsl = query_start_loc; p.num_seqs = num_seqs;
+  p.T = T; p.S = S; p.M = M; p.P = P; p.page_size = page_size; p.lkv = lkv; p.rope = rope; p.rope_off = rope_off;
+  p.row_elems = row_elems;
+  p.token_stride = (int64_t)row_elems * rpa::elem_bytes(kv_dtype);
+  p.page_stride = p.token_stride * page_size;
+  p.kv_dtype = kv_dtype;
+  p.max_chunks = 1;
+  p.min_chunk = 512;
+  return RPA_OK;
+}
+
+int rpa_mla_page_scatter(rpa_stream_t stream, const void* keys_values, const void* keys_pe, void* kv_pages,
+                         const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
+                         const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int kv_lora_rank,
+                         int qk_rope_head_dim, int row_elems, int elem_bytes) {
+  const char* who = "rpa_mla_page_scatter";
+  if (elem_bytes != 2 && elem_bytes != 4) return fail(RPA_ERR_UNSUPPORTED, "%s: elem_bytes %d (want 2 or 4)", who, elem_bytes);
+  rpa::MlaParams p;
+  const int rc = mla_fill(who, p, keys_values, keys_pe, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, T, S,
+                          M, P, page_size, kv_lora_rank, qk_rope_head_dim, row_elems, elem_bytes == 4 ? RPA_F32 : RPA_BF16);
+  if (rc) return rc;
+  if (T == 0) return RPA_OK;
+  if (!keys_values || (!keys_pe && qk_rope_head_dim > 0) || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  return hip_fail(rpa::launch_mla_scatter((hipStream_t)stream, p), "rpa_mla_page_scatter launch");
+}
+
+int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope, const void* queries_pe,
+                                   const void* keys_values, const void* keys_pe, void* kv_pages,
+                                   const int32_t* context_lens, const int32_t* block_tables,
+                                   const int32_t* query_start_loc, const int32_t* distribution, void* out,
+                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P, int page_size,
+                                   int Hq, int kv_lora_rank, int qk_rope_head_dim, int row_elems, int q_dtype,
+                                   int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
+                                   const float* softmax_aux) {
+  const char* who = "rpa_mla_ragged_paged_attention";
+  if (Hq <= 0) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (Hq=%d)", who, Hq);
+  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16) return fail(RPA_ERR_UNSUPPORTED, "%s: q_dtype %d (want f32 or bf16)", who, q_dtype);
+  if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null distribution", who);
+  if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_scale is not finite", who);
+  if (softmax_aux && ((uintptr_t)softmax_aux & 3)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_aux must be 4-byte aligned", who);
+  rpa::MlaParams p;
+  const int rc = mla_fill(who, p, keys_values, keys_pe, kv_pages, context_lens, block_tables, query_start_loc, distribution + 2,
+                          T, S, M, P, page_size, kv_lora_rank, qk_rope_head_dim, row_elems, kv_dtype);
+  if (rc) return rc;
+  if (T == 0) return RPA_OK;
+  if (!queries_nope || (!queries_pe && qk_rope_head_dim > 0) || !kv_pages || !context_lens || !block_tables || !query_start_loc || !out)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+  if (keys_values && !keys_pe && qk_rope_head_dim > 0) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: keys_values without keys_pe", who);
+  if ((((uintptr_t)queries_nope) | ((uintptr_t)queries_pe) | ((uintptr_t)out) | ((uintptr_t)kv_pages)) & 15)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: queries, out and the page pool must be 16-byte aligned", who);
+  p.q_nope = queries_nope; p.q_pe = queries_pe; p.out = out; p.sinks = softmax_aux;
+  p.Hq = Hq; p.q_dtype = q_dtype;
+  p.scale = softmax_scale;
+  p.scale_log2 = softmax_scale * 1.4426950408889634f;
+  p.window = sliding_window > 0 ? sliding_window : 0;
+  p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
+  p.mfma = (!g_force_generic.load() && rpa::mla_mfma_supported(p)) ? 1 : 0;
+  hipStream_t s = (hipStream_t)stream;
+  if (keys_values) {
+    const int err = rpa::launch_mla_scatter(s, p);
+    if (err) return hip_fail(err, "MLA page write launch");
+  }
+  if (p.mfma) {
+    int chunks, min_chunk;
+    mla_split(T, S, Hq, kv_lora_rank, &chunks, &min_chunk);
+    const size_t po = part_o_bytes(T, Hq, kv_lora_rank), pml = part_ml_bytes(T, Hq);
+    char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    const size_t usable = (workspace && workspace_bytes > 256) ? workspace_bytes - 256 : 0;
+    if ((size_t)chunks * (po + pml) > usable) chunks = (int)(usable / (po + pml));  // a small workspace: fewer, longer chunks
+    if (chunks < 2) chunks = 1;  // a single chunk writes its rows directly and needs no workspace
+    p.max_chunks = chunks;
+    p.min_chunk = min_chunk;
+    p.part_o = (float*)base;
+    p.part_ml = (float*)(base + (size_t)chunks * po);
+    const int err = rpa::launch_mla_mfma(s, p);
+    if (err) return hip_fail(err, "MLA kernel launch");
+  } else {
+    const int err = rpa::launch_mla_generic(s, p);
+    if (err) return hip_fail(err, "MLA fp32 kernel launch");
+  }
+  return hip_fail(rpa::launch_mla_merge(s, p), "MLA merge kernel launch");
 }
 
 }  // extern "C"

@@ -1,0 +1,602 @@
+// Multi-latent attention (MLA) over latent ragged pages: page write, MFMA kernel, fp32 kernel, merge.
+//
+// The cache holds one row per token, shared by every query head: [latent (lkv) | rope key (rope)], each part padded
+// to a multiple of 128 elements.  For query row (token t, head h) at position pos the operation computes
+//     s_j = scale * (q_nope[t][h] . latent_j + q_pe[t][h] . rope_j)      over the visible keys j
+//     out[t][h] = sum_j softmax(s)_j * latent_j                          (lkv values; the caller applies the value
+//                                                                         half of the up-projection afterwards)
+// i.e. attention with one KV head, key width lkv + rope, value width lkv, and values that are a prefix of the keys.
+//
+// MFMA kernel (bf16, lkv = 512, rope = 64): a workgroup of eight waves owns 128 consecutive rows (row = (token,
+// head), token-major) of one sequence and one chunk of its keys; every wave keeps one 16-row block in registers
+// (Q as MFMA B operands: 18 k-steps of 32 = 72 registers; O^T accumulators: 32 tiles of 16 dims = 128 registers), two
+// waves per SIMD.  Tiles of 32 keys x 576 elements go global -> LDS through the load unit (global_load_lds_dwordx4,
+// no staging registers) into a ring of three slots, two tiles ahead of their use; the one tile serves all eight waves
+// and both products:
+//     S^T[key][row]  = K[key][:] . Q[row][:]            A = 16 keys x 32 dims read row-wise
+//     O^T[dim][row] += V^T[dim][key] . P^T[key][row]    A = 16 dims x 32 keys read with the transposing LDS load
+// Every matrix instruction takes one operand from LDS (1 KiB), which bounds the kernel: a compute unit's LDS delivers
+// 128 B a clock against the 256 B a clock its four SIMDs could consume at full rate.  Two row blocks per wave would
+// halve that, but their 256 accumulators and 144 query registers leave the compiler no working set in 512 registers
+// (it spilled the queries); that variant needs hand-placed registers and is not built.
+#include "rpa_mfma.h"
+#include "rpa_mla.h"
+
+namespace rpa {
+
+namespace {
+
+// ---- page write ------------------------------------------------------------------------------------------------
+// One wavefront per query token: its latent row and rope key into the page slot of its position, padding zeroed.
+template <typename E>
+__global__ __launch_bounds__(256) void mla_scatter_kernel(MlaParams p) {
+  const int lane = threadIdx.x & 63;
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= p.T) return;
+  const int n_live = mla_live_rows(p);
+  if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) return;
+  const int i = find_seq_wave(p.qsl, n_live, t);
+  const int q0 = p.qsl[i], q_len = p.qsl[i + 1] - q0;
+  const int pos = p.context_lens[i] - q_len + (t - q0);
+  if (pos < 0) return;
+  const int page_idx = pos / p.page_size;
+  if (page_idx >= p.M) return;
+  const int page = p.block_tables[(int64_t)i * p.M + page_idx];
+  if (page < 0 || page >= p.P) return;
+  E* row = (E*)((char*)p.pages + (int64_t)page * p.page_stride + (int64_t)(pos % p.page_size) * p.token_stride);
+  const E* kv = (const E*)p.new_kv + (int64_t)t * p.lkv;
+  const E* pe = (const E*)p.new_pe + (int64_t)t * p.rope;
+  for (int e = lane; e < p.row_elems; e += 64) {
+    E v = 0;
+    if (e < p.lkv) v = kv[e];
+    else if (e >= p.rope_off && e < p.rope_off + p.rope) v = pe[e - p.rope_off];
+    row[e] = v;
+  }
+}
+
+// ---- fp32 kernel: one wavefront per (query token, head) ----------------------------------------------------------
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+constexpr int kGenMaxLkv = 512, kGenMaxRope = 256;
+
+template <int QT, int KVT>
+__global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
+  __shared__ float q_s[kGenMaxLkv + kGenMaxRope];
+  const int t = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
+  const int n_live = mla_live_rows(p);
+  if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) return;
+  const int i = find_seq_wave(p.qsl, n_live, t);
+  const MlaSeq sp = mla_seq(p, i);
+  if (!sp.live) return;
+  const int lkv = p.lkv, rope = p.rope;
+  const int pos = sp.ctx - sp.q_len + (t - sp.q0);
+  const int k_hi = min(pos + 1, sp.ctx);
+  const int k_lo = (p.window > 0 && pos - p.window + 1 > 0) ? pos - p.window + 1 : 0;
+
+  for (int d = lane; d < lkv; d += 64) q_s[d] = load_elem<QT>(p.q_nope, ((int64_t)t * p.Hq + hq) * lkv + d);
+  for (int d = lane; d < rope; d += 64) q_s[lkv + d] = load_elem<QT>(p.q_pe, ((int64_t)t * p.Hq + hq) * rope + d);
+  __syncthreads();
+
+  const char* pages = (const char*)p.pages;
+  const int32_t* bt = p.block_tables + (int64_t)i * p.M;
+  float m = -INFINITY, l = 0.f;
+  float acc[kGenMaxLkv / 64];
+#pragma unroll
+  for (int k = 0; k < kGenMaxLkv / 64; ++k) acc[k] = 0.f;
+
+  for (int base = k_lo; base < k_hi; base += 64) {
+    const int j = base + lane;
+    float s = -INFINITY;
+    int64_t row = 0;
+    if (j < k_hi) {
+      const int page = min(max(bt[j / p.page_size], 0), p.P - 1);
+      row = (int64_t)page * p.page_stride + (int64_t)(j % p.page_size) * p.token_stride;
+      const void* kp = pages + row;
+      float dot = 0.f;
+      for (int d = 0; d < lkv; ++d) dot = fmaf(q_s[d], load_elem<KVT>(kp, d), dot);
+      for (int d = 0; d < rope; ++d) dot = fmaf(q_s[lkv + d], load_elem<KVT>(kp, p.rope_off + d), dot);
+      s = dot * p.scale;
+      if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
+    }
+    const float m_new = fmaxf(m, wave_max(s));  // finite: lane 0 of every block holds a visible key
+    const float pj = (j < k_hi) ? __expf(s - m_new) : 0.f;
+    const float alpha = __expf(m - m_new);
+    l = l * alpha + wave_sum(pj);
+    m = m_new;
+#pragma unroll
+    for (int k = 0; k < kGenMaxLkv / 64; ++k) acc[k] *= alpha;
+    const int n_keys = min(64, k_hi - base);
+    for (int jj = 0; jj < n_keys; ++jj) {
+      const float w = __shfl(pj, jj);
+      const char* vrow = pages + (int64_t)__shfl((unsigned long long)row, jj);
+#pragma unroll
+      for (int k = 0; k < kGenMaxLkv / 64; ++k) {
+        const int d = lane + 64 * k;
+        if (d < lkv) acc[k] = fmaf(w, load_elem<KVT>(vrow, d), acc[k]);
+      }
+    }
+  }
+  if (p.sinks && l > 0.f) l += expf(p.sinks[hq] - m);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int k = 0; k < kGenMaxLkv / 64; ++k) {
+    const int d = lane + 64 * k;
+    if (d < lkv) {
+      const int64_t o = ((int64_t)t * p.Hq + hq) * lkv + d;
+      const float r = acc[k] * inv;
+      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
+      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
+    }
+  }
+}
+
+// ---- MFMA kernel ----------------------------------------------------------------------------------------------------
+// One LDS DMA of 1 KiB: every lane fetches 16 bytes from base + voff; lane L's bytes land at LDS byte address
+// lds_addr + 16 L.
+__device__ __forceinline__ void mla_dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void mla_wait_loads_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// XOR key (on the low three bits of the 16-byte chunk index) of LDS row r.  Rows are 1152 bytes, so rows of equal
+// parity start in the same bank group and rows of different parity half the banks apart.  The row-wise reads (16 rows,
+// one chunk each) need the eight rows of a parity in eight different chunks; the transposing reads (per half wave 8
+// rows, a pair of chunks each) need the four rows of a parity in four different pairs.  Bits 1-2 from the row's
+// bits 1-2 and bit 0 from its bit 3 give both.
+__device__ __forceinline__ int mla_key(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
+
+constexpr int kMlaWaves = 8;  // waves of an MFMA-kernel workgroup
+
+template <bool CAP>
+__global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p) {
+  constexpr int TT = 32, NW = kMlaWaves, RB = 1;
+  constexpr int LKV = 512, ROPE = 64, DK = LKV + ROPE;
+  constexpr int RKL = DK * 2;            // bytes of a key row in LDS
+  constexpr int CPR = RKL / 16;          // 16-byte chunks per row
+  constexpr int TILE = TT * RKL;         // bytes of a tile
+  constexpr int NINS = TILE / 1024;      // DMA instructions per tile, dealt round-robin to the waves
+  constexpr int NDMA = (NINS + NW - 1) / NW;  // most per wave
+  static_assert(NINS % NW == NW / 2, "the first half of the waves issue NDMA instructions a tile, the others one fewer");
+  constexpr int NSLOT = 3;
+  constexpr int NS = TT / 16;            // 16-key sub-tiles per tile
+  constexpr int DPL = LKV / 16;          // 16-dim row tiles of O^T
+  constexpr int NKK = DK / 32;           // k-steps of the score product
+  constexpr int NKN = LKV / 32;          // of which over the latent part
+  constexpr float kMaxSlack = 8.f;       // how far a score may exceed the softmax reference before it is raised
+  static_assert(NW * RB * 16 == kMlaRows, "merge kernel assumes this row-tile height");
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[NSLOT * TILE];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, g4 = lane >> 4;
+  const int Hq = p.Hq;
+
+  // ---- block -> (sequence, row tile, key chunk) -------------------------------------------------------------
+  const int n_slots = gridDim.x / p.max_chunks;
+  const int slot = blockIdx.x % n_slots;
+  const int chunk = blockIdx.x / n_slots;  // slowest: neighbouring blocks are row tiles of neighbouring sequences
+  const int n_live = mla_live_rows(p);
+  if (n_live <= 0) return;
+  // sequence i starts at slot floor(qsl[i]*Hq/128) + i; find the last sequence starting at or before `slot`
+  int lo_i = 0, hi_i = n_live;
+  while (hi_i - lo_i > 1) {
+    const int mid = (lo_i + hi_i) >> 1;
+    if ((int)(((int64_t)p.qsl[mid] * Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
+  }
+  const int i = lo_i;
+  const MlaSeq sp = mla_seq(p, i);
+  if (!sp.live) return;
+  const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * Hq) / kMlaRows) + i);
+  const int rows_total = sp.q_len * Hq;
+  const int R0 = tile_in_seq * kMlaRows;
+  if (tile_in_seq < 0 || R0 >= rows_total) return;
+
+  const MlaTile mt = mla_tile(p, sp, R0);
+  if (chunk >= mt.n_chunks) return;  // also: queries before position 0 have no keys; such rows stay unwritten
+  const int base_pos = sp.ctx - sp.q_len;
+  const int vis_lo = mt.vis_lo;
+  // the first tile must hold vis_lo, so that rows of it that nobody may see can borrow a visible row's address
+  const int kv_lo = max(mt.kv_lo + chunk * mt.chunk, vis_lo & ~(TT - 1));
+  const int kv_hi = min(mt.kv_hi, mt.kv_lo + (chunk + 1) * mt.chunk);
+  const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
+  const bool single = mt.n_chunks == 1;
+
+  // ---- per row-block lane state ----------------------------------------------------------------------------
+  int row_lo[RB], row_hi[RB];
+  bool row_ok[RB];
+  int out_tok[RB], out_head[RB];
+  bf16x8 qf[RB][NKK];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = R0 + (wave * RB + rb) * 16 + n;
+    row_ok[rb] = row < rows_total;
+    const int r_tok = row_ok[rb] ? row / Hq : (rows_total - 1) / Hq;  // padded rows shadow the last row
+    const int r_head = row_ok[rb] ? row - r_tok * Hq : 0;
+    const int pos = base_pos + r_tok;
+    row_hi[rb] = min(pos + 1, sp.ctx);
+    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+    out_tok[rb] = sp.q0 + r_tok;
+    out_head[rb] = r_head;
+    const int64_t qrow = (int64_t)out_tok[rb] * Hq + r_head;
+    const char* qn = (const char*)p.q_nope + qrow * (LKV * 2);
+    const char* qp = (const char*)p.q_pe + qrow * (ROPE * 2);
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok[rb]) v = kk < NKN ? *(const u32x4*)(qn + (kk * 32 + 8 * g4) * 2) : *(const u32x4*)(qp + ((kk - NKN) * 32 + 8 * g4) * 2);
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  // Use the query registers once here, so that the compiler waits for these loads now and not at their first use
+  // inside the loop, where its wait would also cover every tile in flight.
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = __builtin_bit_cast(u32x4, qf[rb][kk]);
+      asm volatile("" : "+v"(v));
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  // a wave whose row blocks all lie past the sequence's rows only helps with the loads
+  const bool wave_active = (R0 + wave * RB * 16) < rows_total;
+
+  // ---- tile loads --------------------------------------------------------------------------------------------
+  // The tile is 36 KiB of LDS in row order (72 chunks a row); DMA instruction u = wave + 4 j fills its bytes
+  // [1024 u, 1024 u + 1024): lane L holds chunk c = 64 u + L = (row c / 72, LDS chunk c % 72) and fetches the global
+  // chunk that the swizzle maps there.  The block table is read through the constant address space: it does not change
+  // while the kernel runs, and only so may the compiler keep these loads scalar after the assembly statements.
+  typedef const __attribute__((address_space(4))) int32_t* ConstI32;
+  ConstI32 bt = (ConstI32)(uintptr_t)(p.block_tables + (int64_t)i * p.M);
+  const char* pages = (const char*)p.pages;
+  const int pg = p.page_size;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
+  // (row, global chunk) of DMA instruction j for this lane; recomputed at every issue -- a few integer instructions
+  // against the hundred-odd MFMAs of a tile -- rather than held in eighteen registers
+  auto dma_row = [&](int j) -> int { return (64 * (wave + NW * j) + lane) / CPR; };
+  auto dma_chunk = [&](int j, int r) -> int { return ((64 * (wave + NW * j) + lane) - r * CPR) ^ mla_key(r); };
+  const bool dma_full = wave < NINS % NW;  // this wave issues NDMA instructions per tile (else NDMA - 1)
+  int cur_idx = kv_lo / pg;
+  int cur_off = kv_lo - cur_idx * pg;
+  int cur_tb = kv_lo;
+  int cur_slot = 0;
+  auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
+  int cur_page_raw = load_page(cur_idx);
+  auto issue = [&]() __attribute__((always_inline)) {
+    const int cur_page = min(max(cur_page_raw, 0), p.P - 1);
+    const char* base = pages + (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride;
+    const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
+    const uint32_t dst = lds_base + (uint32_t)cur_slot * TILE + (uint32_t)wave * 1024u;
+    const uint32_t ts = (uint32_t)p.token_stride;
+    if (!edge) {
+#pragma unroll
+      for (int j = 0; j < NDMA; ++j) {
+        if (j == NDMA - 1 && !dma_full) break;
+        const int r = dma_row(j);
+        mla_dma16(dst + j * NW * 1024, (uint32_t)r * ts + (uint32_t)(dma_chunk(j, r) << 4), base);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NDMA; ++j) {  // keys nobody may see: any visible row's bytes
+        if (j == NDMA - 1 && !dma_full) break;
+        const int r = dma_row(j);
+        const int rv = min(max(cur_tb + r, vis_lo), sp.ctx - 1) - cur_tb;
+        mla_dma16(dst + j * NW * 1024, (uint32_t)rv * ts + (uint32_t)(dma_chunk(j, r) << 4), base);
+      }
+    }
+    cur_tb += TT;
+    cur_off += TT;
+    if (cur_off >= pg) {
+      cur_off -= pg;
+      ++cur_idx;
+    }
+    cur_slot = (cur_slot == NSLOT - 1) ? 0 : cur_slot + 1;
+    cur_page_raw = load_page(cur_idx);
+  };
+
+  const float cap_out = p.softcap * 1.4426950408889634f;
+  const float cap_in = CAP ? p.scale / p.softcap : 0.f;
+  const float sc_mul = CAP ? cap_out : p.scale_log2;
+
+  float m_run[RB], l_run[RB];
+  f32x4 o_acc[RB][DPL];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    m_run[rb] = -INFINITY;
+    l_run[rb] = 0.f;
+#pragma unroll
+    for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // per-lane LDS offsets of the operand reads inside a tile
+  int k_base[NS][2];  // row-wise read of key st*16 + n, k-step parity
+#pragma unroll
+  for (int st = 0; st < NS; ++st)
+#pragma unroll
+    for (int par = 0; par < 2; ++par) k_base[st][par] = (st * 16 + n) * RKL + (((4 * par + g4) ^ mla_key(st * 16 + n)) << 4);
+  // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16 (key 4g4 + l/4,
+  // dims d0 + 4(l%4)..) and receives the transposed column: for dim d0 + (l&15) the values of keys 4g4..4g4+3
+  const int tr_key = 4 * g4 + (n >> 2);  // key (within a 16-key sub-tile) this lane addresses in a transposing read
+  const int tr_byte = (n & 3) * 8;       // byte offset of its 4 dims inside the 32-byte row-tile span
+  int v_base[NS][4];  // transposing read of sub-tile st, row tile rt & 3
+#pragma unroll
+  for (int st = 0; st < NS; ++st)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int tk = st * 16 + tr_key;
+      v_base[st][q] = tk * RKL + (((2 * q + (tr_byte >> 4)) ^ mla_key(tk)) << 4) + (tr_byte & 15);
+    }
+
+  issue();
+  if (n_tiles > 1) issue();
+  int rd_slot = 0;
+  for (int tile = 0; tile < n_tiles; ++tile) {
+    // tile `tile` has landed (tile + 1 may still be in flight), and every wave is done with tile - 1
+    if (tile + 1 >= n_tiles) mla_wait_loads_and_barrier<0>();
+    else if (dma_full) mla_wait_loads_and_barrier<NDMA>();
+    else mla_wait_loads_and_barrier<NDMA - 1>();
+    if (tile + 2 < n_tiles) issue();  // into the slot of tile - 1
+    const unsigned char* lds_t = lds_all + rd_slot * TILE;
+    rd_slot = (rd_slot == NSLOT - 1) ? 0 : rd_slot + 1;
+    if (!wave_active) continue;
+    const int tb = kv_lo + tile * TT;
+
+    // ---- S^T = K . Q^T for both row blocks (K operands shared) ---------------------------------------------
+    f32x4 s_acc[RB][NS];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int st = 0; st < NS; ++st) s_acc[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+#pragma unroll
+      for (int kk = 0; kk < NKK; ++kk) {
+        // chunk 4 kk + g4 under the key: only its low three bits move, so a k-step's address is one of two
+        // per-lane bases (kk even / odd) plus a constant
+        const u32x4 a = *(const u32x4*)(lds_t + k_base[st][kk & 1] + (kk >> 1) * 128);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+          s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
+      }
+    }
+
+    // ---- online softmax per row block ------------------------------------------------------------------------
+    // The reference every probability of a row is taken against need not be the exact running maximum: any common
+    // value works as long as exp2 stays in range.  It is raised -- the lanes of a row agree on the new maximum and
+    // everything accumulated so far is scaled down -- only when some key of the tile exceeds it by more than kMaxSlack
+    // (log2 units).  After the first tiles of a sequence that is rare, which matters here: the 256 accumulators of a
+    // wave live in the accumulation registers, which the vector ALU reaches only through moves.
+    uint32_t pfrag[RB][NS][2];
+    {
+      float lmx[RB];
+      bool grow = false;
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        lmx[rb] = -INFINITY;
+#pragma unroll
+        for (int st = 0; st < NS; ++st)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            float sv = s_acc[rb][st][j];
+            if constexpr (CAP) sv = fast_tanh(sv * cap_in);
+            const int tok = tb + st * 16 + 4 * g4 + j;
+            sv = (tok >= row_lo[rb] && tok < row_hi[rb]) ? sv : -INFINITY;
+            s_acc[rb][st][j] = sv;
+            lmx[rb] = fmaxf(lmx[rb], sv);
+          }
+        lmx[rb] *= sc_mul;  // sc_mul > 0: scaling commutes with the maximum
+        grow |= lmx[rb] > m_run[rb] + kMaxSlack;
+      }
+      if (__any(grow)) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const float m_new = fmaxf(m_run[rb], xor32_max(xor16_max(lmx[rb])));
+          const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+          float alpha = __builtin_amdgcn_exp2f(m_run[rb] - m_use);
+          m_run[rb] = m_new;
+          // opaque multiplications: the compiler does not pad the distance this chip wants between a transcendental
+          // instruction and a reader of its result, so the padding is put here by hand
+          asm volatile("s_nop 1" : "+v"(alpha));
+          asm("v_mul_f32 %0, %1, %0" : "+v"(l_run[rb]) : "v"(alpha));
+          if (tile > 0) {  // in a chunk's first tile nothing has been accumulated yet
+#pragma unroll
+            for (int rt = 0; rt < DPL; ++rt) o_acc[rb][rt] *= alpha;
+          }
+        }
+      }
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const float m_use = (m_run[rb] == -INFINITY) ? 0.f : m_run[rb];
+        float psum = 0.f;
+#pragma unroll
+        for (int st = 0; st < NS; ++st) {
+          float pr[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[rb][st][j], sc_mul, -m_use));
+            psum += pr[j];
+          }
+          pfrag[rb][st][0] = pack_bf16(pr[0], pr[1]);
+          pfrag[rb][st][1] = pack_bf16(pr[2], pr[3]);
+        }
+        l_run[rb] += psum;
+      }
+    }
+
+    // ---- O^T += V^T . P^T: the values are the first LKV elements of the same rows -----------------------------
+#pragma unroll
+    for (int rt = 0; rt < DPL; ++rt) {
+      // row tile rt spans chunks 2 rt, 2 rt + 1: under the key one of four per-lane bases (rt & 3) plus a constant
+      const unsigned char* p0 = lds_t + v_base[0][rt & 3] + (rt >> 2) * 128;
+      const unsigned char* p1 = lds_t + v_base[1][rt & 3] + (rt >> 2) * 128;
+      const u32x2 a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0));
+      const u32x2 a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p1));
+      const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
+        o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
+                                                                o_acc[rb][rt], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- epilogue ---------------------------------------------------------------------------------------------------
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    if (!row_ok[rb]) continue;
+    if (single) {
+      float l_fin = l_tot;
+      if (p.sinks != nullptr && l_tot > 0.f)
+        l_fin += __builtin_amdgcn_exp2f(__builtin_fmaf(p.sinks[out_head[rb]], 1.4426950408889634f, -m_run[rb]));
+      const float inv = l_fin > 0.f ? 1.f / l_fin : 0.f;
+      uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * Hq + out_head[rb]) * LKV + 4 * g4;
+#pragma unroll
+      for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
+        const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                         pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+        *(u32x2*)(orow + 16 * rt) = w;
+      }
+    } else {
+      const int64_t pslot = ((int64_t)chunk * p.T + out_tok[rb]) * Hq + out_head[rb];
+      float* prow = p.part_o + pslot * LKV + 4 * g4;
+#pragma unroll
+      for (int rt = 0; rt < DPL; ++rt) *(f32x4*)(prow + 16 * rt) = o_acc[rb][rt];
+      if (g4 == 0) {
+        p.part_ml[pslot * 2 + 0] = m_run[rb];
+        p.part_ml[pslot * 2 + 1] = l_tot;
+      }
+    }
+  }
+}
+
+// ---- merge: combines the key chunks of a row, and zero-fills the rows of padded tokens -----------------------------
+template <int QT>
+__global__ __launch_bounds__(256) void mla_merge_kernel(MlaParams p) {
+  constexpr int NK = kGenMaxLkv / 64;
+  const int lane = threadIdx.x & 63;
+  const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= p.T * p.Hq) return;
+  const int t = pair / p.Hq, hq = pair - t * p.Hq;
+  const int n_live = mla_live_rows(p);
+  const int lkv = p.lkv;
+  bool zero = false;
+  int n_pieces = 0;
+  if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) {
+    zero = true;
+  } else {
+    const int i = find_seq_wave(p.qsl, n_live, t);
+    const MlaSeq sp = mla_seq(p, i);
+    if (!sp.live) zero = true;
+    else if (p.mfma && p.max_chunks > 1) {
+      const int row = (t - sp.q0) * p.Hq + hq;
+      n_pieces = mla_tile(p, sp, (row / kMlaRows) * kMlaRows).n_chunks;
+    }
+  }
+  const bool merge = n_pieces > 1;
+  if (!zero && !merge) return;
+  float acc[NK];
+#pragma unroll
+  for (int k = 0; k < NK; ++k) acc[k] = 0.f;
+  float inv = 0.f;
+  if (merge) {
+    const int64_t slot0 = (int64_t)t * p.Hq + hq;
+    const int64_t stride = (int64_t)p.T * p.Hq;
+    float m = -INFINITY;
+    for (int c = lane; c < n_pieces; c += 64) m = fmaxf(m, p.part_ml[(slot0 + c * stride) * 2]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    const float m_use = (m == -INFINITY) ? 0.f : m;
+    float l = 0.f;
+    for (int c = 0; c < n_pieces; ++c) {  // n_pieces <= kMlaMaxChunks
+      const float2 ml = *(const float2*)(p.part_ml + (slot0 + c * stride) * 2);
+      const float w = __builtin_amdgcn_exp2f(ml.x - m_use);
+      l += w * ml.y;
+      const float* row = p.part_o + (slot0 + c * stride) * lkv;
+#pragma unroll
+      for (int k = 0; k < NK; ++k) {
+        const int d = lane + 64 * k;
+        if (d < lkv) acc[k] = fmaf(w, row[d], acc[k]);
+      }
+    }
+    if (p.sinks != nullptr && l > 0.f) l += __builtin_amdgcn_exp2f(__builtin_fmaf(p.sinks[hq], 1.4426950408889634f, -m_use));
+    inv = l > 0.f ? 1.f / l : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    const int d = lane + 64 * k;
+    if (d < lkv) {
+      const int64_t o = ((int64_t)t * p.Hq + hq) * lkv + d;
+      const float r = acc[k] * inv;
+      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
+      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
+    }
+  }
+}
+
+template <int QT>
+int launch_generic_q(hipStream_t stream, const MlaParams& p) {
+  dim3 grid(p.T, p.Hq), block(64);
+  switch (p.kv_dtype) {
+    case RPA_F32: hipLaunchKernelGGL((mla_generic_kernel<QT, RPA_F32>), grid, block, 0, stream, p); break;
+    case RPA_BF16: hipLaunchKernelGGL((mla_generic_kernel<QT, RPA_BF16>), grid, block, 0, stream, p); break;
+    default: return (int)hipErrorInvalidValue;
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int launch_mla_scatter(hipStream_t stream, const MlaParams& p) {
+  const int blocks = (p.T + 3) / 4;
+  if (p.kv_dtype == RPA_F32) hipLaunchKernelGGL((mla_scatter_kernel<uint32_t>), dim3(blocks), dim3(256), 0, stream, p);
+  else if (p.kv_dtype == RPA_BF16) hipLaunchKernelGGL((mla_scatter_kernel<uint16_t>), dim3(blocks), dim3(256), 0, stream, p);
+  else return (int)hipErrorInvalidValue;
+  return (int)hipGetLastError();
+}
+
+int launch_mla_generic(hipStream_t stream, const MlaParams& p) {
+  if (p.lkv > kGenMaxLkv || p.rope > kGenMaxRope) return (int)hipErrorInvalidValue;
+  return p.q_dtype == RPA_F32 ? launch_generic_q<RPA_F32>(stream, p) : launch_generic_q<RPA_BF16>(stream, p);
+}
+
+// bf16 queries and pages of the one shape every model with this cache uses (latent 512, rope 64, the rope key right
+// behind the latent part), pages a multiple of the 32-key tile, and page rows a 32-bit byte offset can address
+bool mla_mfma_supported(const MlaParams& p) {
+  return p.q_dtype == RPA_BF16 && p.kv_dtype == RPA_BF16 && p.lkv == 512 && p.rope == 64 && p.rope_off == 512 &&
+         p.page_size % 32 == 0 && (p.token_stride & 15) == 0 && (int64_t)32 * p.token_stride < ((int64_t)1 << 31);
+}
+
+int launch_mla_mfma(hipStream_t stream, const MlaParams& p) {
+  const int64_t slots = ((int64_t)p.T * p.Hq) / kMlaRows + p.S;  // upper bound on row tiles of the batch
+  const int64_t blocks = slots * p.max_chunks;
+  if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
+  if (p.softcap > 0.f) hipLaunchKernelGGL((mla_attn_kernel<true>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
+  else hipLaunchKernelGGL((mla_attn_kernel<false>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+int launch_mla_merge(hipStream_t stream, const MlaParams& p) {
+  if (p.lkv > kGenMaxLkv) return (int)hipErrorInvalidValue;
+  const int blocks = (int)(((int64_t)p.T * p.Hq + 3) / 4);
+  if (p.q_dtype == RPA_F32) hipLaunchKernelGGL((mla_merge_kernel<RPA_F32>), dim3(blocks), dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL((mla_merge_kernel<RPA_BF16>), dim3(blocks), dim3(256), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+}  // namespace rpa

@@ -307,3 +307,87 @@ def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, 
             _i32(query_start_loc, "query_start_loc"), _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(),
             ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap, aux_ptr))
     return out, kv_pages, kv_scales
+
+
+def mla_row_geometry(kv_pages: torch.Tensor) -> tuple[int, int, int]:
+    """(P, page_size, row_elems) of a latent page pool: ``[P, pg, row]`` or the reference's
+    ``[P, pg / packing, packing, row]`` (easydel/caching/mla_ragged_page/cache.py:270-287), the same bytes."""
+    if kv_pages.ndim == 3:
+        return kv_pages.shape[0], kv_pages.shape[1], kv_pages.shape[2]
+    if kv_pages.ndim == 4:
+        return kv_pages.shape[0], kv_pages.shape[1] * kv_pages.shape[2], kv_pages.shape[3]
+    raise ValueError(f"latent kv_pages must be 3-D or 4-D, got shape {tuple(kv_pages.shape)}")
+
+
+def _mla_shapes(queries_nope, queries_pe, kv_pages, context_lens, block_tables):
+    if queries_nope.ndim != 3 or queries_pe.ndim != 3 or queries_nope.shape[:2] != queries_pe.shape[:2]:
+        raise ValueError("`queries_nope` and `queries_pe` must share [total_tokens, num_q_heads]. "
+                         f"Got {tuple(queries_nope.shape)} vs {tuple(queries_pe.shape)}.")
+    T, Hq, lkv = queries_nope.shape
+    rope = queries_pe.shape[2]
+    P, pg, row = mla_row_geometry(kv_pages)
+    S = context_lens.shape[0]
+    if block_tables.numel() % S:
+        raise ValueError("block_tables size is not a multiple of the number of sequence rows")
+    return T, Hq, lkv, rope, P, pg, row, S, block_tables.numel() // S
+
+
+def mla_page_scatter(keys_values, keys_pe, kv_pages, context_lens, block_tables, query_start_loc, num_seqs):
+    """In-place write of latent rows and rope keys: tokens of sequence i land at positions
+    ``[ctx_i - q_len_i, ctx_i)`` of its pages (latent at 0, rope key at the padded latent width, padding zeroed)."""
+    lib = _lib.load()
+    if keys_values.dtype != kv_pages.dtype or keys_pe.dtype != kv_pages.dtype:
+        raise TypeError(f"keys_values/keys_pe dtype {keys_values.dtype}/{keys_pe.dtype} must equal the cache dtype {kv_pages.dtype}")
+    if keys_values.ndim != 2 or keys_pe.ndim != 2 or keys_values.shape[0] != keys_pe.shape[0]:
+        raise ValueError(f"keys_values [T, kv_lora_rank] and keys_pe [T, rope] expected, got {tuple(keys_values.shape)}, {tuple(keys_pe.shape)}")
+    T, lkv = keys_values.shape
+    rope = keys_pe.shape[1]
+    P, pg, row = mla_row_geometry(kv_pages)
+    S = context_lens.shape[0]
+    M = block_tables.numel() // S
+    if T == 0:
+        return kv_pages
+    _dev(kv_pages, "kv_pages")
+    with torch.cuda.device(kv_pages.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_mla_page_scatter(
+            _stream(kv_pages), _dev(keys_values, "keys_values"), _dev(keys_pe, "keys_pe"), _dev(kv_pages, "kv_pages"),
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, lkv, rope, row, keys_values.element_size()))
+    return kv_pages
+
+
+def mla_ragged_paged_attention(queries_nope, queries_pe, keys_values, keys_pe, kv_pages, context_lens, block_tables,
+                               query_start_loc, distribution, *, softmax_scale=None, sliding_window=None,
+                               logits_soft_cap=None, softmax_aux=None, out=None):
+    """Multi-latent attention over latent pages, fused with the write of the new rows (``keys_values`` may be None:
+    the pages are then read as they are).  Returns ``(out [T, Hq, kv_lora_rank], kv_pages)``."""
+    lib = _lib.load()
+    T, Hq, lkv, rope, P, pg, row, S, M = _mla_shapes(queries_nope, queries_pe, kv_pages, context_lens, block_tables)
+    if queries_pe.dtype != queries_nope.dtype:
+        raise TypeError(f"queries_pe dtype {queries_pe.dtype} != queries_nope dtype {queries_nope.dtype}")
+    if keys_values is not None:
+        if keys_pe is None:
+            raise ValueError("multi_latent_ragged_page_attention requires `keys_pe`. Pass it as `keys_pe=` (or `k_pe=`).")
+        if keys_values.dtype != kv_pages.dtype or keys_pe.dtype != kv_pages.dtype:
+            raise TypeError(f"keys_values/keys_pe dtype {keys_values.dtype}/{keys_pe.dtype} must equal the cache dtype {kv_pages.dtype}")
+        if tuple(keys_values.shape) != (T, lkv) or tuple(keys_pe.shape) != (T, rope):
+            raise ValueError(f"keys_values {tuple(keys_values.shape)} / keys_pe {tuple(keys_pe.shape)} must be [{T}, {lkv}] / [{T}, {rope}]")
+    if out is None:
+        out = torch.empty_like(queries_nope)
+    if T == 0:
+        return out, kv_pages
+    qd, kd = dtype_tag(queries_nope.dtype), dtype_tag(kv_pages.dtype)
+    scale = float(lkv + rope) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    window = int(sliding_window) if sliding_window else 0
+    cap = float(logits_soft_cap) if logits_soft_cap else 0.0
+    aux, aux_ptr = _sinks(softmax_aux, Hq, queries_nope.device)
+    ws = _workspace(queries_nope.device, int(lib.rpa_mla_workspace_bytes(T, S, M, pg, Hq, lkv, qd, kd)))
+    with torch.cuda.device(queries_nope.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_mla_ragged_paged_attention(
+            _stream(queries_nope), _dev(queries_nope, "queries_nope"), _dev(queries_pe, "queries_pe"),
+            None if keys_values is None else _dev(keys_values, "keys_values"),
+            None if keys_values is None else _dev(keys_pe, "keys_pe"), _dev(kv_pages, "kv_pages"),
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
+            T, S, M, P, pg, Hq, lkv, rope, row, qd, kd, scale, window, cap, aux_ptr))
+    return out, kv_pages

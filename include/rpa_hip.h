@@ -197,6 +197,55 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
                                   const float* softmax_aux);
 
 /*
+ * Multi-latent attention (MLA) over latent ragged pages.  Replaces
+ * ejkernel.modules.multi_latent_ragged_page_attention (and its _v2 twin, same operands) as called at
+ * easydel/operations/kernels/multi_latent_ragged_page_attention.py:495-511, 611-624 (v1) and :1019-1030, 1090-1101 (v2).
+ * Fused like the v3 operation: the new rows are written into the pages, then every query attends.
+ *
+ *   queries_nope  device, [T][Hq][kv_lora_rank], q_dtype: queries already multiplied by the key half of the
+ *                 up-projection (the caller's "weight absorption", layers/attention/_unified.py:1292-1298)
+ *   queries_pe    device, [T][Hq][qk_rope_head_dim], q_dtype
+ *   keys_values   device, [T][kv_lora_rank], already in the pages' element type, or NULL: the pages are read as they
+ *                 are (then keys_pe is ignored)
+ *   keys_pe       device, [T][qk_rope_head_dim], pages' element type
+ *   kv_pages      device, [P][page_size][row_elems] (the reference's
+ *                 [P][page_size / packing][packing][kv_dim_padded], caching/mla_ragged_page/cache.py:270-287, is the
+ *                 same bytes): per token the latent row at [0, kv_lora_rank), the rope key at
+ *                 [align128(kv_lora_rank), + qk_rope_head_dim), padding zeroed by the write.  row_elems is at least
+ *                 align128(kv_lora_rank) + qk_rope_head_dim; the reference uses align128 of both parts (640 for 512 + 64)
+ *   distribution  device, int32 [3]; only [2], the number of live rows, is read (the reference passes [0, 0, total],
+ *                 multi_latent_ragged_page_attention.py:376-378)
+ *   out           device, [T][Hq][kv_lora_rank], q_dtype: softmax-weighted sums of latent rows (the caller applies the
+ *                 value half of the up-projection, _unified.py:1366-1371)
+ *   workspace     device scratch of at least rpa_mla_workspace_bytes(...) bytes
+ *   softmax_scale as passed by the caller: (qk_nope_head_dim + qk_rope_head_dim) ** -0.5 (_unified.py:1310)
+ * q_dtype RPA_F32 or RPA_BF16; kv_dtype RPA_F32 or RPA_BF16; kv_lora_rank <= 512, qk_rope_head_dim <= 256, both
+ * multiples of 8.  bf16 with kv_lora_rank 512, rope 64 and page_size % 32 == 0 runs on the matrix cores; every other
+ * combination on the fp32 kernel.  Window, soft cap, softmax_aux, padding and error behaviour as for
+ * rpa_ragged_paged_attention.
+ */
+int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope, const void* queries_pe,
+                                   const void* keys_values, const void* keys_pe, void* kv_pages,
+                                   const int32_t* context_lens, const int32_t* block_tables,
+                                   const int32_t* query_start_loc, const int32_t* distribution, void* out,
+                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P, int page_size,
+                                   int Hq, int kv_lora_rank, int qk_rope_head_dim, int row_elems, int q_dtype,
+                                   int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
+                                   const float* softmax_aux);
+
+/* Workspace the call above needs, from the static bounds alone. */
+size_t rpa_mla_workspace_bytes(int T, int S, int M, int page_size, int Hq, int kv_lora_rank, int q_dtype, int kv_dtype);
+
+/*
+ * The write half of the MLA operation on its own (same operands and placement as above; num_seqs: device int32 [1]).
+ * elem_bytes 2 or 4.
+ */
+int rpa_mla_page_scatter(rpa_stream_t stream, const void* keys_values, const void* keys_pe, void* kv_pages,
+                         const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
+                         const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int kv_lora_rank,
+                         int qk_rope_head_dim, int row_elems, int elem_bytes);
+
+/*
  * Measurement aid with no counterpart in the reference: copies `bytes` (a multiple of 16, both
  * pointers 16-byte aligned) with a plain vector copy kernel.  Profiling a known-size copy next to
  * the attention kernels gives the factor that turns raw HBM traffic counters into bytes.

@@ -46,6 +46,12 @@ Pinning status
   invariants in ``tests/test_oracle_formats.py`` (round-trip error bounds, monotone scales,
   equivalence with one-shot quantisation when nothing is re-coded, placement equal to the
   unquantised ragged write).
+* ``mla_ragged_paged_attention_ref`` / ``mla_page_scatter_ref``: the arithmetic lives in ejkernel and the
+  reference holds no vector for it: "parity unpinned" against ejkernel.  Pinned in ``tests/test_oracle_mla.py`` to the
+  reference's own non-absorbed branch of the same layer (keys and values decompressed through the up-projection,
+  then ordinary attention, ``layers/attention/_unified.py:1240-1248, 1380-1395``), i.e. to
+  ``ragged_paged_attention_ref`` on decompressed pages, and to the reductions of that function's tests.
+  ``mla_page_layout_ref`` is pinned by the shape arithmetic of ``caching/mla_ragged_page/cache.py:198-201``.
 """
 
 from __future__ import annotations
@@ -408,4 +414,110 @@ def ragged_paged_attention_ref(query, kv_pages, context_lens, block_tables, quer
             if sinks is not None:
                 denom = denom + np.exp(sinks[h] - m)
             out[q0:q1, h, :] = (p @ v) / np.where(denom > 0, denom, 1.0)
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# Multi-latent attention (MLA) over latent ragged pages
+# --------------------------------------------------------------------------------------
+def mla_page_layout_ref(kv_lora_rank: int, qk_rope_head_dim: int, page_size: int, bits: int = 16) -> dict:
+    """Shape of the latent page pool (caching/mla_ragged_page/cache.py:198-201, 250-287).
+
+    One row per token, no head axis: the latent ``kv_lora_rank`` values and the rope key ``qk_rope_head_dim`` values,
+    each padded to a multiple of 128 on its own (``:257-258``); tokens are packed ``32 // bits`` to a storage row
+    (``:199-200``), which in memory is the same as ``[P, page_size', row]`` with ``page_size'`` rounded up to the packing.
+    The rope part is taken to start at the padded latent width (the reference states only the total; where ejkernel
+    puts the parts inside a row cannot be read from the tree, and for ``kv_lora_rank`` a multiple of 128 -- every model
+    that uses the operation has 512 -- the two readings coincide).
+    """
+    packing = 32 // int(bits)
+    lkv_pad = -(-int(kv_lora_rank) // 128) * 128
+    rope_pad = -(-int(qk_rope_head_dim) // 128) * 128
+    per = -(-int(page_size) // packing)
+    return dict(kv_packing=packing, page_size_per_kv_packing=per, kv_dim_padded=lkv_pad + rope_pad, rope_offset=lkv_pad,
+                shape_tail=(per, packing, lkv_pad + rope_pad))
+
+
+def mla_page_scatter_ref(keys_values, keys_pe, kv_pages, context_lens, block_tables, query_start_loc, num_seqs) -> np.ndarray:
+    """The write half of the MLA operation (call site multi_latent_ragged_page_attention.py:495-511, 611-624).
+
+    ``kv_pages [P, pg, row]``; sequence ``i`` writes the latent rows ``keys_values[qsl[i]:qsl[i+1]]`` and the rope keys
+    ``keys_pe[...]`` to token positions ``[ctx_i - q_len_i, ctx_i)`` of its pages (the positions of the fused v3 write,
+    the operation takes the same metadata): latent at ``[0, lkv)``, rope key at ``[rope_offset, rope_offset + rope)``,
+    the padding of a written row set to zero.
+    """
+    pages = np.array(kv_pages, copy=True)
+    pg, row = pages.shape[1], pages.shape[2]
+    lkv, rope = keys_values.shape[1], keys_pe.shape[1]
+    off = -(-lkv // 128) * 128
+    assert off + rope <= row
+    bt = np.asarray(block_tables).reshape(len(context_lens), -1)
+    for i in range(int(np.asarray(num_seqs).reshape(-1)[0])):
+        q0, q1 = int(query_start_loc[i]), int(query_start_loc[i + 1])
+        ctx = int(context_lens[i])
+        for r in range(q1 - q0):
+            pos = ctx - (q1 - q0) + r
+            if pos < 0:
+                continue
+            page = int(bt[i, pos // pg])
+            pages[page, pos % pg, :] = 0
+            pages[page, pos % pg, :lkv] = keys_values[q0 + r]
+            pages[page, pos % pg, off:off + rope] = keys_pe[q0 + r]
+    return pages
+
+
+def mla_ragged_paged_attention_ref(queries_nope, queries_pe, kv_pages, context_lens, block_tables, query_start_loc,
+                                   num_seqs, *, kv_lora_rank, qk_rope_head_dim, softmax_scale=None, sliding_window=None,
+                                   logits_soft_cap=None, softmax_aux=None) -> np.ndarray:
+    """Multi-latent attention over latent pages in float64 (operation called at
+    multi_latent_ragged_page_attention.py:495-511; inputs and output as its caller builds and consumes them,
+    layers/attention/_unified.py:1280-1375).
+
+    ``queries_nope [T, Hq, lkv]`` are the queries already multiplied by the key half of the up-projection ("weight
+    absorption", ``_unified.py:1292-1298``), ``queries_pe [T, Hq, rope]`` their rotary part; every head reads the same
+    row per token: score = ``scale * (q_nope . latent + q_pe . k_pe)``, the values are the latent rows themselves, and the
+    output ``[T, Hq, lkv]`` is the softmax-weighted sum of latent rows, which the caller multiplies by the value half
+    of the up-projection (``:1366-1371``).  Masking, window, soft cap, sinks, positions and padding as in
+    ``ragged_paged_attention_ref``.  ``softmax_scale=None`` means ``(lkv + rope) ** -0.5`` here; the caller always
+    passes ``(qk_nope_head_dim + qk_rope_head_dim) ** -0.5`` (``:1310``).
+    """
+    qn = np.asarray(queries_nope, dtype=np.float64)
+    qp = np.asarray(queries_pe, dtype=np.float64)
+    pages = np.asarray(kv_pages, dtype=np.float64)
+    n_tok, hq, lkv = qn.shape
+    rope = qp.shape[2]
+    assert lkv == kv_lora_rank and rope == qk_rope_head_dim
+    off = -(-lkv // 128) * 128
+    pg = pages.shape[1]
+    scale = float(lkv + rope) ** -0.5 if softmax_scale is None else float(softmax_scale)
+    bt = np.asarray(block_tables).reshape(len(context_lens), -1)
+    out = np.zeros((n_tok, hq, lkv), dtype=np.float64)
+    sinks = None if softmax_aux is None else np.asarray(softmax_aux, dtype=np.float64).reshape(-1)
+    for i in range(int(np.asarray(num_seqs).reshape(-1)[0])):
+        q0, q1 = int(query_start_loc[i]), int(query_start_loc[i + 1])
+        ctx, q_len = int(context_lens[i]), q1 - q0
+        if q_len <= 0 or ctx <= 0:
+            continue
+        n_pages = -(-ctx // pg)
+        seq = pages[bt[i, :n_pages]].reshape(n_pages * pg, -1)[:ctx]
+        latent, k_pe = seq[:, :lkv], seq[:, off:off + rope]
+        pos = ctx - q_len + np.arange(q_len)
+        j = np.arange(ctx)
+        visible = j[None, :] <= pos[:, None]
+        if sliding_window is not None and int(sliding_window) > 0:
+            visible &= j[None, :] > (pos[:, None] - int(sliding_window))
+        for h in range(hq):
+            s = (qn[q0:q1, h, :] @ latent.T + qp[q0:q1, h, :] @ k_pe.T) * scale
+            if logits_soft_cap is not None and float(logits_soft_cap) > 0:
+                s = float(logits_soft_cap) * np.tanh(s / float(logits_soft_cap))
+            s = np.where(visible, s, -np.inf)
+            m = s.max(axis=1, keepdims=True)
+            if sinks is not None:
+                m = np.maximum(m, sinks[h])
+            m = np.where(np.isfinite(m), m, 0.0)
+            p = np.exp(s - m)
+            denom = p.sum(axis=1, keepdims=True)
+            if sinks is not None:
+                denom = denom + np.exp(sinks[h] - m)
+            out[q0:q1, h, :] = (p @ latent) / np.where(denom > 0, denom, 1.0)
     return out

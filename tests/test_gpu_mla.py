@@ -1,0 +1,198 @@
+"""Parity of the multi-latent attention entry point (rpa_mla_ragged_paged_attention, through the C ABI) against the
+numpy oracle: the fused write bit-exact, the attention output to 1e-5 (fp32) / 2e-2 max-abs, 5e-3 mean-abs (bf16)."""
+
+import numpy as np
+import pytest
+
+import rpa_testlib as tl
+from rpa_testlib import BF16, F32, orc
+
+pytestmark = pytest.mark.gpu
+
+
+class MlaBatch:
+    pass
+
+
+def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64, dtype=BF16, pad_rows=0, pad_tokens=0,
+                   row=None, max_pages=None):
+    rng = np.random.default_rng(seed)
+    ctx_lens = np.asarray(ctx_lens, np.int32)
+    q_lens = np.asarray(q_lens, np.int32)
+    n = len(ctx_lens)
+    b = MlaBatch()
+    lay = orc.mla_page_layout_ref(lkv, rope, page_size)
+    b.row = row or lay["kv_dim_padded"]
+    b.off = lay["rope_offset"]
+    b.Hq, b.lkv, b.rope, b.page_size, b.n, b.q_dtype = Hq, lkv, rope, page_size, n, dtype
+    need = [-(-int(c) // page_size) for c in ctx_lens]
+    b.S = n + pad_rows
+    b.M = max_pages or max(max(need), 1)
+    b.P = sum(need) + 5
+    perm = rng.permutation(np.arange(1, b.P))
+    bt = np.zeros((b.S, b.M), np.int32)
+    k = 0
+    for i, m in enumerate(need):
+        bt[i, :m] = perm[k:k + m]
+        k += m
+    b.block_tables = bt
+    b.context_lens = np.zeros(b.S, np.int32)
+    b.context_lens[:n] = ctx_lens
+    qsl = np.zeros(b.S + 1, np.int32)
+    qsl[1:n + 1] = np.cumsum(q_lens)
+    qsl[n + 1:] = qsl[n]
+    b.query_start_loc = qsl
+    b.T = int(qsl[n]) + pad_tokens
+    b.distribution = np.array([0, 0, n], np.int32)
+    b.num_seqs = np.array([n], np.int32)
+
+    def enc(x):
+        if dtype == BF16:
+            raw = orc.f32_to_bf16_bits(x.astype(np.float32))
+            return raw, orc.bf16_bits_to_f32(raw).astype(np.float64)
+        x = x.astype(np.float32)
+        return x, x.astype(np.float64)
+
+    b.qn_raw, b.qn_val = enc(rng.standard_normal((b.T, Hq, lkv)))
+    b.qp_raw, b.qp_val = enc(rng.standard_normal((b.T, Hq, rope)))
+    b.kv_raw, b.kv_val = enc(rng.standard_normal((b.T, lkv)))
+    b.pe_raw, b.pe_val = enc(rng.standard_normal((b.T, rope)))
+    b.pages_raw, b.pages_val = enc(rng.standard_normal((b.P, page_size, b.row)))  # padding holds noise: never read
+    return b
+
+
+def mla_oracle(b, *, fused=True, **kw):
+    pages = b.pages_val
+    if fused:
+        pages = orc.mla_page_scatter_ref(b.kv_val, b.pe_val, pages, b.context_lens, b.block_tables, b.query_start_loc, b.num_seqs)
+    out = orc.mla_ragged_paged_attention_ref(b.qn_val, b.qp_val, pages, b.context_lens, b.block_tables, b.query_start_loc,
+                                             b.num_seqs, kv_lora_rank=b.lkv, qk_rope_head_dim=b.rope, **kw)
+    return out, pages
+
+
+def run_gpu_mla(b, *, fused=True, softmax_aux=None, device="cuda:0", **kw):
+    import torch
+
+    from easydel_amd import kernels
+
+    t = lambda raw: tl.to_torch(raw, b.q_dtype, device)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(device)
+    pages = t(b.pages_raw)
+    aux = None if softmax_aux is None else torch.from_numpy(np.asarray(softmax_aux, np.float32)).to(device)
+    out, pages = kernels.mla_ragged_paged_attention(
+        t(b.qn_raw), t(b.qp_raw), t(b.kv_raw) if fused else None, t(b.pe_raw) if fused else None, pages,
+        i32(b.context_lens), i32(b.block_tables), i32(b.query_start_loc), i32(b.distribution), softmax_aux=aux, **kw)
+    torch.cuda.synchronize()
+    return tl.from_torch(out, b.q_dtype), tl.from_torch(pages, b.q_dtype)
+
+
+def check(b, what, *, fused=True, softmax_aux=None, **kw):
+    print(f"[mla] {what}: T={b.T} S={b.S} Hq={b.Hq} lkv={b.lkv} rope={b.rope} pg={b.page_size} kw={kw}", flush=True)
+    want, want_pages = mla_oracle(b, fused=fused, softmax_aux=softmax_aux, **kw)
+    got, got_pages = run_gpu_mla(b, fused=fused, softmax_aux=softmax_aux, **kw)
+    np.testing.assert_array_equal(got_pages, want_pages, err_msg=f"{what}: pages after the write")
+    return tl.assert_close(got, want, b, what)
+
+
+SCALE = (128 + 64) ** -0.5  # what the caller passes for DeepSeek-V3: (qk_nope_head_dim + qk_rope_head_dim) ** -0.5
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_small_shapes_run_on_the_fp32_kernel(dtype):
+    b = make_mla_batch(0, [17, 64, 130, 255, 1], [1, 1, 8, 33, 1], Hq=4, lkv=64, rope=16, page_size=16, dtype=dtype, pad_rows=2, pad_tokens=3)
+    check(b, "small", softmax_scale=0.11)
+    check(b, "small window+cap", softmax_scale=0.11, sliding_window=20, logits_soft_cap=5.0)
+    check(b, "small read-only", fused=False)
+    check(b, "small sinks", softmax_aux=np.array([0.5, -1.0, 2.0, 0.0]))
+
+
+def test_fp32_queries_at_the_model_shape():
+    b = make_mla_batch(1, [70, 300, 5], [1, 4, 5], Hq=3, page_size=32, dtype=F32)
+    check(b, "fp32 512+64", softmax_scale=SCALE)
+
+
+@pytest.mark.parametrize("Hq", [16, 128, 20])
+def test_decode_batches_on_the_matrix_cores(Hq):
+    rng = np.random.default_rng(2)
+    ctx = rng.integers(1, 700, size=9).tolist() + [1, 32, 33, 64, 65]
+    b = make_mla_batch(3, ctx, [1] * len(ctx), Hq=Hq, pad_rows=3, pad_tokens=2)
+    check(b, f"decode Hq={Hq}", softmax_scale=SCALE)
+
+
+def test_chunked_prefill_and_mixed_rows():
+    b = make_mla_batch(4, [200, 97, 400, 31, 1000], [1, 97, 150, 31, 3], Hq=16)
+    check(b, "mixed", softmax_scale=SCALE)
+    b = make_mla_batch(5, [300, 64], [40, 64], Hq=128, page_size=32)
+    check(b, "prefill Hq=128 pg=32", softmax_scale=SCALE)
+
+
+def test_window_soft_cap_and_sinks_on_the_matrix_cores():
+    b = make_mla_batch(6, [500, 260, 90, 700], [1, 130, 90, 5], Hq=16)
+    check(b, "window", softmax_scale=SCALE, sliding_window=100)
+    check(b, "window 1", softmax_scale=SCALE, sliding_window=1)
+    check(b, "cap", softmax_scale=SCALE, logits_soft_cap=2.0)
+    check(b, "sinks", softmax_scale=SCALE, softmax_aux=np.linspace(-2.0, 3.0, 16))
+    check(b, "read-only", softmax_scale=SCALE, fused=False)
+
+
+def test_rows_split_over_key_chunks_agree_with_single_chunks():
+    from easydel_amd import _lib
+
+    b = make_mla_batch(7, [2500, 1300, 700, 4000], [1, 2, 70, 1], Hq=16)
+    for chunks in (1, 3, 16):
+        prev = _lib.set_tunable("mla_chunks", chunks)
+        try:
+            check(b, f"chunks={chunks}", softmax_scale=SCALE)
+            check(b, f"chunks={chunks} window", softmax_scale=SCALE, sliding_window=1500)
+            check(b, f"chunks={chunks} sinks", softmax_scale=SCALE, softmax_aux=np.linspace(-1.0, 4.0, 16))
+        finally:
+            _lib.set_tunable("mla_chunks", prev)
+    check(b, "default chunks", softmax_scale=SCALE)
+
+
+def test_matrix_core_kernel_matches_the_fp32_kernel():
+    from easydel_amd import _lib
+
+    b = make_mla_batch(8, [333, 64, 1200], [1, 64, 20], Hq=32)
+    got, _ = run_gpu_mla(b, softmax_scale=SCALE)
+    prev = _lib.set_tunable("force_generic", 1)
+    try:
+        ref, _ = run_gpu_mla(b, softmax_scale=SCALE)
+    finally:
+        _lib.set_tunable("force_generic", prev)
+    rows = tl.valid_rows(b)
+    assert np.abs(got[rows] - ref[rows]).max() <= 2e-2
+
+
+def test_large_scores_raise_the_softmax_reference():
+    # scores growing along the sequence (through the rope part, so the values stay of order one) force the running
+    # reference up tile after tile
+    b = make_mla_batch(9, [600], [1], Hq=16)
+    ramp = np.linspace(0.0, 40.0, 600)
+    pages = b.pages_val.copy()
+    qp = np.zeros_like(b.qp_val); qp[..., 0] = 1.0
+    for pos in range(599):
+        pages[b.block_tables[0, pos // 64], pos % 64, b.off] = ramp[pos]
+    b.pe_val[0, 0] = 40.0
+    b.pe_raw = orc.f32_to_bf16_bits(b.pe_val.astype(np.float32)); b.pe_val = orc.bf16_bits_to_f32(b.pe_raw).astype(np.float64)
+    b.pages_raw = orc.f32_to_bf16_bits(pages.astype(np.float32)); b.pages_val = orc.bf16_bits_to_f32(b.pages_raw).astype(np.float64)
+    b.qp_raw = orc.f32_to_bf16_bits(qp.astype(np.float32)); b.qp_val = orc.bf16_bits_to_f32(b.qp_raw).astype(np.float64)
+    b.qn_raw = np.zeros_like(b.qn_raw); b.qn_val = np.zeros_like(b.qn_val)
+    check(b, "ramp", softmax_scale=1.0)
+
+
+def test_padded_tokens_are_zeroed_and_bad_arguments_are_reported():
+    import torch
+
+    from easydel_amd import _lib, kernels
+
+    b = make_mla_batch(10, [100, 50], [1, 1], Hq=16, pad_tokens=5)
+    got, _ = run_gpu_mla(b, softmax_scale=SCALE)
+    assert not got[2:].any()
+    q = torch.zeros(2, 16, 512, dtype=torch.bfloat16, device="cuda:0")
+    pages = torch.zeros(4, 64, 576 - 8, dtype=torch.bfloat16, device="cuda:0")  # row too short for latent + rope
+    i = lambda *v: torch.tensor(v, dtype=torch.int32, device="cuda:0")
+    with pytest.raises(_lib.RpaError, match="row_elems"):
+        kernels.mla_ragged_paged_attention(q, q[..., :64].contiguous(), None, None, pages, i(5, 5), i(1, 2), i(0, 1, 2), i(0, 0, 2))
+    with pytest.raises(ValueError, match="must share"):
+        kernels.mla_ragged_paged_attention(q, q[:1, :, :64].contiguous(), None, None, pages, i(5, 5), i(1, 2), i(0, 1, 2), i(0, 0, 2))
