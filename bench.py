@@ -35,7 +35,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill"])
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill",
+                             "mla-decode-h128", "mla-decode-h16", "mla-prefill-h128"])
     ap.add_argument("--layout", default="interleaved", choices=["interleaved", "unified"],
                     help="interleaved: one pool [P, page, 2*Hkv, D], scatter fused with the attention call (v3); "
                          "unified: separate K and V pools [P, page, Hkv, D], two slice scatters then the attention call")
@@ -46,6 +47,8 @@ def parse_args():
     ap.add_argument("--prefill-chunks", type=int, default=0)
     ap.add_argument("--decode-sync", type=int, default=-1)
     ap.add_argument("--max-splits", type=int, default=0)
+    ap.add_argument("--mla-chunks", type=int, default=0)
+    ap.add_argument("--mla-min-chunk", type=int, default=0)
     ap.add_argument("--sequential-pages", action="store_true", help="experiment: block tables in pool order")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so a counter run shows what a known-size kernel reads")
@@ -132,6 +135,97 @@ def cpu_baseline(w, tens, sample_seqs):
     }, out, rows
 
 
+def bench_mla(args):
+    """Multi-latent attention over latent pages (kv_lora_rank 512, rope 64, bf16, page size 64): a decode batch
+    shaped like the default workload (256 sequences of 512..8192 tokens, one new token each) with 128 query heads
+    (DeepSeek-V3 on one GPU) or 16 (its eighth, DeepSeek-V2-Lite), or a chunked prefill of 8 x 512 tokens after
+    3 584.  One step = the fused call: page write + attention.  Same output line as the default workload; no CPU
+    sample is timed for these."""
+    import torch
+
+    from easydel_amd import kernels
+
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(args.seed)
+    lkv, rope, row, pg = 512, 64, 640, 64
+    if args.workload == "mla-prefill-h128":
+        Hq, n = 128, 8
+        q_lens = np.full(n, 512, np.int32)
+        ctx = np.full(n, 4096, np.int32)
+    else:
+        Hq, n = (128 if args.workload.endswith("h128") else 16), 256
+        q_lens = np.ones(n, np.int32)
+        ctx = rng.integers(512, 8193, size=n).astype(np.int32)
+    need = -(-ctx // pg)
+    M = int(need.max())
+    P = int(need.sum()) + 64
+    perm = rng.permutation(np.arange(1, P)).astype(np.int32)
+    bt = np.zeros((n, M), np.int32)
+    k = 0
+    for i, m in enumerate(need):
+        bt[i, :m] = perm[k:k + m]
+        k += m
+    T = int(q_lens.sum())
+    qsl = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    g = torch.Generator(device=dev).manual_seed(args.seed)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)  # noqa: E731
+    pages = torch.empty(P, pg, row, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, P, 4096):
+        pages[lo:lo + 4096] = rnd(min(4096, P - lo), pg, row)
+    qn, qp, kv, pe = rnd(T, Hq, lkv), rnd(T, Hq, rope), rnd(T, lkv), rnd(T, rope)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(dev)  # noqa: E731
+    ctx_d, bt_d, qsl_d, dist_d = i32(ctx), i32(bt), i32(qsl), i32([0, 0, n])
+    out = torch.empty_like(qn)
+    scale = (128 + rope) ** -0.5
+
+    def step(write=True):
+        kernels.mla_ragged_paged_attention(qn, qp, kv if write else None, pe if write else None, pages, ctx_d, bt_d, qsl_d,
+                                           dist_d, softmax_scale=scale, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    stream = torch.cuda.current_stream(dev)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:  # the call without the page write: attention kernel + merge, bracketed on the launch stream
+        a.record(stream)
+        step(write=False)
+        b.record(stream)
+    torch.cuda.synchronize()
+    att_ms = float(np.mean([a.elapsed_time(b) for a, b in evs]))
+    # algorithmic bytes: every visible latent row once per sequence (it is key and value at once), queries, outputs,
+    # block-table entries, lengths; flops: 2 (lkv + rope) for the scores + 2 lkv for the values, per (row, visible key)
+    pos0 = ctx - q_lens
+    pairs = int(sum(int(q) * int(p0) + int(q) * (int(q) + 1) // 2 for q, p0 in zip(q_lens, pos0)))
+    nbytes = int(ctx.sum()) * (lkv + rope) * 2 + T * Hq * (2 * lkv + rope) * 2 + int(need.sum()) * 4 + (2 * n + 1) * 4
+    flops = 2 * Hq * (2 * lkv + rope) * pairs
+    hbm_frac = nbytes / (att_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+    mfma_frac = flops / (att_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS
+    bound = "hbm" if nbytes / (HBM_PEAK_GBS * 1e9) >= flops / (MFMA_BF16_PEAK_TFLOPS * 1e12) else "mfma"
+    roofline = ({"bound": "hbm", "achieved": nbytes / (att_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": hbm_frac}
+                if bound == "hbm" else
+                {"bound": "mfma", "achieved": flops / (att_ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mfma_frac})
+    roofline.update({"traffic": None, "kernel": "mla_attn_kernel + mla_merge_kernel (the call without the page write)",
+                     "kernel_ms": att_ms, "algorithmic_bytes_per_launch": nbytes, "algorithmic_flops_per_launch": flops,
+                     "hbm_frac": hbm_frac, "mfma_frac": mfma_frac})
+    print(json.dumps({
+        "metric": "decode tokens/s + attn HBM TB/s (% of 8 TB/s), Llama-3-8B-shaped, 1 GPU",
+        "value": T / (ms_per_step * 1e-3),
+        "unit": "tokens/s (one attention-layer call: latent page write + multi-latent ragged paged attention)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "sequences": n, "query_tokens": T, "q_heads": Hq, "kv_lora_rank": lkv,
+                   "qk_rope_head_dim": rope, "page_row_elems": row, "page_size": pg, "pool_pages": P,
+                   "context_tokens_total": int(ctx.sum()), "context_range": [int(ctx.min()), int(ctx.max())], "seed": args.seed},
+        "roofline": roofline, "cpu_baseline": None,
+    }))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -145,6 +239,12 @@ def main():
     from easydel_amd import _lib, kernels, workloads
 
     _lib.load()
+    if args.workload.startswith("mla-"):
+        if args.mla_chunks:
+            _lib.set_tunable("mla_chunks", args.mla_chunks)
+        if args.mla_min_chunk:
+            _lib.set_tunable("mla_min_chunk", args.mla_min_chunk)
+        return bench_mla(args)
     if args.decode_wgs:
         _lib.set_tunable("decode_wgs", args.decode_wgs)
     if args.decode_sync >= 0:

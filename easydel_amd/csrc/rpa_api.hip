@@ -29,6 +29,7 @@ std::atomic<int> g_force_generic{0};
 std::atomic<int> g_prefill_dma{1};
 std::atomic<int> g_decode_pace{1};
 std::atomic<int> g_mla_chunks{0};  // 0 = sized from the shapes
+std::atomic<int> g_mla_min_chunk{0};  // 0 = default
 std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
 
 int fail(int code, const char* fmt, ...) {
@@ -126,7 +127,7 @@ void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* min_chunk) {
   const size_t per = part_o_bytes(T, Hq, lkv) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   *max_chunks = (int)chunks;
-  *min_chunk = Hq >= 64 ? 2048 : 512;
+  *min_chunk = g_mla_min_chunk.load() > 0 ? g_mla_min_chunk.load() : (Hq >= 64 ? 2048 : 512);
 }
 
 bool mla_shape_on_mfma(int page_size, int lkv, int rope, int row_elems, int q_dtype, int kv_dtype) {
@@ -158,6 +159,7 @@ int rpa_set_tunable(const char* name, int value) {
   if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
   if (!strcmp(name, "prefill_dma")) return g_prefill_dma.exchange(value != 0);
   if (!strcmp(name, "decode_pace")) return g_decode_pace.exchange(value != 0);
+  if (!strcmp(name, "mla_min_chunk")) return g_mla_min_chunk.exchange(value <= 0 ? 0 : ((value + 63) & ~63));
   if (!strcmp(name, "mla_chunks")) return g_mla_chunks.exchange(value < 0 ? 0 : (value > rpa::kMlaMaxChunks ? rpa::kMlaMaxChunks : value));
   if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
   return -1;
@@ -419,7 +421,8 @@ size_t rpa_mla_workspace_bytes(int T, int S, int M, int page_size, int Hq, int k
   if (T <= 0 || S <= 0 || Hq <= 0 || kv_lora_rank <= 0) return 256;
   int chunks, min_chunk;
   mla_split(T, S, Hq, kv_lora_rank, &chunks, &min_chunk);
-  return (chunks > 1 ? (size_t)chunks * (part_o_bytes(T, Hq, kv_lora_rank) + part_ml_bytes(T, Hq)) : 0) + 512;
+  return (chunks > 1 ? (size_t)chunks * (part_o_bytes(T, Hq, kv_lora_rank) + part_ml_bytes(T, Hq)) : 0) +
+         rpa::mla_plan_bytes(T, S, Hq, chunks) + 512;
 }
 
 static int mla_fill(const char* who, rpa::MlaParams& p, const void* keys_values, const void* keys_pe, void* kv_pages,
@@ -506,13 +509,21 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
     mla_split(T, S, Hq, kv_lora_rank, &chunks, &min_chunk);
     const size_t po = part_o_bytes(T, Hq, kv_lora_rank), pml = part_ml_bytes(T, Hq);
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
-    const size_t usable = (workspace && workspace_bytes > 256) ? workspace_bytes - 256 : 0;
-    if ((size_t)chunks * (po + pml) > usable) chunks = (int)(usable / (po + pml));  // a small workspace: fewer, longer chunks
-    if (chunks < 2) chunks = 1;  // a single chunk writes its rows directly and needs no workspace
+    // the plan is sized for the chunks the shapes ask for; a small workspace then gets fewer, longer chunks
+    const size_t plan_bytes_mla = rpa::mla_plan_bytes(T, S, Hq, chunks);
+    if (!workspace || workspace_bytes < plan_bytes_mla + 256)
+      return fail(RPA_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu needed for the plan", who, workspace_bytes, plan_bytes_mla + 256);
+    const size_t usable = workspace_bytes - 256 - plan_bytes_mla;
+    if ((size_t)chunks * (po + pml) > usable) chunks = (int)(usable / (po + pml));
+    if (chunks < 2) chunks = 1;  // a single chunk writes its rows directly and needs no partial buffers
     p.max_chunks = chunks;
     p.min_chunk = min_chunk;
-    p.part_o = (float*)base;
-    p.part_ml = (float*)(base + (size_t)chunks * po);
+    const size_t slots = (size_t)rpa::mla_plan_slots(T, S, Hq);
+    p.plan = (int2*)base;
+    p.n_units = (int32_t*)(base + align256(slots * 8));
+    p.units = (int2*)(base + align256(slots * 8) + 256);
+    p.part_o = (float*)(base + plan_bytes_mla);
+    p.part_ml = (float*)(base + plan_bytes_mla + (size_t)chunks * po);
     const int err = rpa::launch_mla_mfma(s, p);
     if (err) return hip_fail(err, "MLA kernel launch");
   } else {

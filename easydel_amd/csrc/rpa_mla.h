@@ -24,6 +24,9 @@ struct MlaParams {
   void* out;       // [T][Hq][lkv], query dtype
   float* part_o;   // [max_chunks][T][Hq][lkv]
   float* part_ml;  // [max_chunks][T][Hq][2]  (running max in log2 units, running sum)
+  int2* plan;      // [row-tile slots] (sequence, key chunks) of the row tile at a slot; chunks = 0: no such tile
+  int32_t* n_units;  // [1] number of (row tile, key chunk) units of the batch = workgroups with work
+  int2* units;     // [n_units] (slot, chunk), slot-major
   int T, S, M, P, page_size, Hq, lkv, rope, rope_off, row_elems;
   int64_t token_stride, page_stride;  // bytes
   int q_dtype, kv_dtype;
@@ -80,6 +83,8 @@ __device__ __forceinline__ MlaTile mla_tile(const MlaParams& p, const MlaSeq& sp
 int launch_mla_scatter(hipStream_t stream, const MlaParams& p);
 int launch_mla_generic(hipStream_t stream, const MlaParams& p);
 int launch_mla_mfma(hipStream_t stream, const MlaParams& p);
+int64_t mla_plan_slots(int T, int S, int Hq);  // row-tile slots of a batch (upper bound) = entries of MlaParams::plan
+size_t mla_plan_bytes(int T, int S, int Hq, int max_chunks);  // plan + unit count + unit list
 int launch_mla_merge(hipStream_t stream, const MlaParams& p);
 bool mla_mfma_supported(const MlaParams& p);
 

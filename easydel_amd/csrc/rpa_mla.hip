@@ -139,6 +139,63 @@ __global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
   }
 }
 
+// ---- plan: which sequence and how many key chunks each row-tile slot of the MFMA kernel's grid holds -------------
+// Sequence i starts at slot floor(qsl[i] * Hq / 128) + i (its row tiles follow), so the slots of a batch are found
+// without a scan; slots between sequences, past the live ones, or of rows before position 0 hold no tile.
+__global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots) {
+  const int slot = blockIdx.x * 256 + threadIdx.x;
+  if (slot >= n_slots) return;
+  int2 unit = {0, 0};
+  const int n_live = mla_live_rows(p);
+  if (n_live > 0) {
+    int lo_i = 0, hi_i = n_live;  // the last sequence starting at or before `slot`
+    while (hi_i - lo_i > 1) {
+      const int mid = (lo_i + hi_i) >> 1;
+      if ((int)(((int64_t)p.qsl[mid] * p.Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
+    }
+    const MlaSeq sp = mla_seq(p, lo_i);
+    const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * p.Hq) / kMlaRows) + lo_i);
+    if (sp.live && tile_in_seq >= 0 && tile_in_seq * kMlaRows < sp.q_len * p.Hq) {
+      unit.x = lo_i;
+      unit.y = mla_tile(p, sp, tile_in_seq * kMlaRows).n_chunks;
+    }
+  }
+  p.plan[slot] = unit;
+}
+
+// The units (row tile, key chunk) of the batch in one dense list, slot-major.  The MFMA kernel's grid is sized from
+// the static bounds and most of its slots are empty; left in place, the empty ones form a regular pattern (a batch of
+// single tokens with 128 heads fills every other slot) that the hardware's round-robin placement of consecutive
+// blocks turns into idle shader engines: measured, each engine was busy 43 % of such a kernel's duration.
+// One block: a scan over the plan's chunk counts, 1024 slots a pass.
+__global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_slots) {
+  __shared__ int wave_tot[16];
+  __shared__ int running_s;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  if (tid == 0) running_s = 0;
+  __syncthreads();
+  for (int base = 0; base < n_slots; base += 1024) {
+    const int slot = base + tid;
+    const int v = slot < n_slots ? p.plan[slot].y : 0;
+    int incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) wave_tot[wv] = incl;
+    __syncthreads();
+    int before = running_s;
+    for (int w = 0; w < wv; ++w) before += wave_tot[w];
+    const int first = before + incl - v;
+    for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c);
+    __syncthreads();
+    if (tid == 1023) running_s = before + incl;
+    __syncthreads();
+  }
+  if (tid == 0) p.n_units[0] = running_s;
+}
+
 // ---- MFMA kernel ----------------------------------------------------------------------------------------------------
 // One LDS DMA of 1 KiB: every lane fetches 16 bytes from base + voff; lane L's bytes land at LDS byte address
 // lds_addr + 16 L.
@@ -151,13 +208,15 @@ __device__ __forceinline__ void mla_wait_loads_and_barrier() {
 }
 
 // XOR key (on the low three bits of the 16-byte chunk index) of LDS row r.  Rows are 1152 bytes, so rows of equal
-// parity start in the same bank group and rows of different parity half the banks apart.  The row-wise reads (16 rows,
-// one chunk each) need the eight rows of a parity in eight different chunks; the transposing reads (per half wave 8
-// rows, a pair of chunks each) need the four rows of a parity in four different pairs.  Bits 1-2 from the row's
-// bits 1-2 and bit 0 from its bit 3 give both.
-__device__ __forceinline__ int mla_key(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
+// parity start in the same bank group and rows of different parity half the banks apart.  Chosen by measurement
+// (SQ_LDS_BANK_CONFLICT over the kernel, 32-key tiles read row-wise with ds_read_b128 and transposed with
+// ds_read_b64_tr_b16): this key and `r & 7` count no conflict cycle at all; no key: three conflict cycles per
+// useful one (8.4 ms instead of 5.7 ms on a 4 096-token prefill); keys that map two rows of equal parity among
+// rows 0-7 to the same chunk pair, or that ignore the parity: 0.5 to 1 conflict cycle per useful one.
+__device__ __forceinline__ int mla_key(int r) { return ((r >> 1) & 3) << 1; }
 
 constexpr int kMlaWaves = 8;  // waves of an MFMA-kernel workgroup
+constexpr int kXcds = 8;      // accelerator dies a grid's blocks are dealt to in turn
 
 template <bool CAP>
 __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p) {
@@ -169,11 +228,13 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   constexpr int NINS = TILE / 1024;      // DMA instructions per tile, dealt round-robin to the waves
   constexpr int NDMA = (NINS + NW - 1) / NW;  // most per wave
   static_assert(NINS % NW == NW / 2, "the first half of the waves issue NDMA instructions a tile, the others one fewer");
-  constexpr int NSLOT = 3;
+  constexpr int NSLOT = 3;               // tiles of the LDS ring: NSLOT - 1 are in flight ahead of the one in use
   constexpr int NS = TT / 16;            // 16-key sub-tiles per tile
   constexpr int DPL = LKV / 16;          // 16-dim row tiles of O^T
   constexpr int NKK = DK / 32;           // k-steps of the score product
   constexpr int NKN = LKV / 32;          // of which over the latent part
+  constexpr int NKO = NS * NKK;          // K operands of a tile
+  constexpr int KPD = 4, PD = 4;         // operand reads in flight ahead of the score / PV matrix instructions
   constexpr float kMaxSlack = 8.f;       // how far a score may exceed the softmax reference before it is raised
   static_assert(NW * RB * 16 == kMlaRows, "merge kernel assumes this row-tile height");
 
@@ -186,27 +247,26 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   const int Hq = p.Hq;
 
   // ---- block -> (sequence, row tile, key chunk) -------------------------------------------------------------
-  const int n_slots = gridDim.x / p.max_chunks;
-  const int slot = blockIdx.x % n_slots;
-  const int chunk = blockIdx.x / n_slots;  // slowest: neighbouring blocks are row tiles of neighbouring sequences
-  const int n_live = mla_live_rows(p);
-  if (n_live <= 0) return;
-  // sequence i starts at slot floor(qsl[i]*Hq/128) + i; find the last sequence starting at or before `slot`
-  int lo_i = 0, hi_i = n_live;
-  while (hi_i - lo_i > 1) {
-    const int mid = (lo_i + hi_i) >> 1;
-    if ((int)(((int64_t)p.qsl[mid] * Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
-  }
-  const int i = lo_i;
+  // The grid is sized from the static bounds, so most of its blocks have nothing to do, and a workgroup holds a
+  // whole compute unit: the plan kernel has looked every slot up beforehand, and a block learns with one load
+  // whether it has work.
+  // Block -> unit of the dense list.  Consecutive blocks go to the eight XCDs in turn; unit = (block % 8) * n8 +
+  // block / 8 hands every XCD a contiguous eighth of the list, so that the row tiles of a long prompt, which read
+  // the same keys, share one XCD's L2.
+  const int total = p.n_units[0];
+  const int n8 = (total + kXcds - 1) / kXcds;
+  const int u = (blockIdx.x % kXcds) * n8 + blockIdx.x / kXcds;
+  if ((int)(blockIdx.x / kXcds) >= n8 || u >= total) return;
+  const int2 sc = p.units[u];
+  const int slot = sc.x, chunk = sc.y;
+  const int2 unit = p.plan[slot];
+  const int i = unit.x;
   const MlaSeq sp = mla_seq(p, i);
-  if (!sp.live) return;
   const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * Hq) / kMlaRows) + i);
   const int rows_total = sp.q_len * Hq;
   const int R0 = tile_in_seq * kMlaRows;
-  if (tile_in_seq < 0 || R0 >= rows_total) return;
 
   const MlaTile mt = mla_tile(p, sp, R0);
-  if (chunk >= mt.n_chunks) return;  // also: queries before position 0 have no keys; such rows stay unwritten
   const int base_pos = sp.ctx - sp.q_len;
   const int vis_lo = mt.vis_lo;
   // the first tile must hold vis_lo, so that rows of it that nobody may see can borrow a visible row's address
@@ -214,45 +274,6 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   const int kv_hi = min(mt.kv_hi, mt.kv_lo + (chunk + 1) * mt.chunk);
   const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
   const bool single = mt.n_chunks == 1;
-
-  // ---- per row-block lane state ----------------------------------------------------------------------------
-  int row_lo[RB], row_hi[RB];
-  bool row_ok[RB];
-  int out_tok[RB], out_head[RB];
-  bf16x8 qf[RB][NKK];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const int row = R0 + (wave * RB + rb) * 16 + n;
-    row_ok[rb] = row < rows_total;
-    const int r_tok = row_ok[rb] ? row / Hq : (rows_total - 1) / Hq;  // padded rows shadow the last row
-    const int r_head = row_ok[rb] ? row - r_tok * Hq : 0;
-    const int pos = base_pos + r_tok;
-    row_hi[rb] = min(pos + 1, sp.ctx);
-    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
-    out_tok[rb] = sp.q0 + r_tok;
-    out_head[rb] = r_head;
-    const int64_t qrow = (int64_t)out_tok[rb] * Hq + r_head;
-    const char* qn = (const char*)p.q_nope + qrow * (LKV * 2);
-    const char* qp = (const char*)p.q_pe + qrow * (ROPE * 2);
-#pragma unroll
-    for (int kk = 0; kk < NKK; ++kk) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (row_ok[rb]) v = kk < NKN ? *(const u32x4*)(qn + (kk * 32 + 8 * g4) * 2) : *(const u32x4*)(qp + ((kk - NKN) * 32 + 8 * g4) * 2);
-      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
-    }
-  }
-  // Use the query registers once here, so that the compiler waits for these loads now and not at their first use
-  // inside the loop, where its wait would also cover every tile in flight.
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-    for (int kk = 0; kk < NKK; ++kk) {
-      u32x4 v = __builtin_bit_cast(u32x4, qf[rb][kk]);
-      asm volatile("" : "+v"(v));
-      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
-    }
-  // a wave whose row blocks all lie past the sequence's rows only helps with the loads
-  const bool wave_active = (R0 + wave * RB * 16) < rows_total;
 
   // ---- tile loads --------------------------------------------------------------------------------------------
   // The tile is 36 KiB of LDS in row order (72 chunks a row); DMA instruction u = wave + 4 j fills its bytes
@@ -266,8 +287,11 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
   // (row, global chunk) of DMA instruction j for this lane; recomputed at every issue -- a few integer instructions
   // against the hundred-odd MFMAs of a tile -- rather than held in eighteen registers
-  auto dma_row = [&](int j) -> int { return (64 * (wave + NW * j) + lane) / CPR; };
-  auto dma_chunk = [&](int j, int r) -> int { return ((64 * (wave + NW * j) + lane) - r * CPR) ^ mla_key(r); };
+  // (the lane number passes through an empty assembly statement at every issue, or the compiler would compute the
+  // offsets once before the loop after all and spill them)
+  int dma_lane = lane;
+  auto dma_row = [&](int j) -> int { return (64 * (wave + NW * j) + dma_lane) / CPR; };
+  auto dma_chunk = [&](int j, int r) -> int { return ((64 * (wave + NW * j) + dma_lane) - r * CPR) ^ mla_key(r); };
   const bool dma_full = wave < NINS % NW;  // this wave issues NDMA instructions per tile (else NDMA - 1)
   int cur_idx = kv_lo / pg;
   int cur_off = kv_lo - cur_idx * pg;
@@ -281,6 +305,8 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
     const bool edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
     const uint32_t dst = lds_base + (uint32_t)cur_slot * TILE + (uint32_t)wave * 1024u;
     const uint32_t ts = (uint32_t)p.token_stride;
+    dma_lane = lane;
+    asm volatile("" : "+v"(dma_lane));
     if (!edge) {
 #pragma unroll
       for (int j = 0; j < NDMA; ++j) {
@@ -340,15 +366,64 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
       v_base[st][q] = tk * RKL + (((2 * q + (tr_byte >> 4)) ^ mla_key(tk)) << 4) + (tr_byte & 15);
     }
 
-  issue();
-  if (n_tiles > 1) issue();
+  constexpr int AHEAD = NSLOT - 1;  // tiles issued ahead of the one in use
+  static_assert(AHEAD >= 1 && AHEAD <= 3, "the waits below are written out for up to three tiles ahead");
+#pragma unroll
+  for (int a = 0; a < AHEAD; ++a)
+    if (a < n_tiles) issue();
+
+  // ---- per row-block lane state ----------------------------------------------------------------------------
+  int row_lo[RB], row_hi[RB];
+  bool row_ok[RB];
+  int out_tok[RB], out_head[RB];
+  bf16x8 qf[RB][NKK];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = R0 + (wave * RB + rb) * 16 + n;
+    row_ok[rb] = row < rows_total;
+    const int r_tok = row_ok[rb] ? row / Hq : (rows_total - 1) / Hq;  // padded rows shadow the last row
+    const int r_head = row_ok[rb] ? row - r_tok * Hq : 0;
+    const int pos = base_pos + r_tok;
+    row_hi[rb] = min(pos + 1, sp.ctx);
+    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+    out_tok[rb] = sp.q0 + r_tok;
+    out_head[rb] = r_head;
+    const int64_t qrow = (int64_t)out_tok[rb] * Hq + r_head;
+    const char* qn = (const char*)p.q_nope + qrow * (LKV * 2);
+    const char* qp = (const char*)p.q_pe + qrow * (ROPE * 2);
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok[rb]) v = kk < NKN ? *(const u32x4*)(qn + (kk * 32 + 8 * g4) * 2) : *(const u32x4*)(qp + ((kk - NKN) * 32 + 8 * g4) * 2);
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  }
+  // (The queries are loaded behind the first tiles' DMAs, so that the two latencies overlap.)  Use the query
+  // registers once here, so that the compiler waits for these loads now and not at their first use inside the loop,
+  // where its wait would also cover every tile in flight.
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      u32x4 v = __builtin_bit_cast(u32x4, qf[rb][kk]);
+      asm volatile("" : "+v"(v));
+      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+    }
+  // a wave whose row blocks all lie past the sequence's rows only helps with the loads
+  const bool wave_active = (R0 + wave * RB * 16) < rows_total;
+
   int rd_slot = 0;
   for (int tile = 0; tile < n_tiles; ++tile) {
-    // tile `tile` has landed (tile + 1 may still be in flight), and every wave is done with tile - 1
-    if (tile + 1 >= n_tiles) mla_wait_loads_and_barrier<0>();
-    else if (dma_full) mla_wait_loads_and_barrier<NDMA>();
-    else mla_wait_loads_and_barrier<NDMA - 1>();
-    if (tile + 2 < n_tiles) issue();  // into the slot of tile - 1
+    // tile `tile` must have landed; the tiles issued after it (at most AHEAD - 1) may still be in flight.  Behind the
+    // barrier every wave is done with tile - 1, whose slot takes tile + AHEAD.
+    const int later = min(AHEAD - 1, n_tiles - 1 - tile);
+    if (later <= 0) mla_wait_loads_and_barrier<0>();
+    else if (later == 1) {
+      if (dma_full) mla_wait_loads_and_barrier<NDMA>(); else mla_wait_loads_and_barrier<NDMA - 1>();
+    } else {
+      if (dma_full) mla_wait_loads_and_barrier<2 * NDMA>(); else mla_wait_loads_and_barrier<2 * (NDMA - 1)>();
+    }
+    if (tile + AHEAD < n_tiles) issue();
     const unsigned char* lds_t = lds_all + rd_slot * TILE;
     rd_slot = (rd_slot == NSLOT - 1) ? 0 : rd_slot + 1;
     if (!wave_active) continue;
@@ -360,17 +435,34 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
     for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
       for (int st = 0; st < NS; ++st) s_acc[rb][st] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // Operand i = (sub-tile i % NS, k-step i / NS): the two sub-tiles' accumulation chains alternate.  Chunk 4 kk + g4 under the key: only its low three bits move, so
+    // a k-step's address is one of two per-lane bases (kk even / odd) plus a constant.  The operands are read KPD
+    // steps ahead of the matrix instructions that use them: an LDS read under load lasts several times the 16 clocks
+    // of one instruction, and read just in time the wave would wait at every step.
+    {
+      auto read_k = [&](int i) __attribute__((always_inline)) -> u32x4 {
+        const int st = i % NS, kk = i / NS;
+        return *(const u32x4*)(lds_t + k_base[st][kk & 1] + (kk >> 1) * 128);
+      };
+      u32x4 kp[KPD];
 #pragma unroll
-    for (int st = 0; st < NS; ++st) {
+      for (int i = 0; i < KPD; ++i) kp[i] = read_k(i);
 #pragma unroll
-      for (int kk = 0; kk < NKK; ++kk) {
-        // chunk 4 kk + g4 under the key: only its low three bits move, so a k-step's address is one of two
-        // per-lane bases (kk even / odd) plus a constant
-        const u32x4 a = *(const u32x4*)(lds_t + k_base[st][kk & 1] + (kk >> 1) * 128);
+      for (int i = 0; i < NKO; ++i) {
+        const u32x4 a = kp[i % KPD];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb)
-          s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
+          s_acc[rb][i % NS] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][i / NS], s_acc[rb][i % NS], 0, 0, 0);
+        if (i + KPD < NKO) kp[i % KPD] = read_k(i + KPD);
       }
+      // the order the scheduler must keep: KPD reads first, then a matrix instruction and the next read in turn
+      __builtin_amdgcn_sched_group_barrier(0x100, KPD, 0);
+#pragma unroll
+      for (int i = 0; i + KPD < NKO; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, RB * KPD, 0);
     }
 
     // ---- online softmax per row block ------------------------------------------------------------------------
@@ -437,20 +529,38 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
     }
 
     // ---- O^T += V^T . P^T: the values are the first LKV elements of the same rows -----------------------------
+    // Row tile rt spans chunks 2 rt, 2 rt + 1: under the key one of four per-lane bases (rt & 3) plus a constant.
+    // Read PD row tiles ahead, as above.
+    {
+      auto read_v = [&](int rt) __attribute__((always_inline)) -> u32x4 {
+        const unsigned char* p0 = lds_t + v_base[0][rt & 3] + (rt >> 2) * 128;
+        const unsigned char* p1 = lds_t + v_base[1][rt & 3] + (rt >> 2) * 128;
+        const u32x2 a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0));
+        const u32x2 a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p1));
+        return (u32x4){a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
+      };
+      __builtin_amdgcn_sched_barrier(0);  // keep the V operand reads out of the softmax: they would only pile up in registers
+      u32x4 av[PD];
 #pragma unroll
-    for (int rt = 0; rt < DPL; ++rt) {
-      // row tile rt spans chunks 2 rt, 2 rt + 1: under the key one of four per-lane bases (rt & 3) plus a constant
-      const unsigned char* p0 = lds_t + v_base[0][rt & 3] + (rt >> 2) * 128;
-      const unsigned char* p1 = lds_t + v_base[1][rt & 3] + (rt >> 2) * 128;
-      const u32x2 a_lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0));
-      const u32x2 a_hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p1));
-      const u32x4 a4 = {a_lo[0], a_lo[1], a_hi[0], a_hi[1]};
+      for (int rt = 0; rt < PD; ++rt) av[rt] = read_v(rt);
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb) {
-        const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
-        o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
-                                                                o_acc[rb][rt], 0, 0, 0);
+      for (int rt = 0; rt < DPL; ++rt) {
+        const u32x4 a4 = av[rt % PD];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
+          o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
+                                                                  o_acc[rb][rt], 0, 0, 0);
+        }
+        if (rt + PD < DPL) av[rt % PD] = read_v(rt + PD);
       }
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * PD, 0);
+#pragma unroll
+      for (int rt = 0; rt + PD < DPL; ++rt) {
+        __builtin_amdgcn_sched_group_barrier(0x008, RB, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, RB * PD, 0);
     }
   }
 
@@ -582,10 +692,20 @@ bool mla_mfma_supported(const MlaParams& p) {
          p.page_size % 32 == 0 && (p.token_stride & 15) == 0 && (int64_t)32 * p.token_stride < ((int64_t)1 << 31);
 }
 
+int64_t mla_plan_slots(int T, int S, int Hq) { return ((int64_t)T * Hq) / kMlaRows + S; }  // upper bound on row tiles of the batch
+
+static size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+size_t mla_plan_bytes(int T, int S, int Hq, int max_chunks) {
+  const size_t slots = (size_t)mla_plan_slots(T, S, Hq);
+  return up256(slots * 8) + 256 + up256(slots * (size_t)max_chunks * 8);
+}
+
 int launch_mla_mfma(hipStream_t stream, const MlaParams& p) {
-  const int64_t slots = ((int64_t)p.T * p.Hq) / kMlaRows + p.S;  // upper bound on row tiles of the batch
-  const int64_t blocks = slots * p.max_chunks;
+  const int64_t slots = mla_plan_slots(p.T, p.S, p.Hq);
+  const int64_t blocks = (slots * p.max_chunks + kXcds - 1) / kXcds * kXcds;  // most units the batch can have
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(mla_plan_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, stream, p, (int)slots);
+  hipLaunchKernelGGL(mla_compact_kernel, dim3(1), dim3(1024), 0, stream, p, (int)slots);
   if (p.softcap > 0.f) hipLaunchKernelGGL((mla_attn_kernel<true>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
   else hipLaunchKernelGGL((mla_attn_kernel<false>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
   return (int)hipGetLastError();

@@ -377,6 +377,8 @@ def mla_ragged_paged_attention(queries_nope, queries_pe, keys_values, keys_pe, k
     if T == 0:
         return out, kv_pages
     qd, kd = dtype_tag(queries_nope.dtype), dtype_tag(kv_pages.dtype)
+    for name, t in (("queries_nope", queries_nope), ("queries_pe", queries_pe), ("kv_pages", kv_pages), ("out", out)):
+        _dev(t, name)
     scale = float(lkv + rope) ** -0.5 if softmax_scale is None else float(softmax_scale)
     window = int(sliding_window) if sliding_window else 0
     cap = float(logits_soft_cap) if logits_soft_cap else 0.0

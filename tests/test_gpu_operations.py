@@ -134,3 +134,67 @@ def test_quantised_view_is_read_through_scales(gpu):
     out = OperationRegistry.create("ragged_page_attention_v3", OperationMetadata())(d["query"], None, None, view, meta)
     torch.cuda.synchronize()
     tl.assert_close(tl.from_torch(out.attention_outputs, BF16), tl.oracle_out(b), b, "quantised view")
+
+
+@pytest.mark.parametrize("name", ["multi_latent_ragged_page_attention_v1", "multi_latent_ragged_page_attention_v2"])
+def test_mla_operation_follows_the_model_flow(gpu, name):
+    """The layer's flow around the operation (layers/attention/_unified.py:1280-1371): queries absorbed through the key
+    half of the up-projection, the operation over latent pages, the output through the value half -- against ordinary
+    attention on decompressed keys and values."""
+    from easydel_amd.caching import MLARaggedPagesCacheConfig, MLARaggedPagesCacheView
+
+    rng = np.random.default_rng(5)
+    heads, lkv, rope, nope, vdim, page_size = 16, 512, 64, 128, 128, 64
+    scheduled, computed = [1, 1, 40, 7], [300, 63, 100, 0]
+    max_reqs, max_pages = 6, 8
+    n_pages = max_reqs * max_pages + 1
+    table = np.zeros((max_reqs, max_pages), dtype=np.int32)
+    perm = rng.permutation(np.arange(1, n_pages))
+    k = 0
+    for r in range(len(scheduled)):
+        need = -(-(computed[r] + scheduled[r]) // page_size)
+        table[r, :need] = perm[k:k + need]
+        k += need
+    cfg = MLARaggedPagesCacheConfig.create(torch.bfloat16, num_hidden_layers=1, num_kv_heads=heads, max_model_length=max_pages * page_size,
+                                           kv_lora_rank=lkv, qk_rope_head_dim=rope, page_size=page_size, num_pages=n_pages)
+    view = MLARaggedPagesCacheView.init(cfg, layer_index=0, device=gpu)
+    assert tuple(view.kv_pages.shape) == (n_pages, page_size // 2, 2, 640)
+    sched_full = np.zeros(max_reqs, np.int32); sched_full[:len(scheduled)] = scheduled
+    comp_full = np.zeros(max_reqs, np.int32); comp_full[:len(computed)] = computed
+    fields = compute_ragged_batch_fields(scheduled_full=sched_full, active_mask_full=sched_full > 0, num_computed_tokens=comp_full,
+                                         page_table=table, version="v3", max_num_reqs=max_reqs, page_size=page_size)
+    meta = RaggedPagesMetadata.from_numpy(fields, version="v3", page_size=page_size, device=gpu)
+    T = int(sum(scheduled))
+    bf = lambda a: orc.bf16_bits_to_f32(orc.f32_to_bf16_bits(a.astype(np.float32))).astype(np.float64)  # noqa: E731
+    w_k = bf(rng.standard_normal((lkv, heads, nope)) / np.sqrt(lkv))
+    w_v = bf(rng.standard_normal((lkv, heads, vdim)) / np.sqrt(lkv))
+    q_nope, q_pe = bf(rng.standard_normal((T, heads, nope))), bf(rng.standard_normal((T, heads, rope)))
+    latent, k_pe = bf(rng.standard_normal((T, lkv))), bf(rng.standard_normal((T, rope)))
+    pool = np.zeros((n_pages, page_size, 640))
+    pool[..., :lkv] = bf(rng.standard_normal((n_pages, page_size, lkv)))
+    pool[..., 512:576] = bf(rng.standard_normal((n_pages, page_size, rope)))
+    view.kv_pages.copy_(torch.from_numpy(pool).to(torch.bfloat16).view(view.kv_pages.shape))
+    q_abs = bf(np.einsum("tnd,and->tna", q_nope, w_k))  # the layer casts the absorbed queries back to the model dtype
+    tt = lambda a: torch.from_numpy(a).to(torch.bfloat16).to(gpu)  # noqa: E731
+    op = OperationRegistry.create(name, OperationMetadata())
+    scale = (nope + rope) ** -0.5
+    out = op(queries_nope=tt(q_abs)[None], queries_pe=tt(q_pe)[None], keys_values=tt(latent)[None], keys_pe=tt(k_pe)[None],
+             cache_view=view, cache_metadata=meta, softmax_scale=scale, causal=True, mask_info=None)
+    assert isinstance(out, AttentionOutput) and out.cache_view is view
+    assert tuple(out.attention_outputs.shape) == (1, T, heads, lkv)
+    got = np.einsum("tna,anh->tnh", out.attention_outputs[0].float().cpu().numpy().astype(np.float64), w_v)
+    # the same step through ordinary attention: per-head keys [latent W_k | k_pe] and values latent W_v
+    pages = orc.mla_page_scatter_ref(latent, k_pe, pool, fields["context_lens"], table, fields["query_start_loc"],
+                                     fields["request_distribution"][2:3])
+    np.testing.assert_array_equal(view.kv_pages.view(n_pages, page_size, 640).float().cpu().numpy(), pages)
+    d = nope + rope
+    dense = np.zeros((n_pages, page_size, 2 * heads, d))
+    dense[:, :, 0::2, :nope] = np.einsum("pta,and->ptnd", pages[..., :lkv], w_k)
+    dense[:, :, 0::2, nope:] = pages[:, :, None, 512:576]
+    dense[:, :, 1::2, :vdim] = np.einsum("pta,anh->ptnh", pages[..., :lkv], w_v)
+    want = orc.ragged_paged_attention_ref(np.concatenate([q_nope, q_pe], -1), dense, fields["context_lens"], table,
+                                          fields["query_start_loc"], fields["request_distribution"][2:3], softmax_scale=scale,
+                                          num_kv_heads=heads)[..., :vdim]
+    err = np.abs(got - want)
+    # the absorbed queries are rounded to bf16 once more than in the decompressed form; same bars as the kernel tests
+    assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())

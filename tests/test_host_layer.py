@@ -203,3 +203,60 @@ def test_unified_product_path_refuses_cpu_tensors():
         kernels.unified_attention(q, pool, pool.clone(), i32(2), i32(2, 4), i32(3))
     with pytest.raises(ValueError, match="must match"):
         kernels.unified_attention(q, pool, pool[:, :8].contiguous(), i32(2), i32(2, 4), i32(3))
+
+
+def test_mla_registry_requirements_config_and_errors():
+    from easydel_amd.caching import MLARaggedPagesCache, MLARaggedPagesCacheConfig, MLARaggedPagesCacheView
+    from easydel_amd.operations import MultiLatentRaggedPageAttn, MultiLatentRaggedPageAttnV2
+
+    assert OperationRegistry.get("multi_latent_ragged_page_attention_v1") is MultiLatentRaggedPageAttn
+    assert OperationRegistry.get("multi_latent_ragged_page_attention_v2") is MultiLatentRaggedPageAttnV2
+    req = MultiLatentRaggedPageAttnV2.get_requirements(ExecutionMode.MIXED)
+    assert req.name == "multi_latent_ragged_page_attention"
+    assert req.cache.cache_view_class is MLARaggedPagesCacheView  # the allocator compares view classes by identity
+    assert req.metadata.required & MetadataField.REQUEST_DISTRIBUTION and req.cache.is_compatible_with(CacheType.RAGGED_PAGES)
+
+    # sizing rule of caching/mla_ragged_page/cache.py:196-206: a page costs layers * packed tokens * padded row * bytes
+    cfg = MLARaggedPagesCacheConfig.create(torch.bfloat16, num_hidden_layers=3, num_kv_heads=128, max_model_length=4096,
+                                           kv_lora_rank=512, qk_rope_head_dim=64, page_size=64, free_hbm_bytes=10 * 3 * 64 * 640 * 2,
+                                           hbm_utilization=1.0)
+    assert cfg.num_pages == 10 and cfg.max_num_pages_per_req == 64 and cfg.version == "v1"
+    assert (cfg.kv_lora_rank, cfg.qk_rope_head_dim, cfg.kv_dim, cfg.kv_dim_padded) == (512, 64, 576, 640)
+    assert cfg.get_shape_and_axes()[0] == (10, 32, 2, 640)
+    # legacy aliases (cache.py:163-171) and the checks of create (:172-194)
+    legacy = MLARaggedPagesCacheConfig.create(torch.float32, 1, 1, 128, k_headdim=192, v_headdim=32, page_size=16, num_pages=4)
+    assert legacy.kv_dim_padded == 256 + 128 and legacy.get_shape_and_axes()[0] == (4, 16, 1, 384)
+    with pytest.raises(ValueError, match="kv_lora_rank"):
+        MLARaggedPagesCacheConfig.create(torch.bfloat16, 1, 1, 128, num_pages=4)
+    with pytest.raises(ValueError, match="only supports version='v1'"):
+        MLARaggedPagesCacheConfig.create(torch.bfloat16, 1, 1, 128, kv_lora_rank=512, version="v3", num_pages=4)
+    cache = MLARaggedPagesCache.init_cache(legacy, device="cpu")
+    assert len(cache.views) == 1 and cache.metadata is legacy
+    view = cache.views[0]
+    assert view.key_pages is view.kv_pages and view.value_pages is view.kv_pages and view.concatenate_to_cache(None, None, None) is view
+
+    # argument checks of the operation (multi_latent_ragged_page_attention.py:340-378), before any device work
+    op = OperationRegistry.create("multi_latent_ragged_page_attention_v1", OperationMetadata())
+    qn, qp = torch.zeros(5, 2, 192), torch.zeros(5, 2, 32)
+    kv, pe = torch.zeros(5, 192), torch.zeros(5, 32)
+    meta = SimpleNamespace(context_lens=torch.zeros(2, dtype=torch.int32), pages_tables=torch.zeros(2, 8, dtype=torch.int32),
+                           query_start_loc=torch.zeros(3, dtype=torch.int32), request_distribution=torch.zeros(3, dtype=torch.int32))
+    with pytest.raises(ValueError, match="requires `keys_pe`"):
+        op(queries_nope=qn, queries_pe=qp, keys_values=kv, keys_pe=None, cache_view=view, cache_metadata=meta)
+    with pytest.raises(ValueError, match="must share"):
+        op(queries_nope=qn, queries_pe=qp[:4], keys_values=kv, keys_pe=pe, cache_view=view, cache_metadata=meta)
+    with pytest.raises(ValueError, match="token dimension must match"):
+        op(queries_nope=qn, queries_pe=qp, keys_values=kv[:3], keys_pe=pe, cache_view=view, cache_metadata=meta)
+    with pytest.raises(ValueError, match="rank-3 or rank-4"):
+        op(queries_nope=qn[0], queries_pe=qp, keys_values=kv, keys_pe=pe, cache_view=view, cache_metadata=meta)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):  # CPU tensors reach the product path and are refused
+        op(queries_nope=qn, queries_pe=qp, keys_values=kv, keys_pe=pe, cache_view=view, cache_metadata=meta, unknown_kwarg=1)
+
+
+def test_mla_distribution_is_derived_on_the_device_when_absent():
+    from easydel_amd.operations.multi_latent_ragged_page_attention import _resolve_distribution
+
+    meta = SimpleNamespace(request_distribution=None, query_start_loc=torch.tensor([0, 4, 5, 5], dtype=torch.int32),
+                           context_lens=torch.tensor([4, 9, 0], dtype=torch.int32))
+    # the second vector of tests/inference/test_request_distribution_bounds.py:30-36
+    assert _resolve_distribution(meta).tolist() == [1, 2, 2]
