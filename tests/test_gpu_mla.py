@@ -10,80 +10,7 @@ from rpa_testlib import BF16, F32, orc
 pytestmark = pytest.mark.gpu
 
 
-class MlaBatch:
-    pass
-
-
-def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64, dtype=BF16, pad_rows=0, pad_tokens=0,
-                   row=None, max_pages=None):
-    rng = np.random.default_rng(seed)
-    ctx_lens = np.asarray(ctx_lens, np.int32)
-    q_lens = np.asarray(q_lens, np.int32)
-    n = len(ctx_lens)
-    b = MlaBatch()
-    lay = orc.mla_page_layout_ref(lkv, rope, page_size)
-    b.row = row or lay["kv_dim_padded"]
-    b.off = lay["rope_offset"]
-    b.Hq, b.lkv, b.rope, b.page_size, b.n, b.q_dtype = Hq, lkv, rope, page_size, n, dtype
-    need = [-(-int(c) // page_size) for c in ctx_lens]
-    b.S = n + pad_rows
-    b.M = max_pages or max(max(need), 1)
-    b.P = sum(need) + 5
-    perm = rng.permutation(np.arange(1, b.P))
-    bt = np.zeros((b.S, b.M), np.int32)
-    k = 0
-    for i, m in enumerate(need):
-        bt[i, :m] = perm[k:k + m]
-        k += m
-    b.block_tables = bt
-    b.context_lens = np.zeros(b.S, np.int32)
-    b.context_lens[:n] = ctx_lens
-    qsl = np.zeros(b.S + 1, np.int32)
-    qsl[1:n + 1] = np.cumsum(q_lens)
-    qsl[n + 1:] = qsl[n]
-    b.query_start_loc = qsl
-    b.T = int(qsl[n]) + pad_tokens
-    b.distribution = np.array([0, 0, n], np.int32)
-    b.num_seqs = np.array([n], np.int32)
-
-    def enc(x):
-        if dtype == BF16:
-            raw = orc.f32_to_bf16_bits(x.astype(np.float32))
-            return raw, orc.bf16_bits_to_f32(raw).astype(np.float64)
-        x = x.astype(np.float32)
-        return x, x.astype(np.float64)
-
-    b.qn_raw, b.qn_val = enc(rng.standard_normal((b.T, Hq, lkv)))
-    b.qp_raw, b.qp_val = enc(rng.standard_normal((b.T, Hq, rope)))
-    b.kv_raw, b.kv_val = enc(rng.standard_normal((b.T, lkv)))
-    b.pe_raw, b.pe_val = enc(rng.standard_normal((b.T, rope)))
-    b.pages_raw, b.pages_val = enc(rng.standard_normal((b.P, page_size, b.row)))  # padding holds noise: never read
-    return b
-
-
-def mla_oracle(b, *, fused=True, **kw):
-    pages = b.pages_val
-    if fused:
-        pages = orc.mla_page_scatter_ref(b.kv_val, b.pe_val, pages, b.context_lens, b.block_tables, b.query_start_loc, b.num_seqs)
-    out = orc.mla_ragged_paged_attention_ref(b.qn_val, b.qp_val, pages, b.context_lens, b.block_tables, b.query_start_loc,
-                                             b.num_seqs, kv_lora_rank=b.lkv, qk_rope_head_dim=b.rope, **kw)
-    return out, pages
-
-
-def run_gpu_mla(b, *, fused=True, softmax_aux=None, device="cuda:0", **kw):
-    import torch
-
-    from easydel_amd import kernels
-
-    t = lambda raw: tl.to_torch(raw, b.q_dtype, device)
-    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(device)
-    pages = t(b.pages_raw)
-    aux = None if softmax_aux is None else torch.from_numpy(np.asarray(softmax_aux, np.float32)).to(device)
-    out, pages = kernels.mla_ragged_paged_attention(
-        t(b.qn_raw), t(b.qp_raw), t(b.kv_raw) if fused else None, t(b.pe_raw) if fused else None, pages,
-        i32(b.context_lens), i32(b.block_tables), i32(b.query_start_loc), i32(b.distribution), softmax_aux=aux, **kw)
-    torch.cuda.synchronize()
-    return tl.from_torch(out, b.q_dtype), tl.from_torch(pages, b.q_dtype)
+from rpa_testlib import make_mla_batch, mla_oracle, run_gpu_mla  # noqa: E402
 
 
 def check(b, what, *, fused=True, softmax_aux=None, **kw):
@@ -196,3 +123,51 @@ def test_padded_tokens_are_zeroed_and_bad_arguments_are_reported():
         kernels.mla_ragged_paged_attention(q, q[..., :64].contiguous(), None, None, pages, i(5, 5), i(1, 2), i(0, 1, 2), i(0, 0, 2))
     with pytest.raises(ValueError, match="must share"):
         kernels.mla_ragged_paged_attention(q, q[:1, :, :64].contiguous(), None, None, pages, i(5, 5), i(1, 2), i(0, 1, 2), i(0, 0, 2))
+
+
+def test_hip_graph_replay_matches_eager_and_follows_new_metadata():
+    # the call neither allocates nor synchronises nor clears memory with a memset node: the write, the plan, the unit
+    # list, the attention (rows split over key chunks) and the merge replay from a captured graph
+    import torch
+
+    from easydel_amd import kernels
+
+    dev = "cuda:0"
+    b = make_mla_batch(11, [2500, 65, 700, 1, 1200], [1, 1, 30, 1, 2], Hq=16, pad_rows=2, pad_tokens=1)
+    t = lambda raw: tl.to_torch(raw, BF16, dev)  # noqa: E731
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(dev)  # noqa: E731
+    qn, qp, kv, pe, pages = t(b.qn_raw), t(b.qp_raw), t(b.kv_raw), t(b.pe_raw), t(b.pages_raw)
+    ctx, bt, qsl, dist = i32(b.context_lens), i32(b.block_tables), i32(b.query_start_loc), i32(b.distribution)
+    out = torch.empty_like(qn)
+
+    def call():
+        kernels.mla_ragged_paged_attention(qn, qp, kv, pe, pages, ctx, bt, qsl, dist, softmax_scale=SCALE, out=out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()  # warm-up on the capture stream: sizes the cached workspace outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = out.clone()
+    want, _ = mla_oracle(b, softmax_scale=SCALE)
+    tl.assert_close(tl.from_torch(eager, BF16), want, b, "eager")
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call()
+    for rep in range(4):
+        out.zero_()
+        qn.mul_(1.0)  # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
+    ctx[0] = 2100  # new metadata in the same buffers: nothing is baked in on the host
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    b.context_lens[0] = 2100
+    b.pages_raw = pages.view(torch.int16).cpu().numpy().view(np.uint16)  # the pages as the replays left them
+    b.pages_val = orc.bf16_bits_to_f32(b.pages_raw).astype(np.float64)
+    want, _ = mla_oracle(b, softmax_scale=SCALE)
+    tl.assert_close(tl.from_torch(out, BF16), want, b, "graph replay with new metadata")
