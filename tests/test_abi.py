@@ -62,3 +62,29 @@ def test_host_only_entry_points():
     assert lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1) < n
     _lib.set_tunable("max_splits", prev)
     assert _lib.set_tunable("no_such_knob", 1) == -1
+
+
+def test_multi_latent_entry_points_validate_before_any_device_work():
+    lib = _lib.load()
+    a = 0x7000_0000_0000
+    args = dict(T=4, S=2, M=8, P=16, pg=64, Hq=16, rank=512, rope=64, row=640, qd=1, kd=1)
+
+    def call(qn=a, qp=a, kv=None, pe=None, pages=a, ctx=a, bt=a, qsl=a, dist=a, out=a, ws=a, ws_bytes=1 << 24, aux=None, **over):
+        v = dict(args, **over)
+        return lib.rpa_mla_ragged_paged_attention(None, qn, qp, kv, pe, pages, ctx, bt, qsl, dist, out, ws, ws_bytes, v["T"], v["S"],
+                                                  v["M"], v["P"], v["pg"], v["Hq"], v["rank"], v["rope"], v["row"], v["qd"], v["kd"],
+                                                  0.07, 0, 0.0, aux)
+
+    assert call(row=568) == _lib.RPA_ERR_INVALID_ARGUMENT and b"row_elems" in lib.rpa_last_error()
+    assert call(rank=1024, row=2048) == _lib.RPA_ERR_UNSUPPORTED and b"kv_lora_rank" in lib.rpa_last_error()
+    assert call(kd=2) == _lib.RPA_ERR_UNSUPPORTED and b"kv_dtype" in lib.rpa_last_error()
+    assert call(dist=None) == _lib.RPA_ERR_INVALID_ARGUMENT and b"distribution" in lib.rpa_last_error()
+    assert call(qn=None) == _lib.RPA_ERR_INVALID_ARGUMENT and b"null pointer" in lib.rpa_last_error()
+    assert call(kv=a, pe=None) == _lib.RPA_ERR_INVALID_ARGUMENT and b"keys_pe" in lib.rpa_last_error()
+    assert call(out=a + 8) == _lib.RPA_ERR_INVALID_ARGUMENT and b"16-byte aligned" in lib.rpa_last_error()
+    assert call(ws_bytes=64) == _lib.RPA_ERR_WORKSPACE and b"workspace" in lib.rpa_last_error()
+    assert call(T=0) == 0  # an empty batch is a no-op
+    n = lib.rpa_mla_workspace_bytes(256, 256, 128, 64, 128, 512, 1, 1)
+    assert n > 256 * 128 * 514 * 4  # at least one chunk's partial rows when the shapes ask for a split
+    assert lib.rpa_mla_page_scatter(None, a, a, a, a, a, a, a, 4, 2, 8, 16, 64, 512, 64, 640, 1) == _lib.RPA_ERR_UNSUPPORTED
+    assert lib.rpa_mla_page_scatter(None, None, a, a, a, a, a, a, 4, 2, 8, 16, 64, 512, 64, 640, 2) == _lib.RPA_ERR_INVALID_ARGUMENT
