@@ -127,7 +127,7 @@ void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* min_chunk) {
   const size_t per = part_o_bytes(T, Hq, lkv) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   *max_chunks = (int)chunks;
-  *min_chunk = g_mla_min_chunk.load() > 0 ? g_mla_min_chunk.load() : (Hq >= 64 ? 2048 : 512);
+  *min_chunk = g_mla_min_chunk.load() > 0 ? g_mla_min_chunk.load() : (Hq >= 64 ? 1024 : 512);
 }
 
 bool mla_shape_on_mfma(int page_size, int lkv, int rope, int row_elems, int q_dtype, int kv_dtype) {

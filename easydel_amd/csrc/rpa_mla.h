@@ -24,9 +24,11 @@ struct MlaParams {
   void* out;       // [T][Hq][lkv], query dtype
   float* part_o;   // [max_chunks][T][Hq][lkv]
   float* part_ml;  // [max_chunks][T][Hq][2]  (running max in log2 units, running sum)
-  int2* plan;      // [row-tile slots] (sequence, key chunks) of the row tile at a slot; chunks = 0: no such tile
-  int32_t* n_units;  // [1] number of (row tile, key chunk) units of the batch = workgroups with work
-  int2* units;     // [n_units] (slot, chunk), slot-major
+  int2* plan;      // [row-tile slots] (sequence, key chunks | keys / 64 of a chunk << 8) of the row tile at a slot;
+                   // chunks = 0: no such tile
+  int32_t* n_units;  // [0] number of (row tile, key chunk) units of the batch = workgroups with work;
+                     // [1] 1 if the list is sorted longest first, 0 if it is in slot order
+  int2* units;     // [n_units[0]] (slot, chunk)
   int T, S, M, P, page_size, Hq, lkv, rope, rope_off, row_elems;
   int64_t token_stride, page_stride;  // bytes
   int q_dtype, kv_dtype;

@@ -156,44 +156,77 @@ __global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots)
     const MlaSeq sp = mla_seq(p, lo_i);
     const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * p.Hq) / kMlaRows) + lo_i);
     if (sp.live && tile_in_seq >= 0 && tile_in_seq * kMlaRows < sp.q_len * p.Hq) {
+      const MlaTile mt = mla_tile(p, sp, tile_in_seq * kMlaRows);
       unit.x = lo_i;
-      unit.y = mla_tile(p, sp, tile_in_seq * kMlaRows).n_chunks;
+      unit.y = mt.n_chunks | ((min(mt.chunk, mt.kv_hi - mt.kv_lo) >> 6) << 8);  // chunks, and keys / 64 of one chunk
     }
   }
   p.plan[slot] = unit;
 }
 
-// The units (row tile, key chunk) of the batch in one dense list, slot-major.  The MFMA kernel's grid is sized from
-// the static bounds and most of its slots are empty; left in place, the empty ones form a regular pattern (a batch of
-// single tokens with 128 heads fills every other slot) that the hardware's round-robin placement of consecutive
-// blocks turns into idle shader engines: measured, each engine was busy 43 % of such a kernel's duration.
-// One block: a scan over the plan's chunk counts, 1024 slots a pass.
+// The units (row tile, key chunk) of the batch in one dense list.  The MFMA kernel's grid is sized from the static
+// bounds and most of its slots are empty; left in place, the empty ones form a regular pattern (a batch of single tokens
+// with 128 heads fills every other slot) that the hardware's round-robin placement of consecutive blocks turns into
+// idle shader engines: measured, each engine was busy 43 % of such a kernel's duration.
+// One block: a scan over the plan's chunk counts, 1024 slots a pass.  A batch of up to kMlaSortSlots slots (decode
+// and small mixed batches, where a unit is a sizeable share of a CU's work and the lengths differ many-fold) is listed
+// longest first, in eight classes of chunk length, one scan per class: workgroups are handed out in list order, so
+// the long units start first and the short ones fill in behind them.  Larger batches are listed in slot order in
+// one scan; n_units[1] says which.
+constexpr int kMlaSortSlots = 4096;
+constexpr int kMlaLenClasses = 8;
+
 __global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_slots) {
   __shared__ int wave_tot[16];
   __shared__ int running_s;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const bool sort = n_slots <= kMlaSortSlots;
+  int max_len = 0;
+  if (sort) {
+    for (int slot = tid; slot < n_slots; slot += 1024) {
+      const int y = p.plan[slot].y;
+      if (y & 0xff) max_len = max(max_len, y >> 8);
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) max_len = max(max_len, __shfl_xor(max_len, o));
+    if (lane == 0) wave_tot[wv] = max_len;
+    __syncthreads();
+    for (int w = 0; w < 16; ++w) max_len = max(max_len, wave_tot[w]);
+  }
+  __syncthreads();
   if (tid == 0) running_s = 0;
   __syncthreads();
-  for (int base = 0; base < n_slots; base += 1024) {
-    const int slot = base + tid;
-    const int v = slot < n_slots ? p.plan[slot].y : 0;
-    int incl = v;
+  const int classes = sort ? kMlaLenClasses : 1;
+  for (int cls = classes - 1; cls >= 0; --cls) {
+    for (int base = 0; base < n_slots; base += 1024) {
+      const int slot = base + tid;
+      int v = 0;
+      if (slot < n_slots) {
+        const int y = p.plan[slot].y;
+        const int mine = sort ? min(kMlaLenClasses - 1, ((y >> 8) * kMlaLenClasses) / (max_len + 1)) : 0;
+        if (mine == cls) v = y & 0xff;
+      }
+      int incl = v;
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int up = __shfl_up(incl, o);
-      if (lane >= o) incl += up;
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(incl, o);
+        if (lane >= o) incl += up;
+      }
+      if (lane == 63) wave_tot[wv] = incl;
+      __syncthreads();
+      int before = running_s;
+      for (int w = 0; w < wv; ++w) before += wave_tot[w];
+      const int first = before + incl - v;
+      for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c);
+      __syncthreads();
+      if (tid == 1023) running_s = before + incl;
+      __syncthreads();
     }
-    if (lane == 63) wave_tot[wv] = incl;
-    __syncthreads();
-    int before = running_s;
-    for (int w = 0; w < wv; ++w) before += wave_tot[w];
-    const int first = before + incl - v;
-    for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c);
-    __syncthreads();
-    if (tid == 1023) running_s = before + incl;
-    __syncthreads();
   }
-  if (tid == 0) p.n_units[0] = running_s;
+  if (tid == 0) {
+    p.n_units[0] = running_s;
+    p.n_units[1] = sort ? 1 : 0;
+  }
 }
 
 // ---- MFMA kernel ----------------------------------------------------------------------------------------------------
@@ -250,13 +283,14 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   // The grid is sized from the static bounds, so most of its blocks have nothing to do, and a workgroup holds a
   // whole compute unit: the plan kernel has looked every slot up beforehand, and a block learns with one load
   // whether it has work.
-  // Block -> unit of the dense list.  Consecutive blocks go to the eight XCDs in turn; unit = (block % 8) * n8 +
-  // block / 8 hands every XCD a contiguous eighth of the list, so that the row tiles of a long prompt, which read
-  // the same keys, share one XCD's L2.
+  // Block -> unit of the dense list.  Consecutive blocks go to the eight XCDs in turn.  A list in slot order (large
+  // batches) is dealt in contiguous eighths, unit = (block % 8) * n8 + block / 8, so that the row tiles of a long
+  // prompt, which read the same keys, share one XCD's L2; a list sorted longest first is dealt block by block.
   const int total = p.n_units[0];
   const int n8 = (total + kXcds - 1) / kXcds;
-  const int u = (blockIdx.x % kXcds) * n8 + blockIdx.x / kXcds;
-  if ((int)(blockIdx.x / kXcds) >= n8 || u >= total) return;
+  const bool sorted = p.n_units[1] != 0;
+  const int u = sorted ? (int)blockIdx.x : (int)((blockIdx.x % kXcds) * n8 + blockIdx.x / kXcds);
+  if ((!sorted && (int)(blockIdx.x / kXcds) >= n8) || u >= total) return;
   const int2 sc = p.units[u];
   const int slot = sc.x, chunk = sc.y;
   const int2 unit = p.plan[slot];

@@ -266,7 +266,7 @@ int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t
  *                    applies (page_size % 32 == 0); 0: every prefill tile is staged through registers
  *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
  *                    the shapes); set it before sizing the workspace
- *   "mla_min_chunk"  fewest keys of such a chunk (rounded up to 64; 0 = default: 2048 at 64 heads and more, else 512)
+ *   "mla_min_chunk"  fewest keys of such a chunk (rounded up to 64; 0 = default: 1024 at 64 heads and more, else 512)
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
  *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
  *                    1 = decode plan kernel, 2 = decode kernel, 4 = prefill / large-row kernel,
