@@ -115,3 +115,71 @@ def test_config5_gemma_long_context_first_sequence(gpu, windowed):
                                 softmax_scale=w.softmax_scale, logits_soft_cap=w.logits_soft_cap)
         worst = _oracle_on_sample(w2, tens, [0], out)
     print(f"C5 windowed={windowed}: worst max-abs {worst:.3e}", flush=True)
+
+
+@pytest.mark.parametrize("Hq", [128, 16])
+def test_multi_latent_decode_at_benchmark_size(gpu, Hq):
+    """256 sequences of 512..8192 tokens over latent pages (512 + 64, bf16), one new token each: the fused write is in
+    place bit-exactly, sampled sequences match the oracle on the pages fetched back, a split over more key chunks
+    agrees, and two runs are bit-identical (the unit list is built by scans, not atomics)."""
+    from easydel_amd import _lib
+
+    rng = np.random.default_rng(0)
+    n, lkv, rope, row, pg = 256, 512, 64, 640, 64
+    ctx = rng.integers(512, 8193, size=n).astype(np.int32)
+    need = -(-ctx // pg)
+    M, P = int(need.max()), int(need.sum()) + 64
+    perm = rng.permutation(np.arange(1, P)).astype(np.int32)
+    bt = np.zeros((n, M), np.int32)
+    k = 0
+    for i, m in enumerate(need):
+        bt[i, :m] = perm[k:k + m]
+        k += m
+    g = torch.Generator(device=gpu).manual_seed(1)
+    rnd = lambda *shape: torch.randn(*shape, generator=g, device=gpu, dtype=torch.float32).to(torch.bfloat16)  # noqa: E731
+    pages = torch.empty(P, pg, row, dtype=torch.bfloat16, device=gpu)
+    for lo in range(0, P, 4096):
+        pages[lo:lo + 4096] = rnd(min(4096, P - lo), pg, row)
+    qn, qp, kv, pe = rnd(n, Hq, lkv), rnd(n, Hq, rope), rnd(n, lkv), rnd(n, rope)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(gpu)  # noqa: E731
+    ctx_d, bt_d, qsl_d, dist_d = i32(ctx), i32(bt), i32(np.arange(n + 1)), i32([0, 0, n])
+    scale = 192 ** -0.5
+    sample = sorted({int(np.argmin(ctx)), int(np.argmax(ctx)), 3, 100, 200})
+    last = torch.from_numpy(np.array([bt[i, (ctx[i] - 1) // pg] for i in range(n)], np.int64)).to(gpu)
+    before = pages[last].clone()
+
+    out, pages_after = kernels.mla_ragged_paged_attention(qn, qp, kv, pe, pages, ctx_d, bt_d, qsl_d, dist_d, softmax_scale=scale)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    # the write: latent row, rope key, zeroed padding at slot (ctx - 1) of the last page; the other slots untouched
+    after = pages_after[last]
+    slots = torch.from_numpy(((ctx - 1) % pg).astype(np.int64)).to(gpu)
+    rows = after[torch.arange(n, device=gpu), slots]
+    assert torch.equal(rows[:, :lkv], kv) and torch.equal(rows[:, lkv:lkv + rope], pe) and not rows[:, lkv + rope:].any()
+    keep = torch.ones(n, pg, dtype=torch.bool, device=gpu)
+    keep[torch.arange(n, device=gpu), slots] = False
+    assert torch.equal(after[keep], before[keep])
+    # sampled sequences against the oracle, on the pages as they are now
+    bf = lambda t: orc.bf16_bits_to_f32(t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)  # noqa: E731
+    worst = 0.0
+    for i in sample:
+        m = int(need[i])
+        seq_pages = bf(pages_after[torch.from_numpy(bt[i, :m].astype(np.int64)).to(gpu)])
+        want = orc.mla_ragged_paged_attention_ref(bf(qn[i:i + 1]), bf(qp[i:i + 1]), seq_pages, [ctx[i]], np.arange(m)[None], [0, 1], [1],
+                                                  kv_lora_rank=lkv, qk_rope_head_dim=rope, softmax_scale=scale)
+        err = np.abs(bf(out[i:i + 1]) - want)
+        assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (i, err.max(), err.mean())
+        worst = max(worst, err.max())
+    print(f"MLA decode, {Hq} heads, full size: worst max-abs on sampled sequences {worst:.3e}", flush=True)
+    # read-only repeats: bit-identical run to run; more key chunks: the same within the tolerance
+    again, _ = kernels.mla_ragged_paged_attention(qn, qp, None, None, pages_after, ctx_d, bt_d, qsl_d, dist_d, softmax_scale=scale)
+    again2, _ = kernels.mla_ragged_paged_attention(qn, qp, None, None, pages_after, ctx_d, bt_d, qsl_d, dist_d, softmax_scale=scale)
+    torch.cuda.synchronize()
+    assert torch.equal(again, again2) and torch.equal(again, out)
+    prev = _lib.set_tunable("mla_chunks", 8)
+    try:
+        split, _ = kernels.mla_ragged_paged_attention(qn, qp, None, None, pages_after, ctx_d, bt_d, qsl_d, dist_d, softmax_scale=scale)
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_tunable("mla_chunks", prev)
+    assert (split.float() - out.float()).abs().max().item() <= tl.TOL_BF16_MAX
