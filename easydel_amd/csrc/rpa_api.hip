@@ -500,7 +500,7 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
   p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
   p.mfma = (!g_force_generic.load() && rpa::mla_mfma_supported(p)) ? 1 : 0;
   hipStream_t s = (hipStream_t)stream;
-  if (keys_values) {
+  if (keys_values && !p.mfma) {  // on the matrix-core path the write rides along with the plan kernel's launch
     const int err = rpa::launch_mla_scatter(s, p);
     if (err) return hip_fail(err, "MLA page write launch");
   }

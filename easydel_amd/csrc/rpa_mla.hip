@@ -29,9 +29,8 @@ namespace {
 // ---- page write ------------------------------------------------------------------------------------------------
 // One wavefront per query token: its latent row and rope key into the page slot of its position, padding zeroed.
 template <typename E>
-__global__ __launch_bounds__(256) void mla_scatter_kernel(MlaParams p) {
+__device__ __forceinline__ void mla_scatter_token(const MlaParams& p, int t) {
   const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= p.T) return;
   const int n_live = mla_live_rows(p);
   if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) return;
@@ -52,6 +51,11 @@ __global__ __launch_bounds__(256) void mla_scatter_kernel(MlaParams p) {
     else if (e >= p.rope_off && e < p.rope_off + p.rope) v = pe[e - p.rope_off];
     row[e] = v;
   }
+}
+
+template <typename E>
+__global__ __launch_bounds__(256) void mla_scatter_kernel(MlaParams p) {
+  mla_scatter_token<E>(p, blockIdx.x * 4 + (threadIdx.x >> 6));
 }
 
 // ---- fp32 kernel: one wavefront per (query token, head) ----------------------------------------------------------
@@ -142,7 +146,15 @@ __global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
 // ---- plan: which sequence and how many key chunks each row-tile slot of the MFMA kernel's grid holds -------------
 // Sequence i starts at slot floor(qsl[i] * Hq / 128) + i (its row tiles follow), so the slots of a batch are found
 // without a scan; slots between sequences, past the live ones, or of rows before position 0 hold no tile.
-__global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots) {
+// In the fused call the blocks behind the plan's write the new rows into the pages (four tokens a block): one
+// launch less before the attention kernel, which waits for both anyway.
+__global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots, int plan_blocks) {
+  if ((int)blockIdx.x >= plan_blocks) {
+    const int t = ((int)blockIdx.x - plan_blocks) * 4 + (threadIdx.x >> 6);
+    if (p.kv_dtype == RPA_F32) mla_scatter_token<uint32_t>(p, t);
+    else mla_scatter_token<uint16_t>(p, t);
+    return;
+  }
   const int slot = blockIdx.x * 256 + threadIdx.x;
   if (slot >= n_slots) return;
   int2 unit = {0, 0};
@@ -738,7 +750,9 @@ int launch_mla_mfma(hipStream_t stream, const MlaParams& p) {
   const int64_t slots = mla_plan_slots(p.T, p.S, p.Hq);
   const int64_t blocks = (slots * p.max_chunks + kXcds - 1) / kXcds * kXcds;  // most units the batch can have
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(mla_plan_kernel, dim3((unsigned)((slots + 255) / 256)), dim3(256), 0, stream, p, (int)slots);
+  const int plan_blocks = (int)((slots + 255) / 256);
+  const int write_blocks = p.new_kv ? (p.T + 3) / 4 : 0;  // the page write rides along (see mla_plan_kernel)
+  hipLaunchKernelGGL(mla_plan_kernel, dim3((unsigned)(plan_blocks + write_blocks)), dim3(256), 0, stream, p, (int)slots, plan_blocks);
   hipLaunchKernelGGL(mla_compact_kernel, dim3(1), dim3(1024), 0, stream, p, (int)slots);
   if (p.softcap > 0.f) hipLaunchKernelGGL((mla_attn_kernel<true>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
   else hipLaunchKernelGGL((mla_attn_kernel<false>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
