@@ -105,9 +105,20 @@ __global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
       const int page = min(max(bt[j / p.page_size], 0), p.P - 1);
       row = (int64_t)page * p.page_stride + (int64_t)(j % p.page_size) * p.token_stride;
       const void* kp = pages + row;
-      float dot = 0.f;
-      for (int d = 0; d < lkv; ++d) dot = fmaf(q_s[d], load_elem<KVT>(kp, d), dot);
-      for (int d = 0; d < rope; ++d) dot = fmaf(q_s[lkv + d], load_elem<KVT>(kp, p.rope_off + d), dot);
+      // eight partial sums: a single chain of 576 float additions drifts past the 1e-5 the fp32 path is held to
+      float part[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      int d = 0;
+      for (; d + 8 <= lkv; d += 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) part[u] = fmaf(q_s[d + u], load_elem<KVT>(kp, d + u), part[u]);
+      }
+      for (; d < lkv; ++d) part[d & 7] = fmaf(q_s[d], load_elem<KVT>(kp, d), part[d & 7]);
+      for (d = 0; d + 8 <= rope; d += 8) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) part[u] = fmaf(q_s[lkv + d + u], load_elem<KVT>(kp, p.rope_off + d + u), part[u]);
+      }
+      for (; d < rope; ++d) part[d & 7] = fmaf(q_s[lkv + d], load_elem<KVT>(kp, p.rope_off + d), part[d & 7]);
+      const float dot = ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
       s = dot * p.scale;
       if (p.softcap > 0.f) s = p.softcap * tanhf(s / p.softcap);
     }

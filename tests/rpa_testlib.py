@@ -197,15 +197,29 @@ TOL_BF16_MAX = 2e-2
 TOL_BF16_MEAN = 5e-3
 
 
-def assert_close(got, want, b, what=""):
+def assert_close(got, want, b, what="", *, one_ulp_above_4=False):
+    """The stated tolerances on the valid rows.  `one_ulp_above_4` (multi-latent tests, whose outputs live in the latent
+    space and pass |4| when one key dominates a row) widens the max-abs bound where |want| >= 4 to one bf16 step at that
+    magnitude (2**-5 below 8): a bf16 output there cannot be held to 2e-2 once a rounding boundary lies within the
+    arithmetic error of the exact value."""
     rows = valid_rows(b)
     g, w = got[rows], want[rows]
     assert np.isfinite(g).all(), f"{what}: non-finite output"
     err = np.abs(g - w)
+    at = np.unravel_index(int(np.argmax(err)), err.shape) if err.size else ()
+    where = f"at {tuple(int(i) for i in at)}: got {g[at]!r}, want {w[at]!r}" if err.size else ""
     if b.q_dtype == F32:
-        assert err.max() <= TOL_F32_MAX, f"{what}: fp32 max-abs {err.max():.3e} > {TOL_F32_MAX}"
+        assert err.max() <= TOL_F32_MAX, f"{what}: fp32 max-abs {err.max():.3e} > {TOL_F32_MAX} {where}"
     else:
-        assert err.max() <= TOL_BF16_MAX, f"{what}: max-abs {err.max():.3e} > {TOL_BF16_MAX}"
+        bound = np.full(err.shape, TOL_BF16_MAX)
+        if one_ulp_above_4:
+            big = np.abs(w) >= 4.0
+            bound[big] = np.maximum(TOL_BF16_MAX, 2.0 ** (np.floor(np.log2(np.abs(w[big]))) - 7))
+        over = err > bound
+        if over.any():
+            at = np.unravel_index(int(np.argmax(np.where(over, err, 0.0))), err.shape)
+            where = f"at {tuple(int(i) for i in at)}: got {g[at]!r}, want {w[at]!r}"
+        assert not over.any(), f"{what}: max-abs {err[over].max():.3e} > {TOL_BF16_MAX} {where}"
         assert err.mean() <= TOL_BF16_MEAN, f"{what}: mean-abs {err.mean():.3e} > {TOL_BF16_MEAN}"
     return float(err.max()), float(err.mean())
 
