@@ -197,11 +197,13 @@ TOL_BF16_MAX = 2e-2
 TOL_BF16_MEAN = 5e-3
 
 
-def assert_close(got, want, b, what="", *, one_ulp_above_4=False):
-    """The stated tolerances on the valid rows.  `one_ulp_above_4` (multi-latent tests, whose outputs live in the latent
-    space and pass |4| when one key dominates a row) widens the max-abs bound where |want| >= 4 to one bf16 step at that
-    magnitude (2**-5 below 8): a bf16 output there cannot be held to 2e-2 once a rounding boundary lies within the
-    arithmetic error of the exact value."""
+def assert_close(got, want, b, what="", *, one_ulp_above_4=True):
+    """The stated tolerances on the valid rows.  Where |want| >= 4 the bf16 max-abs bound is one bf16 step at that
+    magnitude (2**-5 below 8, 2**-4 below 16) instead of 2e-2: the output is a bf16 number, whose spacing there exceeds
+    2e-2, so even the correctly rounded result can miss by more (seen: a row with one visible key whose fp8 value
+    dequantises to 8.0353 comes back as 8.0625, the nearest bf16).  Outputs of that size need a row that one key
+    dominates and values beyond four standard deviations, scaled fp8 / int8 pages, or the latent space of the
+    multi-latent operation; on the benchmark shapes every output is below 4 and the bound is the plain 2e-2."""
     rows = valid_rows(b)
     g, w = got[rows], want[rows]
     assert np.isfinite(g).all(), f"{what}: non-finite output"
