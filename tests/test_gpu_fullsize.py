@@ -183,3 +183,74 @@ def test_multi_latent_decode_at_benchmark_size(gpu, Hq):
     finally:
         _lib.set_tunable("mla_chunks", prev)
     assert (split.float() - out.float()).abs().max().item() <= tl.TOL_BF16_MAX
+
+
+def test_pages_at_the_top_of_a_160_gib_pool(gpu):
+    """The pool a 288 GB card can hold: page byte offsets beyond 2**37.  A mixed batch whose pages all lie in the last
+    few hundred pages of a 160 GiB pool (the rest is never initialised and never read) goes through the fused write +
+    attention call: the written pages bit-exact, the output against the oracle, and the same bits as the same batch in
+    a small pool."""
+    Hq, Hkv, D, pg = 32, 8, 128, 64
+    b = tl.make_batch(91, [700, 65, 1500, 300, 2000, 4100], [1, 1, 2, 300, 1, 40], Hq=Hq, Hkv=Hkv, D=D, page_size=pg, pad_rows=2)
+    rng = np.random.default_rng(92)
+    key_raw = orc.f32_to_bf16_bits(rng.standard_normal((b.T, Hkv, D), dtype=np.float32))
+    val_raw = orc.f32_to_bf16_bits(rng.standard_normal((b.T, Hkv, D), dtype=np.float32))
+    key_val = orc.bf16_bits_to_f32(key_raw).astype(np.float64)
+    val_val = orc.bf16_bits_to_f32(val_raw).astype(np.float64)
+    want_pages = orc.page_scatter_ragged_ref(key_val, val_val, b.kv_val, b.context_lens, b.block_tables, b.query_start_loc, b.num_seqs)
+    want = tl.oracle_out(b, kv_val=want_pages)
+
+    page_bytes = pg * 2 * Hkv * D * 2
+    P_big = (160 << 30) // page_bytes
+    base = P_big - b.P
+    assert base * page_bytes > (1 << 37)
+    torch.cuda.empty_cache()  # a pool an earlier test has dropped still sits in torch's allocator
+    free, _ = torch.cuda.mem_get_info()
+    if free < (P_big * page_bytes) + (4 << 30):
+        pytest.skip(f"needs a 160 GiB pool, {free >> 30} GiB free on this device")
+    d = tl.device_batch(b, gpu)
+    key, val = tl.to_torch(key_raw, tl.BF16, gpu), tl.to_torch(val_raw, tl.BF16, gpu)
+    dist = torch.tensor([0, 0, b.n], dtype=torch.int32, device=gpu)
+    print(f"[pool] {P_big} pages of {page_bytes} B, batch pages at {base}..{P_big - 1}", flush=True)
+
+    small = d["kv_pages"].clone()
+    out_small, small = kernels.ragged_paged_attention_v3(d["query"], key, val, small, d["context_lens"], d["block_tables"],
+                                                         d["query_start_loc"], dist)
+    big = torch.empty((P_big, pg, 2 * Hkv, D), dtype=torch.bfloat16, device=gpu)
+    big[base:] = d["kv_pages"]
+    bt_big = torch.where(d["block_tables"] > 0, d["block_tables"] + base, d["block_tables"])
+    out_big, big = kernels.ragged_paged_attention_v3(d["query"], key, val, big, d["context_lens"], bt_big, d["query_start_loc"], dist)
+    torch.cuda.synchronize()
+    got_pages = tl.from_torch(big[base:], tl.BF16)
+    np.testing.assert_array_equal(got_pages, want_pages, err_msg="pages after the write at the top of the pool")
+    tl.assert_close(tl.from_torch(out_big, tl.BF16), want, b, "160 GiB pool")
+    assert torch.equal(out_big, out_small), "the same batch must give the same bits wherever its pages lie"
+    del big
+    torch.cuda.empty_cache()
+
+
+def test_latent_pages_at_the_top_of_a_160_gib_pool(gpu):
+    """The same for the multi-latent call: latent pages (80 KiB each) at the top of a 160 GiB pool."""
+    b = tl.make_mla_batch(93, [700, 65, 1500, 300, 2000], [1, 1, 2, 150, 1], Hq=16, pad_rows=1)
+    want, want_pages = tl.mla_oracle(b, fused=True, softmax_scale=(128 + 64) ** -0.5)
+    page_bytes = b.page_size * b.row * 2
+    P_big = (160 << 30) // page_bytes
+    base = P_big - b.P
+    torch.cuda.empty_cache()  # a pool an earlier test has dropped still sits in torch's allocator
+    free, _ = torch.cuda.mem_get_info()
+    if free < (P_big * page_bytes) + (4 << 30):
+        pytest.skip(f"needs a 160 GiB pool, {free >> 30} GiB free on this device")
+    t = lambda raw: tl.to_torch(raw, tl.BF16, gpu)
+    i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(gpu)
+    big = torch.empty((P_big, b.page_size, b.row), dtype=torch.bfloat16, device=gpu)
+    big[base:] = t(b.pages_raw)
+    bt_big = np.where(b.block_tables > 0, b.block_tables + base, b.block_tables)
+    print(f"[pool] {P_big} latent pages of {page_bytes} B, batch pages at {base}..{P_big - 1}", flush=True)
+    out, big = kernels.mla_ragged_paged_attention(t(b.qn_raw), t(b.qp_raw), t(b.kv_raw), t(b.pe_raw), big, i32(b.context_lens),
+                                                  i32(bt_big), i32(b.query_start_loc), i32(b.distribution),
+                                                  softmax_scale=(128 + 64) ** -0.5)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(tl.from_torch(big[base:], tl.BF16), want_pages, err_msg="latent pages after the write")
+    tl.assert_close(tl.from_torch(out, tl.BF16), want, b, "160 GiB latent pool")
+    del big
+    torch.cuda.empty_cache()
