@@ -488,13 +488,28 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   const int S = p.S, tid = threadIdx.x;
   const int per = (S + 1023) / 1024;
   const int i0 = min(S, tid * per), i1 = min(S, i0 + per);
-  __shared__ int s_large;
-  if (tid == 0) s_large = 0;
+  __shared__ int s_large, s_merge;
+  if (tid == 0) {
+    s_large = 0;
+    // Does the merge kernel have anything to do?  Rows of padded tokens to zero ...
+    const int n_live = live_rows(p);
+    s_merge = (n_live <= 0 || p.qsl[0] > 0 || p.qsl[n_live] < p.T) ? 1 : 0;
+  }
   __syncthreads();
   auto span_of = [&](int i, int& toks) -> int {
     const SeqPlan sp = seq_plan(p, i);
     toks = 0;
     if (sp.live && !sp.small_rows) s_large = 1;  // benign race: every writer stores 1
+    // ... rows of sequences with tokens but no context to zero, partial rows of the decode kernel (any sequence of its
+    // class may be cut by a span boundary), or row tiles of the large-row kernel cut into key chunks (a bound on the
+    // keys one tile visits, not the exact count: a flag that is set without need only costs the merge kernel's look)
+    if (i < live_rows(p) && sp.q_len > 0) {
+      if (!sp.live || sp.small_rows) s_merge = 1;
+      else if (p.pre_max_chunks > 1) {
+        const int reach = p.window > 0 ? min(sp.ctx, p.window + kPrefillRows / p.group + 64) : sp.ctx;
+        if (reach > p.pre_chunk) s_merge = 1;
+      }
+    }
     if (!sp.live || !sp.small_rows) return 0;
     toks = sp.q_len;
     return (sp.hi - sp.lo + 63) & ~63;
@@ -532,6 +547,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     plan[0] = W;
     plan[1] = q;
     plan[2] = s_large;  // any sequence for the large-row (prefill) kernel?
+    plan[3] = s_merge;  // anything for the merge kernel?
     s_Q = q;
   }
   __threadfence_block();

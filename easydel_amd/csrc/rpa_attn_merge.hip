@@ -18,6 +18,9 @@ __global__ __launch_bounds__(256, 8) void attn_merge_kernel(AttnParams p) {
   const int lane = threadIdx.x & 63;
   const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);  // (token, head) index
   if (pair >= p.T * p.Hq) return;
+  // the plan kernel has seen the whole batch: no padded token, no partial row -- nothing to do (a batch of prompts
+  // whose row tiles are not cut would otherwise pay a look-up per row for nothing)
+  if (p.mfma_path && p.plan[3] == 0) return;
   const int t = pair / p.Hq, hq = pair - t * p.Hq;
   const int n_live = live_rows(p);
   const int D = p.D;
