@@ -716,6 +716,88 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(MlaParams p) {
   }
 }
 
+// The same for two neighbouring heads of a token per wave on the matrix-core path (latent 512, an even head count):
+// their partial rows are neighbours in memory, and what bounds a row's merge is its chain of dependent loads (sequence
+// look-up, lengths, (max, sum) pairs, partial rows), which here serves two rows.
+__global__ __launch_bounds__(256, 4) void mla_merge_pair_kernel(MlaParams p) {
+  constexpr int LKV = 512, HPW = 2, NK = LKV / 64, NKT = NK * HPW;
+  const int lane = threadIdx.x & 63;
+  const int groups = p.Hq / HPW;
+  const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= p.T * groups) return;
+  const int t = pair / groups, hq0 = (pair - t * groups) * HPW;
+  const int n_live = mla_live_rows(p);
+  bool zero = false;
+  int n_p[HPW] = {0, 0};
+  if (n_live <= 0 || t < p.qsl[0] || t >= p.qsl[n_live]) {
+    zero = true;
+  } else {
+    const int i = find_seq_wave(p.qsl, n_live, t);
+    const MlaSeq sp = mla_seq(p, i);
+    if (!sp.live) zero = true;
+    else if (p.max_chunks > 1) {
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh) {  // the two heads can lie in different row tiles
+        const int row = (t - sp.q0) * p.Hq + hq0 + hh;
+        const int n = mla_tile(p, sp, (row / kMlaRows) * kMlaRows).n_chunks;
+        n_p[hh] = n > 1 ? n : 0;  // a row in one piece was written by the kernel that computed it
+      }
+    }
+  }
+  const int n_max = max(n_p[0], n_p[1]);
+  if (!zero && n_max == 0) return;
+  float acc[NKT];
+#pragma unroll
+  for (int k = 0; k < NKT; ++k) acc[k] = 0.f;
+  float inv[HPW] = {0.f, 0.f};
+  if (n_max > 0) {
+    const int64_t slot0 = (int64_t)t * p.Hq + hq0;
+    const int64_t stride = (int64_t)p.T * p.Hq;
+    float m_use[HPW], l[HPW], w_c[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {  // n_pieces <= kMlaMaxChunks: lane c holds piece c
+      float2 ml = {-INFINITY, 0.f};
+      if (lane < n_p[hh]) ml = *(const float2*)(p.part_ml + (slot0 + hh + lane * stride) * 2);
+      float m = ml.x;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+      m_use[hh] = (m == -INFINITY) ? 0.f : m;
+      w_c[hh] = lane < n_p[hh] ? __builtin_amdgcn_exp2f(ml.x - m_use[hh]) : 0.f;
+      float lt = w_c[hh] * ml.y;
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) lt += __shfl_xor(lt, o);
+      l[hh] = lt;
+    }
+    for (int c = 0; c < n_max; c += 2) {  // two pieces (32 floats per lane) in flight
+      float v[2][NKT];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const float* row = p.part_o + (slot0 + (int64_t)(c + u) * stride) * LKV;
+#pragma unroll
+        for (int k = 0; k < NKT; ++k) v[u][k] = (c + u < n_p[k / NK]) ? row[lane + 64 * k] : 0.f;  // never a piece nobody wrote
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const float w0 = __shfl(w_c[0], c + u), w1 = __shfl(w_c[1], c + u);  // zero past a head's pieces
+#pragma unroll
+        for (int k = 0; k < NKT; ++k) acc[k] = fmaf(k < NK ? w0 : w1, v[u][k], acc[k]);
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      float lt = l[hh];
+      if (p.sinks != nullptr && lt > 0.f) lt += __builtin_amdgcn_exp2f(__builtin_fmaf(p.sinks[hq0 + hh], 1.4426950408889634f, -m_use[hh]));
+      inv[hh] = lt > 0.f ? 1.f / lt : 0.f;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NKT; ++k) {
+    if (!zero && n_p[k / NK] == 0) continue;
+    const int64_t o = ((int64_t)t * p.Hq + hq0) * LKV + lane + 64 * k;
+    ((uint16_t*)p.out)[o] = float_to_bf16_bits(acc[k] * inv[k / NK]);
+  }
+}
+
 template <int QT>
 int launch_generic_q(hipStream_t stream, const MlaParams& p) {
   dim3 grid(p.T, p.Hq), block(64);
@@ -772,6 +854,11 @@ int launch_mla_mfma(hipStream_t stream, const MlaParams& p) {
 
 int launch_mla_merge(hipStream_t stream, const MlaParams& p) {
   if (p.lkv > kGenMaxLkv) return (int)hipErrorInvalidValue;
+  if (p.mfma && p.q_dtype == RPA_BF16 && p.lkv == 512 && p.Hq % 2 == 0) {
+    const int pairs = (int)(((int64_t)p.T * (p.Hq / 2) + 3) / 4);
+    hipLaunchKernelGGL(mla_merge_pair_kernel, dim3(pairs), dim3(256), 0, stream, p);
+    return (int)hipGetLastError();
+  }
   const int blocks = (int)(((int64_t)p.T * p.Hq + 3) / 4);
   if (p.q_dtype == RPA_F32) hipLaunchKernelGGL((mla_merge_kernel<RPA_F32>), dim3(blocks), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((mla_merge_kernel<RPA_BF16>), dim3(blocks), dim3(256), 0, stream, p);
