@@ -92,7 +92,10 @@ void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, i
   if (g_prefill_chunks.load() <= 0 && Hkv > 0) {
     const long row_tiles = ((long)T * (Hq / Hkv) / rpa::kPrefillRows + S) * Hkv;  // the prefill grid's bound without cutting
     const int cus = device_cus();
-    if (cus > 0 && row_tiles >= 8L * cus) chunks = 1;
+    if (cus > 0) {  // about eight units per CU fill the chip evenly; more chunks than that only add partials
+      const long want = (8L * cus + row_tiles - 1) / row_tiles;
+      if (want < chunks) chunks = (int)(want < 1 ? 1 : want);
+    }
   }
   const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
