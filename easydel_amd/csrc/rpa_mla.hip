@@ -154,6 +154,29 @@ __global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
   }
 }
 
+// What row-tile slot `slot` of the matrix-core kernel's grid holds: (sequence, key chunks | keys / 64 of a chunk << 8),
+// chunks = 0 where there is no tile.
+// `qsl` is query_start_loc, or a copy of its first n_live + 1 entries that is quicker to search.
+__device__ __forceinline__ int2 mla_plan_slot(const MlaParams& p, int slot, const int32_t* qsl) {
+  int2 unit = {0, 0};
+  const int n_live = mla_live_rows(p);
+  if (n_live > 0) {
+    int lo_i = 0, hi_i = n_live;  // the last sequence starting at or before `slot`
+    while (hi_i - lo_i > 1) {
+      const int mid = (lo_i + hi_i) >> 1;
+      if ((int)(((int64_t)qsl[mid] * p.Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
+    }
+    const MlaSeq sp = mla_seq(p, lo_i);
+    const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * p.Hq) / kMlaRows) + lo_i);
+    if (sp.live && tile_in_seq >= 0 && tile_in_seq * kMlaRows < sp.q_len * p.Hq) {
+      const MlaTile mt = mla_tile(p, sp, tile_in_seq * kMlaRows);
+      unit.x = lo_i;
+      unit.y = mt.n_chunks | ((min(mt.chunk, mt.kv_hi - mt.kv_lo) >> 6) << 8);  // chunks, and keys / 64 of one chunk
+    }
+  }
+  return unit;
+}
+
 // ---- plan: which sequence and how many key chunks each row-tile slot of the MFMA kernel's grid holds -------------
 // Sequence i starts at slot floor(qsl[i] * Hq / 128) + i (its row tiles follow), so the slots of a batch are found
 // without a scan; slots between sequences, past the live ones, or of rows before position 0 hold no tile.
@@ -168,87 +191,144 @@ __global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots,
   }
   const int slot = blockIdx.x * 256 + threadIdx.x;
   if (slot >= n_slots) return;
-  int2 unit = {0, 0};
-  const int n_live = mla_live_rows(p);
-  if (n_live > 0) {
-    int lo_i = 0, hi_i = n_live;  // the last sequence starting at or before `slot`
-    while (hi_i - lo_i > 1) {
-      const int mid = (lo_i + hi_i) >> 1;
-      if ((int)(((int64_t)p.qsl[mid] * p.Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
-    }
-    const MlaSeq sp = mla_seq(p, lo_i);
-    const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * p.Hq) / kMlaRows) + lo_i);
-    if (sp.live && tile_in_seq >= 0 && tile_in_seq * kMlaRows < sp.q_len * p.Hq) {
-      const MlaTile mt = mla_tile(p, sp, tile_in_seq * kMlaRows);
-      unit.x = lo_i;
-      unit.y = mt.n_chunks | ((min(mt.chunk, mt.kv_hi - mt.kv_lo) >> 6) << 8);  // chunks, and keys / 64 of one chunk
-    }
-  }
-  p.plan[slot] = unit;
+  p.plan[slot] = mla_plan_slot(p, slot, p.qsl);
 }
+
+// Small batches (up to kMlaSortSlots slots): plan and unit list in one launch of one block -- thread t looks up slots
+// 4t .. 4t+3, keeps them in registers, and the list is built longest first in eight classes of chunk length with one
+// scan over eight counters instead of one scan per class.  Blocks behind the first write the new rows, as above.
+constexpr int kMlaSortSlots = 4096;
+constexpr int kMlaLenClasses = 8;
+__global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int n_slots) {
+  constexpr int PER = kMlaSortSlots / 1024, NC = kMlaLenClasses;
+  if (blockIdx.x > 0) {
+    const int t = ((int)blockIdx.x - 1) * 16 + (threadIdx.x >> 6);
+    if (p.kv_dtype == RPA_F32) mla_scatter_token<uint32_t>(p, t);
+    else mla_scatter_token<uint16_t>(p, t);
+    return;
+  }
+  __shared__ int wave_max_s[16];
+  __shared__ int wave_cnt[16][NC];
+  __shared__ int32_t qsl_s[kMlaSortSlots + 1];  // the sequence starts, searched four times per thread: from LDS, not through
+                                                // a dozen dependent global loads (n_live <= S <= n_slots <= kMlaSortSlots)
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  for (int k = tid; k <= min(mla_live_rows(p), kMlaSortSlots); k += 1024) qsl_s[k] = p.qsl[k];
+  __syncthreads();
+  int y[PER];
+  int max_len = 0;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int slot = tid * PER + k;
+    int2 unit = {0, 0};
+    if (slot < n_slots) {
+      unit = mla_plan_slot(p, slot, qsl_s);
+      p.plan[slot] = unit;
+    }
+    y[k] = unit.y;
+    if (y[k] & 0xff) max_len = max(max_len, y[k] >> 8);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) max_len = max(max_len, __shfl_xor(max_len, o));
+  if (lane == 0) wave_max_s[wv] = max_len;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < 16; ++w) max_len = max(max_len, wave_max_s[w]);
+  // units of this thread's slots per class, then an inclusive scan over the threads for all classes at once
+  int cls[PER], cnt[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) cnt[c] = 0;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    cls[k] = min(NC - 1, ((y[k] >> 8) * NC) / (max_len + 1));
+#pragma unroll
+    for (int c = 0; c < NC; ++c) cnt[c] += (cls[k] == c) ? (y[k] & 0xff) : 0;
+  }
+  int incl[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    incl[c] = cnt[c];
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl[c], o);
+      if (lane >= o) incl[c] += up;
+    }
+    if (lane == 63) wave_cnt[wv][c] = incl[c];
+  }
+  __syncthreads();
+  // first list position of each class's units of this thread: the longer classes in full, then the class's units of
+  // the waves and lanes before
+  int first[NC];
+  int longer = 0, total = 0;
+#pragma unroll
+  for (int c = NC - 1; c >= 0; --c) {
+    int before = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      const int v = wave_cnt[w][c];
+      before += (w < wv) ? v : 0;
+      all += v;
+    }
+    first[c] = longer + before + incl[c] - cnt[c];
+    longer += all;
+  }
+  total = longer;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int v = y[k] & 0xff;
+    if (v == 0) continue;
+    int at = 0;
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+      if (cls[k] == c) {
+        at = first[c];
+        first[c] += v;
+      }
+    for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(tid * PER + k, ch);
+  }
+  if (tid == 0) {
+    p.n_units[0] = total;
+    p.n_units[1] = 1;
+  }
+}
+
+
 
 // The units (row tile, key chunk) of the batch in one dense list.  The MFMA kernel's grid is sized from the static
 // bounds and most of its slots are empty; left in place, the empty ones form a regular pattern (a batch of single tokens
 // with 128 heads fills every other slot) that the hardware's round-robin placement of consecutive blocks turns into
 // idle shader engines: measured, each engine was busy 43 % of such a kernel's duration.
-// One block: a scan over the plan's chunk counts, 1024 slots a pass.  A batch of up to kMlaSortSlots slots (decode
-// and small mixed batches, where a unit is a sizeable share of a CU's work and the lengths differ many-fold) is listed
-// longest first, in eight classes of chunk length, one scan per class: workgroups are handed out in list order, so
-// the long units start first and the short ones fill in behind them.  Larger batches are listed in slot order in
-// one scan; n_units[1] says which.
-constexpr int kMlaSortSlots = 4096;
-constexpr int kMlaLenClasses = 8;
-
+// A batch of up to kMlaSortSlots slots (decode and small mixed batches, where a unit is a sizeable share of a CU's work
+// and the lengths differ many-fold) is listed longest first by mla_plan_sorted_kernel: workgroups are handed out in
+// list order, so the long units start first and the short ones fill in behind them.  Larger batches are listed here,
+// in slot order: one block, a scan over the plan's chunk counts, 1024 slots a pass.  n_units[1] says which.
 __global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_slots) {
   __shared__ int wave_tot[16];
   __shared__ int running_s;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const bool sort = n_slots <= kMlaSortSlots;
-  int max_len = 0;
-  if (sort) {
-    for (int slot = tid; slot < n_slots; slot += 1024) {
-      const int y = p.plan[slot].y;
-      if (y & 0xff) max_len = max(max_len, y >> 8);
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) max_len = max(max_len, __shfl_xor(max_len, o));
-    if (lane == 0) wave_tot[wv] = max_len;
-    __syncthreads();
-    for (int w = 0; w < 16; ++w) max_len = max(max_len, wave_tot[w]);
-  }
-  __syncthreads();
   if (tid == 0) running_s = 0;
   __syncthreads();
-  const int classes = sort ? kMlaLenClasses : 1;
-  for (int cls = classes - 1; cls >= 0; --cls) {
-    for (int base = 0; base < n_slots; base += 1024) {
-      const int slot = base + tid;
-      int v = 0;
-      if (slot < n_slots) {
-        const int y = p.plan[slot].y;
-        const int mine = sort ? min(kMlaLenClasses - 1, ((y >> 8) * kMlaLenClasses) / (max_len + 1)) : 0;
-        if (mine == cls) v = y & 0xff;
-      }
-      int incl = v;
+  for (int base = 0; base < n_slots; base += 1024) {
+    const int slot = base + tid;
+    const int v = slot < n_slots ? (p.plan[slot].y & 0xff) : 0;
+    int incl = v;
 #pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(incl, o);
-        if (lane >= o) incl += up;
-      }
-      if (lane == 63) wave_tot[wv] = incl;
-      __syncthreads();
-      int before = running_s;
-      for (int w = 0; w < wv; ++w) before += wave_tot[w];
-      const int first = before + incl - v;
-      for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c);
-      __syncthreads();
-      if (tid == 1023) running_s = before + incl;
-      __syncthreads();
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o);
+      if (lane >= o) incl += up;
     }
+    if (lane == 63) wave_tot[wv] = incl;
+    __syncthreads();
+    int before = running_s;
+    for (int w = 0; w < wv; ++w) before += wave_tot[w];
+    const int first = before + incl - v;
+    for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c);
+    __syncthreads();
+    if (tid == 1023) running_s = before + incl;
+    __syncthreads();
   }
   if (tid == 0) {
     p.n_units[0] = running_s;
-    p.n_units[1] = sort ? 1 : 0;
+    p.n_units[1] = 0;
   }
 }
 
@@ -843,10 +923,15 @@ int launch_mla_mfma(hipStream_t stream, const MlaParams& p) {
   const int64_t slots = mla_plan_slots(p.T, p.S, p.Hq);
   const int64_t blocks = (slots * p.max_chunks + kXcds - 1) / kXcds * kXcds;  // most units the batch can have
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
-  const int plan_blocks = (int)((slots + 255) / 256);
-  const int write_blocks = p.new_kv ? (p.T + 3) / 4 : 0;  // the page write rides along (see mla_plan_kernel)
-  hipLaunchKernelGGL(mla_plan_kernel, dim3((unsigned)(plan_blocks + write_blocks)), dim3(256), 0, stream, p, (int)slots, plan_blocks);
-  hipLaunchKernelGGL(mla_compact_kernel, dim3(1), dim3(1024), 0, stream, p, (int)slots);
+  if (slots <= kMlaSortSlots) {  // plan, sorted unit list and the page write in one launch
+    const int write_blocks = p.new_kv ? (p.T + 15) / 16 : 0;
+    hipLaunchKernelGGL(mla_plan_sorted_kernel, dim3((unsigned)(1 + write_blocks)), dim3(1024), 0, stream, p, (int)slots);
+  } else {
+    const int plan_blocks = (int)((slots + 255) / 256);
+    const int write_blocks = p.new_kv ? (p.T + 3) / 4 : 0;  // the page write rides along (see mla_plan_kernel)
+    hipLaunchKernelGGL(mla_plan_kernel, dim3((unsigned)(plan_blocks + write_blocks)), dim3(256), 0, stream, p, (int)slots, plan_blocks);
+    hipLaunchKernelGGL(mla_compact_kernel, dim3(1), dim3(1024), 0, stream, p, (int)slots);
+  }
   if (p.softcap > 0.f) hipLaunchKernelGGL((mla_attn_kernel<true>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
   else hipLaunchKernelGGL((mla_attn_kernel<false>), dim3((unsigned)blocks), dim3(64 * kMlaWaves), 0, stream, p);
   return (int)hipGetLastError();
