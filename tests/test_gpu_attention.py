@@ -319,6 +319,18 @@ def test_many_short_sequences(gpu):
     _check(b, "1500 short sequences")
 
 
+def test_more_sequences_than_one_look_up_round_covers(gpu):
+    # 6 000 rows: the wave-wide sequence look-up needs a third round (64 * 64 < 6 000), the plan kernel's threads hold
+    # several sequences each, and a few multi-token rows sit among the single tokens
+    rng = np.random.default_rng(73)
+    ctx = rng.integers(1, 60, size=6000)
+    q = np.ones(6000, dtype=np.int64)
+    for i in rng.choice(6000, size=40, replace=False):
+        q[i] = int(rng.integers(1, min(int(ctx[i]), 9) + 1))
+    b = tl.make_batch(73, ctx.tolist(), q.tolist(), Hq=8, Hkv=2, D=64, page_size=16, pad_rows=100, pad_tokens=7)
+    _check(b, "6000 sequences")
+
+
 def test_hip_graph_replay_matches_eager(gpu):
     # the C ABI neither allocates nor synchronises, so a whole layer call can be captured and replayed
     import torch
