@@ -68,9 +68,14 @@ import numpy as np
 def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
     """Round float32 to bfloat16 (round-to-nearest-even), returned as uint16 bit patterns."""
     u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
-    nan = (u & 0x7FFFFFFF) > 0x7F800000
-    rounded = (u + (0x7FFF + ((u >> 16) & 1))) >> 16
-    rounded = np.where(nan, (u >> 16) | 0x0040, rounded)
+    rounded = u >> np.uint32(16)  # (u + 0x7FFF + lsb of the kept half) >> 16, in place: the test pools are 10^8 elements
+    rounded &= np.uint32(1)
+    rounded += np.uint32(0x7FFF)
+    rounded += u
+    rounded >>= np.uint32(16)
+    nan = (u & np.uint32(0x7FFFFFFF)) > np.uint32(0x7F800000)
+    if nan.any():
+        rounded[nan] = (u[nan] >> np.uint32(16)) | np.uint32(0x0040)
     return rounded.astype(np.uint16)
 
 

@@ -234,7 +234,9 @@ class MlaBatch:
 
 
 def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64, dtype=BF16, pad_rows=0, pad_tokens=0,
-                   row=None, max_pages=None):
+                   row=None, max_pages=None, distinct_pages=0):
+    """`distinct_pages` > 0: the pool repeats that many random pages (thousands of sequences need thousands of pages,
+    and drawing every one takes minutes on a slow host)."""
     rng = np.random.default_rng(seed)
     ctx_lens = np.asarray(ctx_lens, np.int32)
     q_lens = np.asarray(q_lens, np.int32)
@@ -272,11 +274,17 @@ def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64
         x = x.astype(np.float32)
         return x, x.astype(np.float64)
 
-    b.qn_raw, b.qn_val = enc(rng.standard_normal((b.T, Hq, lkv)))
-    b.qp_raw, b.qp_val = enc(rng.standard_normal((b.T, Hq, rope)))
-    b.kv_raw, b.kv_val = enc(rng.standard_normal((b.T, lkv)))
-    b.pe_raw, b.pe_val = enc(rng.standard_normal((b.T, rope)))
-    b.pages_raw, b.pages_val = enc(rng.standard_normal((b.P, page_size, b.row)))  # padding holds noise: never read
+    normal = lambda *shape: rng.standard_normal(shape, dtype=np.float32)
+    b.qn_raw, b.qn_val = enc(normal(b.T, Hq, lkv))
+    b.qp_raw, b.qp_val = enc(normal(b.T, Hq, rope))
+    b.kv_raw, b.kv_val = enc(normal(b.T, lkv))
+    b.pe_raw, b.pe_val = enc(normal(b.T, rope))
+    if distinct_pages and distinct_pages < b.P:
+        raw, val = enc(normal(distinct_pages, page_size, b.row))
+        pick = np.arange(b.P) % distinct_pages
+        b.pages_raw, b.pages_val = raw[pick], val[pick]
+    else:
+        b.pages_raw, b.pages_val = enc(normal(b.P, page_size, b.row))  # padding holds noise: never read
     return b
 
 

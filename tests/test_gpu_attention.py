@@ -331,6 +331,18 @@ def test_more_sequences_than_one_look_up_round_covers(gpu):
     _check(b, "6000 sequences")
 
 
+def test_many_prompts_in_one_call(gpu):
+    # 400 whole prompts and chunks of 17..150 tokens: row tiles of the large-row kernel found by slot among hundreds of
+    # sequences, most tiles partly filled, single tokens in between
+    rng = np.random.default_rng(74)
+    q = rng.integers(17, 151, size=400)
+    q[rng.choice(400, size=60, replace=False)] = 1
+    ctx = q + rng.integers(0, 200, size=400) * (rng.random(400) < 0.5)
+    b = tl.make_batch(74, ctx.tolist(), q.tolist(), Hq=8, Hkv=2, D=64, page_size=16, pad_rows=5, pad_tokens=3)
+    _check(b, "400 prompts")
+    _check(b, "400 prompts, window 50", sliding_window=50)
+
+
 def test_hip_graph_replay_matches_eager(gpu):
     # the C ABI neither allocates nor synchronises, so a whole layer call can be captured and replayed
     import torch

@@ -46,6 +46,16 @@ def test_decode_batches_on_the_matrix_cores(Hq):
     check(b, f"decode Hq={Hq}", softmax_scale=SCALE)
 
 
+def test_more_row_tile_slots_than_the_sorted_unit_list_holds():
+    # 3 900 single tokens at 8 heads: 4 143 row-tile slots, so a decode batch takes the plan and unit list of large batches
+    # (two launches, slot order) instead of the one-block sorted list
+    rng = np.random.default_rng(7)
+    ctx = rng.integers(1, 33, size=3900).tolist()
+    b = make_mla_batch(8, ctx, [1] * len(ctx), Hq=8, page_size=32, pad_rows=10, pad_tokens=2, distinct_pages=97)
+    assert b.T * b.Hq // 128 + b.S > 4096
+    check(b, "3900 sequences", softmax_scale=SCALE)
+
+
 def test_chunked_prefill_and_mixed_rows():
     b = make_mla_batch(4, [200, 97, 400, 31, 1000], [1, 97, 150, 31, 3], Hq=16)
     check(b, "mixed", softmax_scale=SCALE)
