@@ -50,6 +50,9 @@ def parse_args():
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
     ap.add_argument("--sequential-pages", action="store_true", help="experiment: block tables in pool order")
+    ap.add_argument("--read-probe", action="store_true",
+                    help="instead of a workload: time the library's read-only probe over 8 GiB for 32..256 workgroups and "
+                         "16..256 KiB in flight per workgroup, one line per setting")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so a counter run shows what a known-size kernel reads")
     return ap.parse_args()
@@ -226,6 +229,36 @@ def bench_mla(args):
     }))
 
 
+def read_probe():
+    """What the memory system gives a streaming reader: rpa_read_probe over 8 GiB, best of four timed launches."""
+    import torch
+
+    from easydel_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    buf = torch.empty(8 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    for wgs in (32, 64, 128, 192, 256):
+        for kib in (2, 4, 8, 16, 32):
+            best, read = None, 0
+            for rep in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                read = lib.rpa_read_probe(stream.cuda_stream, buf.data_ptr(), buf.numel(), wgs, kib, sink.data_ptr())
+                e1.record(stream)
+                e1.synchronize()
+                if read == 0:
+                    raise RuntimeError(lib.rpa_last_error().decode())
+                ms = e0.elapsed_time(e1)
+                if rep > 0 and (best is None or ms < best):
+                    best = ms
+            print(json.dumps({"probe": "read", "workgroups": wgs, "kib_in_flight_per_workgroup": 8 * kib, "ms": round(best, 4),
+                              "tb_per_s": round(read / best / 1e9, 3), "gb_per_s_per_workgroup": round(read / best / 1e6 / wgs, 1)}),
+                  flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -239,6 +272,8 @@ def main():
     from easydel_amd import _lib, kernels, workloads
 
     _lib.load()
+    if args.read_probe:
+        return read_probe()
     if args.workload.startswith("mla-"):
         if args.mla_chunks:
             _lib.set_tunable("mla_chunks", args.mla_chunks)

@@ -14,6 +14,7 @@ int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_
 int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int);
 int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
+size_t launch_read_probe(hipStream_t, const void*, size_t, int, int, uint32_t*);
 int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
                                 const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int);
 }  // namespace rpa
@@ -173,6 +174,18 @@ int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_calibration_copy: pointers and size must be 16-byte aligned");
   if (bytes == 0) return RPA_OK;
   return hip_fail(rpa::launch_calibration_copy((hipStream_t)stream, dst, src, bytes), "rpa_calibration_copy launch");
+}
+
+size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
+                      void* sink) {
+  if (!src || !sink || ((uintptr_t)src & 15) || ((uintptr_t)sink & 3)) {
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_read_probe: src must be 16-byte aligned and sink a 4-byte device word");
+    return 0;
+  }
+  const size_t read = rpa::launch_read_probe((hipStream_t)stream, src, bytes, workgroups, kib_in_flight_per_wave, (uint32_t*)sink);
+  if (read == 0)
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_read_probe: workgroups > 0, 2 / 4 / 8 / 16 / 32 KiB in flight per wave, and at least one round of loads per wave");
+  return read;
 }
 
 int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32_t* slice_indices,

@@ -221,6 +221,45 @@ int launch_calibration_copy(hipStream_t stream, void* dst, const void* src, size
   return (int)hipGetLastError();
 }
 
+// Read-only probe of the memory system: `workgroups` workgroups of eight waves (96 KiB of LDS each, so one per CU), every
+// wave streaming its own contiguous share of the buffer with 16-byte loads, DEPTH instructions (KiB) in flight.
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+template <int DEPTH>
+__global__ __launch_bounds__(512) void read_probe_kernel(const probe_u32x4* __restrict__ src, size_t kib_per_wave, uint32_t* __restrict__ sink) {
+  __shared__ char occupy[98304];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const probe_u32x4* p = src + ((size_t)blockIdx.x * 8 + wave) * kib_per_wave * 64 + lane;
+  probe_u32x4 acc = {0u, 0u, 0u, 0u};
+  for (size_t c = 0; c + DEPTH <= kib_per_wave; c += DEPTH) {
+    probe_u32x4 v[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) v[d] = __builtin_nontemporal_load(p + (c + d) * 64);
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) acc ^= v[d];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) sink[0] = occupy[lane];  // keeps the loads and the LDS alive
+}
+
+// Returns the bytes the launch reads (0: bad arguments): bytes / (8 workgroups) rounded down to whole rounds of loads.
+size_t launch_read_probe(hipStream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
+                         uint32_t* sink) {
+  if (workgroups <= 0) return 0;
+  size_t per = bytes / ((size_t)workgroups * 8) / 1024;
+  per -= per % (size_t)(kib_in_flight_per_wave > 0 ? kib_in_flight_per_wave : 1);
+  if (per == 0) return 0;
+#define RPA_PROBE(D) hipLaunchKernelGGL(read_probe_kernel<D>, dim3(workgroups), dim3(512), 0, stream, (const probe_u32x4*)src, per, sink)
+  switch (kib_in_flight_per_wave) {
+    case 2: RPA_PROBE(2); break;
+    case 4: RPA_PROBE(4); break;
+    case 8: RPA_PROBE(8); break;
+    case 16: RPA_PROBE(16); break;
+    case 32: RPA_PROBE(32); break;
+    default: return 0;
+  }
+#undef RPA_PROBE
+  return hipGetLastError() == hipSuccess ? per * 1024 * 8 * (size_t)workgroups : 0;
+}
+
 int launch_scatter_slices(hipStream_t stream, const void* new_kv, const int32_t* si, const int32_t* num_slices,
                           void* pages, int T, int N, int64_t num_positions, int page_size, int64_t row_bytes,
                           int shard) {

@@ -253,6 +253,17 @@ int rpa_mla_page_scatter(rpa_stream_t stream, const void* keys_values, const voi
 int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t bytes);
 
 /*
+ * Measurement aid with no counterpart in the reference: a read-only kernel that says what the memory system gives
+ * a streaming reader.  `workgroups` workgroups of eight wavefronts (one per CU: each holds 96 KiB of LDS) read `src`
+ * once, every wavefront its own contiguous share with 16-byte loads, `kib_in_flight_per_wave` (2, 4, 8, 16 or 32) KiB
+ * of them in flight.  Returns the bytes the launch reads (the share of each wavefront is rounded down to whole rounds
+ * of loads), 0 on bad arguments; time the launch with events on `stream`.  `sink` is one device word, never written in
+ * practice.  The decode kernel's bandwidth is judged against this probe's at the same number of workgroups.
+ */
+size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
+                      void* sink);
+
+/*
  * Tuning knobs (process-wide, read at call time).  Returns the previous value.
  *   "max_splits"     partial-output slots per sequence the decode kernel may use (2..256, 0 = sized
  *                    from the shapes); set it before sizing the workspace

@@ -58,6 +58,11 @@ def test_host_only_entry_points():
     assert lib.rpa_page_scatter_slices(None, None, None, None, None, 4, 4, 64, 0, 16, 0) == _lib.RPA_ERR_INVALID_ARGUMENT
     n = lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1)
     assert n > 2 * 256 * 32 * 130 * 4
+    # the read probe reads nothing and launches nothing on bad arguments
+    assert lib.rpa_read_probe(None, None, 1 << 30, 256, 8, None) == 0 and b"rpa_read_probe" in lib.rpa_last_error()
+    assert lib.rpa_read_probe(None, a, 1 << 30, 256, 3, a) == 0  # 2 / 4 / 8 / 16 / 32 KiB in flight per wave
+    assert lib.rpa_read_probe(None, a, 1 << 30, 0, 8, a) == 0
+    assert lib.rpa_read_probe(None, a, 4096, 256, 8, a) == 0  # less than one round of loads per wave
     prev = _lib.set_tunable("max_splits", 4)
     assert lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1) < n
     _lib.set_tunable("max_splits", prev)
