@@ -84,8 +84,9 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   constexpr int VB = DPL * EB;         // bytes of V one lane reads per token
   constexpr int NKK = D / 32;          // k-steps of the score MFMA
   // Tiles in flight per wave (register staging buffers).  Two were measured slower than one on MI355X (780 vs
-  // 766 us on the Llama-shaped decode batch): eight waves with one 8 KiB tile each already saturate a CU's
-  // memory pipe, and the extra registers and code only delay the next issue.
+  // 766 us on the Llama-shaped decode batch) -- but as compiled, the DEPTH = 2 build never has two tiles in flight:
+  // the compiler's waits before a tile's registers are first used (s_waitcnt vmcnt(n), n <= 6 throughout) also
+  // drain the newer tile's loads.  A build that means it has to issue these loads and their waits itself.
   constexpr int DEPTH = 1;
   static_assert(LPT <= 64 && TT % TPI == 0 && TT % 16 == 0, "tile shape");
 
