@@ -74,15 +74,41 @@ def build_workload(name, seed, sequential=False):
     return workloads.config5_gemma_long_prefill(seed, windowed=(name == "c5-window"))
 
 
+KERNEL_SOURCES = {  # the files a kernel is compiled from: a counter run is only valid for the sources it was taken on
+    "attn_decode_kernel": ("rpa_attn_decode.hip", "rpa_mfma.h", "rpa_common.h"),
+    "attn_prefill_kernel": ("rpa_attn_prefill_dma.hip", "rpa_attn_prefill.hip", "rpa_mfma.h", "rpa_common.h"),
+}
+
+
+def kernel_source_sha16(kernel):
+    """First 16 hex digits of the SHA-256 over the source files of a kernel (KERNEL_SOURCES), in order."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES[kernel]:
+        with open(os.path.join(ROOT, "easydel_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(workload, kernel="attn_decode_kernel"):
-    """HBM bytes per launch of a kernel from the committed counter runs (FETCH_SIZE and WRITE_SIZE passes, each
-    scaled by what the same counter reads for a 1 GiB copy); None for workloads without such a run."""
-    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload.replace('-', '_')}_traffic.json")
+    """``(bytes, source)``: HBM bytes per launch of a kernel from a committed counter run (FETCH_SIZE and WRITE_SIZE
+    passes of rocprofv3, each scaled by what the same counter reads for a 1 GiB copy), and where the figure comes
+    from.  It is not measured in this run, so it only counts while the kernel is what it was when the counters were
+    read: the file records the hash of the kernel's sources, and with any other hash (or none) the bytes are None."""
+    name = f"{kernel}_{workload.replace('-', '_')}_traffic.json"
+    source = {"file": f"profiles/{name}", "measured_in_this_run": False}
     try:
-        with open(path) as f:
-            return float(json.load(f)["hbm_bytes_per_launch"])
+        with open(os.path.join(ROOT, "profiles", name)) as f:
+            rec = json.load(f)
+        nbytes = float(rec["hbm_bytes_per_launch"])
     except (OSError, KeyError, ValueError):
-        return None
+        return None, None
+    source["git_head"] = rec.get("git_head")
+    source["kernel_source_sha16"] = rec.get("kernel_source_sha16")
+    source["current_kernel_source_sha16"] = kernel_source_sha16(kernel)
+    source["stale"] = source["kernel_source_sha16"] != source["current_kernel_source_sha16"]
+    return (None if source["stale"] else nbytes), source
 
 
 def cpu_baseline(w, tens, sample_seqs):
@@ -386,17 +412,21 @@ def main():
         nbytes = w.attention_bytes(small)
         kern["attn_decode_kernel"] = {
             "bound": "hbm", "achieved": nbytes / (ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None if unified else measured_traffic(args.workload),
+            "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "traffic_source": None,
             "algorithmic_bytes_per_launch": nbytes, "kernel_ms": ms}
+        if not unified:
+            kern["attn_decode_kernel"]["traffic"], kern["attn_decode_kernel"]["traffic_source"] = measured_traffic(args.workload)
     if (~small & (w.q_lens > 0)).any():
         ms = time_stage(4, args.steps)
         flops = w.attention_flops(~small)
         kern["attn_prefill_kernel"] = {
             "bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-            "traffic": None if unified else measured_traffic(args.workload, "attn_prefill_kernel"),
+            "frac": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None, "traffic_source": None,
             "algorithmic_flops_per_launch": flops, "algorithmic_bytes_per_launch": w.attention_bytes(~small),
             "kernel_ms": ms}
+        if not unified:
+            kern["attn_prefill_kernel"]["traffic"], kern["attn_prefill_kernel"]["traffic_source"] = \
+                measured_traffic(args.workload, "attn_prefill_kernel")
     _lib.set_tunable("stages", prev)
     dominant = max(kern, key=lambda k: kern[k]["kernel_ms"])
     roofline = dict(kern[dominant], kernel=dominant)

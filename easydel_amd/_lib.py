@@ -1,4 +1,4 @@
-"""ctypes binding of librpa_hip.so (the C ABI declared in include/rpa_hip.h).
+"""ctypes binding of librpa_hip.so (the C ABI declared in include/rpa_hip.h and include/rpa_hip_probe.h).
 
 There is no fallback: if the library is missing or fails to load, every call raises.
 """
@@ -12,12 +12,12 @@ from pathlib import Path
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "librpa_hip.so"
 
 # rpa_dtype tags
-RPA_F32, RPA_BF16, RPA_FP8_E4M3, RPA_INT8 = 0, 1, 2, 3
+RPA_F32, RPA_BF16, RPA_FP8_E4M3, RPA_INT8, RPA_F16 = 0, 1, 2, 3, 4
 RPA_ERR_INVALID_ARGUMENT, RPA_ERR_UNSUPPORTED, RPA_ERR_WORKSPACE = -1, -2, -3
 
 _c_int, _c_i64, _c_f32, _c_vp, _c_sz = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t
 
-# name -> (restype, argtypes); mirrors include/rpa_hip.h declaration by declaration.
+# name -> (restype, argtypes); mirrors the two headers declaration by declaration.
 SIGNATURES = {
     "rpa_version": (ctypes.c_char_p, []),
     "rpa_last_error": (ctypes.c_char_p, []),
@@ -25,16 +25,16 @@ SIGNATURES = {
     "rpa_calibration_copy": (_c_int, [_c_vp, _c_vp, _c_vp, _c_sz]),
     "rpa_read_probe": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_vp]),
     "rpa_page_scatter_slices": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_i64, _c_int, _c_i64, _c_int]),
-    "rpa_page_scatter_ragged": (_c_int, [_c_vp] * 8 + [_c_int] * 9),
+    "rpa_page_scatter_ragged": (_c_int, [_c_vp] * 8 + [_c_int] * 10),
     "rpa_attention_workspace_bytes": (_c_sz, [_c_int] * 9),
     "rpa_ragged_paged_attention": (
         _c_int,
-        [_c_vp] * 10 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],
+        [_c_vp] * 10 + [_c_sz] + [_c_int] * 12 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
-    "rpa_page_scatter_ragged_quantised": (_c_int, [_c_vp] * 9 + [_c_int] * 10),
+    "rpa_page_scatter_ragged_quantised": (_c_int, [_c_vp] * 9 + [_c_int] * 11),
     "rpa_ragged_paged_attention_v3_quantised": (
         _c_int,
-        [_c_vp] * 12 + [_c_sz] + [_c_int] * 12 + [_c_f32, _c_int, _c_f32, _c_vp],
+        [_c_vp] * 12 + [_c_sz] + [_c_int] * 13 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
     "rpa_unified_attention": (
         _c_int,
@@ -42,7 +42,7 @@ SIGNATURES = {
     ),
     "rpa_ragged_paged_attention_v3": (
         _c_int,
-        [_c_vp] * 11 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],
+        [_c_vp] * 11 + [_c_sz] + [_c_int] * 12 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
     "rpa_mla_ragged_paged_attention": (
         _c_int,

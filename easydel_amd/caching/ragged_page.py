@@ -2,9 +2,12 @@
 
 Host-side mirror of the reference's ``easydel/caching/ragged_page/cache.py`` and ``utils.py`` for one
 MI355X: the same names, shapes and padding conventions, with torch tensors as the owners of device
-memory.  Two deliberate extensions, both new formats of this build: int8 is accepted as a cache dtype
-(the reference's ``get_dtype_packing`` only takes float dtypes, ``cache.py:143-158``), and a view may
-carry ``kv_scales [num_pages, combined_heads]`` float32 for fp8-e4m3 / int8 pages.
+memory.  An fp8 cache is by default what it is in the reference: pages of cast codes without scales
+(``cache.py:143-158`` gives fp8 a packing of 4; the operation casts K/V to the cache dtype and writes them,
+``operations/kernels/ragged_page_attention.py:570-580``).  Two deliberate extensions, both new formats of
+this build: int8 is accepted as a cache dtype (the reference's ``get_dtype_packing`` only takes float
+dtypes), and a view may carry ``kv_scales [num_pages, combined_heads]`` float32 for fp8-e4m3 / int8 pages
+(``RaggedPagesCacheView.init(..., scaled=True)``; always for int8).
 """
 
 from __future__ import annotations
@@ -143,7 +146,10 @@ class RaggedPagesCacheConfig:
         per_token = 1
         for s in shape[2:]:
             per_token *= s
-        return per_token // self.k_headdim
+        stored = shape[-1]
+        if self.k_headdim == 64 and self.version == "v3":
+            stored = 64  # K_h | V_h share one 128-wide row
+        return per_token // stored
 
 
 @dataclass
@@ -201,11 +207,19 @@ class RaggedPagesCacheView:
     kv_scales: torch.Tensor | None = None  # [num_pages, combined_heads] float32 for fp8 / int8 pages
 
     @classmethod
-    def init(cls, config: RaggedPagesCacheConfig, layer_index: int | None = None, device="cuda:0") -> "RaggedPagesCacheView":
+    def init(cls, config: RaggedPagesCacheConfig, layer_index: int | None = None, device="cuda:0",
+             scaled: bool | None = None) -> "RaggedPagesCacheView":
+        """Zeroed pages (reference ``cache.py:788-823``).  ``scaled``: give 8-bit pages per-(page, combined head)
+        scales, written by the quantising page write; default: only for int8, fp8 pages hold plain casts as in the
+        reference."""
         shape, _ = config.get_shape_and_axes()
         pages = torch.zeros(shape, dtype=config.kvdtype, device=device)
         scales = None
-        if config.kvdtype in (torch.float8_e4m3fn, torch.int8):
+        if scaled is None:
+            scaled = config.kvdtype == torch.int8
+        if scaled:
+            if config.kvdtype not in (torch.float8_e4m3fn, torch.int8):
+                raise ValueError(f"scaled pages are 8-bit pages, not {config.kvdtype}")
             scales = torch.ones((config.num_pages, config.combined_heads_per_token), dtype=torch.float32, device=device)
         return cls(metadata=config, kv_pages=pages, layer_index=layer_index, kv_scales=scales)
 

@@ -4,7 +4,9 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
+#include "../../include/rpa_hip_probe.h"
 #include "rpa_common.h"
 #include "rpa_mla.h"
 
@@ -12,26 +14,33 @@ namespace rpa {
 int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_t*, void*, int, int, int64_t, int,
                           int64_t, int);
 int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
-                          const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int);
+                          const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int);
 int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
 size_t launch_read_probe(hipStream_t, const void*, size_t, int, int, uint32_t*);
 int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
-                                const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int);
+                                const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int, int);
 }  // namespace rpa
 
 namespace {
 
 thread_local char g_err[512] = "";
-std::atomic<int> g_max_splits{0};   // 0 = sized from the shapes
-std::atomic<int> g_prefill_chunks{0};  // 0 = default (kMaxPrefillChunks)
-std::atomic<int> g_decode_sync{8};  // workgroup barrier every this many decode tiles (power of two, 0 = never)
-std::atomic<int> g_decode_wgs{0};   // 0 = as many persistent workgroups as are resident at once
-std::atomic<int> g_force_generic{0};
-std::atomic<int> g_prefill_dma{1};
-std::atomic<int> g_decode_pace{1};
-std::atomic<int> g_mla_chunks{0};  // 0 = sized from the shapes
-std::atomic<int> g_mla_min_chunk{0};  // 0 = default
-std::atomic<int> g_stages{15};  // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
+
+// Test and measurement knobs (rpa_set_tunable, declared in rpa_hip_probe.h).  They belong to the thread that sets
+// them: a call sees the values of its own thread only, read once when it starts, so a thread that never calls
+// rpa_set_tunable always runs with the defaults below, whatever a profiling or test thread of the same process does.
+struct Tunables {
+  int max_splits = 0;      // 0 = sized from the shapes
+  int prefill_chunks = 0;  // 0 = default (kMaxPrefillChunks)
+  int decode_sync = 8;     // workgroup barrier every this many decode tiles (power of two, 0 = never)
+  int decode_wgs = 0;      // 0 = as many persistent workgroups as are resident at once
+  int force_generic = 0;
+  int prefill_dma = 1;
+  int decode_pace = 1;
+  int mla_chunks = 0;      // 0 = sized from the shapes
+  int mla_min_chunk = 0;   // 0 = default
+  int stages = 15;         // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
+};
+thread_local Tunables g_tun;
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -57,7 +66,7 @@ size_t part_ml_bytes(int T, int Hq) { return align256((size_t)T * Hq * 2 * 4); }
 // long spans on every workgroup, so that one long sequence in a batch of short ones leaves most of the chip idle:
 // with a 256 MiB cap a 100k-token sequence among 255 short ones ran on 40 % of the workgroups.)
 int static_splits(int T, int M, int page_size, int Hq, int D) {
-  const int forced = g_max_splits.load();
+  const int forced = g_tun.max_splits;
   if (forced > 0) return forced < 2 ? 2 : forced;
   long want = ((long)M * page_size + 255) / 256 + 1;
   const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
@@ -73,12 +82,13 @@ int static_splits(int T, int M, int page_size, int Hq, int D) {
 // buffers ([chunks][T][Hq][D+2] floats) are kept under ~1 GiB by allowing fewer, longer chunks.
 // Compute units of the current device (256 on MI355X); 0 if the query fails.
 int device_cus() {
-  static std::atomic<int> cached{-1};
-  int v = cached.load();
-  if (v >= 0) return v;
+  static std::atomic<int> cached[rpa::kMaxDevices];  // per device; 0 = not looked up yet (a racing first call stores the same value)
   int dev = 0, cus = 0;
-  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
-  cached.store(cus);
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= rpa::kMaxDevices) return 0;
+  const int v = cached[dev].load(std::memory_order_relaxed);
+  if (v > 0) return v;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) cus = 0;
+  cached[dev].store(cus, std::memory_order_relaxed);
   return cus;
 }
 
@@ -88,9 +98,9 @@ int device_cus() {
 // whose bounds already allow many times more row tiles than workgroups fit on the chip is not cut at all.
 void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int* chunk_keys, int* max_chunks) {
   const long span = (long)M * page_size;
-  int chunks = g_prefill_chunks.load() > 0 ? g_prefill_chunks.load() : rpa::kMaxPrefillChunks;
+  int chunks = g_tun.prefill_chunks > 0 ? g_tun.prefill_chunks : rpa::kMaxPrefillChunks;
   if (chunks > rpa::kMaxPrefillChunks) chunks = rpa::kMaxPrefillChunks;
-  if (g_prefill_chunks.load() <= 0 && Hkv > 0) {
+  if (g_tun.prefill_chunks <= 0 && Hkv > 0) {
     const long row_tiles = ((long)T * (Hq / Hkv) / rpa::kPrefillRows + S) * Hkv;  // the prefill grid's bound without cutting
     const int cus = device_cus();
     if (cus > 0) {  // about eight units per CU fill the chip evenly; more chunks than that only add partials
@@ -125,13 +135,13 @@ int decode_token_bound(int T, int S, int Hq, int Hkv, int dec_rows) {
 // hence the longer minimum there.  The partial buffers stay under ~1 GiB.
 void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* min_chunk) {
   const long slots = (long)T * Hq / rpa::kMlaRows + S;
-  long chunks = g_mla_chunks.load() > 0 ? g_mla_chunks.load() : (768 + slots - 1) / slots;
+  long chunks = g_tun.mla_chunks > 0 ? g_tun.mla_chunks : (768 + slots - 1) / slots;
   if (chunks > rpa::kMlaMaxChunks) chunks = rpa::kMlaMaxChunks;
   if (chunks < 1) chunks = 1;
   const size_t per = part_o_bytes(T, Hq, lkv) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   *max_chunks = (int)chunks;
-  *min_chunk = g_mla_min_chunk.load() > 0 ? g_mla_min_chunk.load() : (Hq >= 64 ? 1024 : 512);
+  *min_chunk = g_tun.mla_min_chunk > 0 ? g_tun.mla_min_chunk : (Hq >= 64 ? 1024 : 512);
 }
 
 bool mla_shape_on_mfma(int page_size, int lkv, int rope, int row_elems, int q_dtype, int kv_dtype) {
@@ -148,24 +158,25 @@ const char* rpa_last_error(void) { return g_err; }
 
 int rpa_set_tunable(const char* name, int value) {
   if (!name) return -1;
+  auto swap = [](int& slot, int v) { const int old = slot; slot = v; return old; };
   if (!strcmp(name, "max_splits")) {
     if (value < 0) value = 0;
     if (value > rpa::kMaxSplitsCap) value = rpa::kMaxSplitsCap;
-    return g_max_splits.exchange(value);
+    return swap(g_tun.max_splits, value);
   }
-  if (!strcmp(name, "prefill_chunks")) return g_prefill_chunks.exchange(value < 0 ? 0 : value);
+  if (!strcmp(name, "prefill_chunks")) return swap(g_tun.prefill_chunks, value < 0 ? 0 : value);
   if (!strcmp(name, "decode_sync")) {
     int pow2 = 0;
     if (value > 0) for (pow2 = 1; pow2 * 2 <= value && pow2 < 1024; pow2 *= 2) {}
-    return g_decode_sync.exchange(pow2);
+    return swap(g_tun.decode_sync, pow2);
   }
-  if (!strcmp(name, "decode_wgs")) return g_decode_wgs.exchange(value < 0 ? 0 : value);
-  if (!strcmp(name, "force_generic")) return g_force_generic.exchange(value != 0);
-  if (!strcmp(name, "prefill_dma")) return g_prefill_dma.exchange(value != 0);
-  if (!strcmp(name, "decode_pace")) return g_decode_pace.exchange(value != 0);
-  if (!strcmp(name, "mla_min_chunk")) return g_mla_min_chunk.exchange(value <= 0 ? 0 : ((value + 63) & ~63));
-  if (!strcmp(name, "mla_chunks")) return g_mla_chunks.exchange(value < 0 ? 0 : (value > rpa::kMlaMaxChunks ? rpa::kMlaMaxChunks : value));
-  if (!strcmp(name, "stages")) return g_stages.exchange(value & 15);
+  if (!strcmp(name, "decode_wgs")) return swap(g_tun.decode_wgs, value < 0 ? 0 : value);
+  if (!strcmp(name, "force_generic")) return swap(g_tun.force_generic, value != 0);
+  if (!strcmp(name, "prefill_dma")) return swap(g_tun.prefill_dma, value != 0);
+  if (!strcmp(name, "decode_pace")) return swap(g_tun.decode_pace, value != 0);
+  if (!strcmp(name, "mla_min_chunk")) return swap(g_tun.mla_min_chunk, value <= 0 ? 0 : ((value + 63) & ~63));
+  if (!strcmp(name, "mla_chunks")) return swap(g_tun.mla_chunks, value < 0 ? 0 : (value > rpa::kMlaMaxChunks ? rpa::kMlaMaxChunks : value));
+  if (!strcmp(name, "stages")) return swap(g_tun.stages, value & 15);
   return -1;
 }
 
@@ -202,30 +213,41 @@ int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32
                   "rpa_page_scatter_slices launch");
 }
 
+// Stored row width of a combined head: Dp >= D elements (the reference pads head sizes that are not 64 or a multiple of
+// 128 up to the next multiple of 128, easydel/caching/ragged_page/cache.py:640-647); rows must keep 4-byte alignment.
+static int check_row_width(const char* who, int D, int Dp, int elem) {
+  if (Dp < D) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: stored head width Dp=%d < head_dim D=%d", who, Dp, D);
+  if (((int64_t)Dp * elem) % 4 != 0 || ((int64_t)D * elem) % 4 != 0)
+    return fail(RPA_ERR_UNSUPPORTED, "%s: head rows of D=%d / Dp=%d elements of %d bytes are not 4-byte multiples", who, D, Dp, elem);
+  return RPA_OK;
+}
+
 int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
                             const int32_t* context_lens, const int32_t* block_tables,
                             const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M, int P,
-                            int page_size, int Hkv, int D, int C, int elem_bytes) {
+                            int page_size, int Hkv, int D, int Dp, int C, int elem_bytes) {
   if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hkv <= 0 || D <= 0 || C < 2 * Hkv ||
       (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4))
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged: bad size (T=%d S=%d M=%d P=%d page_size=%d Hkv=%d D=%d C=%d elem=%d)",
                 T, S, M, P, page_size, Hkv, D, C, elem_bytes);
+  if (const int rc = check_row_width("rpa_page_scatter_ragged", D, Dp, elem_bytes)) return rc;
   if (T == 0) return RPA_OK;
   if (!key || !value || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs)
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged: null pointer");
   return hip_fail(rpa::launch_scatter_ragged((hipStream_t)stream, key, value, kv_pages, context_lens, block_tables,
-                                             query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, elem_bytes),
+                                             query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, Dp, elem_bytes),
                   "rpa_page_scatter_ragged launch");
 }
 
 int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
                                       float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
                                       const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M, int P,
-                                      int page_size, int Hkv, int D, int C, int src_dtype, int kv_dtype) {
+                                      int page_size, int Hkv, int D, int Dp, int C, int src_dtype, int kv_dtype) {
   if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hkv <= 0 || D <= 0 || C < 2 * Hkv)
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: bad size (T=%d S=%d M=%d P=%d page_size=%d Hkv=%d D=%d C=%d)",
                 T, S, M, P, page_size, Hkv, D, C);
-  if (D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "rpa_page_scatter_ragged_quantised: head_dim %d is not a multiple of 4", D);
+  if (D % 4 != 0 || Dp % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "rpa_page_scatter_ragged_quantised: head_dim %d / stored width %d is not a multiple of 4", D, Dp);
+  if (Dp < D) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: stored head width Dp=%d < head_dim D=%d", Dp, D);
   if (src_dtype != RPA_F32 && src_dtype != RPA_BF16)
     return fail(RPA_ERR_UNSUPPORTED, "rpa_page_scatter_ragged_quantised: source dtype %d (want f32 or bf16)", src_dtype);
   if (kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8)
@@ -236,7 +258,7 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
   if ((((uintptr_t)key) | ((uintptr_t)value)) & 15 || ((uintptr_t)kv_pages & 3))
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_page_scatter_ragged_quantised: key/value must be 16-byte and kv_pages 4-byte aligned");
   return hip_fail(rpa::launch_scatter_ragged_quant((hipStream_t)stream, key, value, kv_pages, kv_scales, context_lens,
-                                                   block_tables, query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C,
+                                                   block_tables, query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, Dp,
                                                    src_dtype, kv_dtype),
                   "rpa_page_scatter_ragged_quantised launch");
 }
@@ -256,23 +278,28 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
 
 // Shared body of the attention entry points.  k_pages / v_pages and the strides describe where K and V of
 // (page, token, KV head) lie (sizes are validated here, so the callers' stride arithmetic may see nonsense and
-// must not act on it); C is the row length of kv_scales; num_seqs may be null (every row live) if the caller allows.
+// must not act on it); Dp is the stored row width of a head (>= D), C the row length of kv_scales; num_seqs may be null
+// (every row live) if the caller allows.  The workspace is laid out here from the bytes the caller hands over: the
+// partial slots and key chunks shrink to what fits (never below two slots, else RPA_ERR_WORKSPACE), so the launch
+// never writes past workspace_bytes whatever sizing call preceded it.
 static int attention_impl(const char* who, rpa_stream_t stream, const void* q, const void* k_pages, const void* v_pages,
                           int64_t token_stride, int64_t head_stride, const float* kv_scales,
                           const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
                           const int32_t* num_seqs, bool num_seqs_optional, void* out, void* workspace,
-                          size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
-                          int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
+                          size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int Dp,
+                          int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
                           const float* softmax_aux, const void* new_key = nullptr, const void* new_value = nullptr) {
   if (T < 0 || S <= 0 || M <= 0 || P <= 0 || page_size <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (T=%d S=%d M=%d P=%d page_size=%d Hq=%d Hkv=%d D=%d)", who,
                 T, S, M, P, page_size, Hq, Hkv, D);
   if (Hq % Hkv != 0) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: Hq=%d is not a multiple of Hkv=%d", who, Hq, Hkv);
-  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16) return fail(RPA_ERR_UNSUPPORTED, "%s: q_dtype %d (want f32 or bf16)", who, q_dtype);
-  if (kv_dtype < RPA_F32 || kv_dtype > RPA_INT8) return fail(RPA_ERR_UNSUPPORTED, "%s: kv_dtype %d", who, kv_dtype);
+  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16 && q_dtype != RPA_F16)
+    return fail(RPA_ERR_UNSUPPORTED, "%s: q_dtype %d (want f32, bf16 or f16)", who, q_dtype);
+  if (kv_dtype < RPA_F32 || kv_dtype > RPA_F16) return fail(RPA_ERR_UNSUPPORTED, "%s: kv_dtype %d", who, kv_dtype);
   if (D > 256 || D % 4 != 0) return fail(RPA_ERR_UNSUPPORTED, "%s: head_dim %d (want a multiple of 4, <= 256)", who, D);
-  if ((kv_dtype == RPA_FP8_E4M3 || kv_dtype == RPA_INT8) && !kv_scales)
-    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: 8-bit KV pages need kv_scales", who);
+  if (const int rc = check_row_width(who, D, Dp, rpa::elem_bytes(kv_dtype))) return rc;
+  if (kv_scales && kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: kv_scales with pages that are not 8-bit (kv_dtype %d)", who, kv_dtype);
   if (kv_scales && ((uintptr_t)kv_scales & 7))
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: kv_scales must be 8-byte aligned", who);
   if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_scale is not finite", who);
@@ -284,12 +311,15 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   if ((((uintptr_t)q) | ((uintptr_t)out) | ((uintptr_t)k_pages) | ((uintptr_t)v_pages)) & 15)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: q, out and the page pools must be 16-byte aligned", who);
 
+  const Tunables tun = g_tun;  // this thread's knobs, read once per call
   rpa::AttnParams p;
   memset(&p, 0, sizeof(p));
   p.q = q; p.k_pages = k_pages; p.v_pages = v_pages; p.kv_scales = kv_scales; p.sinks = softmax_aux;
   p.context_lens = context_lens; p.block_tables = block_tables; p.qsl = query_start_loc; p.num_seqs = num_seqs;
   p.out = out;
-  p.T = T; p.S = S; p.M = M; p.P = P; p.page_size = page_size; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv; p.D = D; p.C = C;
+  p.T = T; p.S = S; p.M = M; p.P = P; p.page_size = page_size; p.Hq = Hq; p.Hkv = Hkv; p.group = Hq / Hkv; p.C = C;
+  p.D = D; p.Dq = D;
+  p.kv_pad_bytes = (Dp - D) * rpa::elem_bytes(kv_dtype);
   p.token_stride = token_stride;
   p.head_stride = head_stride;
   p.page_stride = p.token_stride * page_size;
@@ -298,36 +328,41 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.window = sliding_window > 0 ? sliding_window : 0;
   p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
-  p.decode_wgs = g_decode_wgs.load();
-  p.decode_sync = g_decode_sync.load();
-  p.prefill_dma = g_prefill_dma.load();
-  p.decode_pace = g_decode_pace.load();
+  p.decode_wgs = tun.decode_wgs;
+  p.decode_sync = tun.decode_sync;
+  p.prefill_dma = tun.prefill_dma;
+  p.decode_pace = tun.decode_pace;
   p.max_splits = 2;
-  p.dec_rows = rpa::decode_row_limit(T, S, D, kv_dtype);
   p.pre_chunk = 1 << 30;
   p.pre_max_chunks = 1;
-  p.mfma_path = (!g_force_generic.load() && rpa::decode_supported(p)) ? 1 : 0;
+  // Padded head storage (Dp = 128 or 256 > D): the MFMA kernels compute with the stored width -- q rows are padded with
+  // zeros in registers, the pages' padding holds zeros (the write puts them there), output dims past D are not stored.
+  if (Dp > D && (Dp == 128 || Dp == 256)) p.D = Dp;
+  p.dec_rows = rpa::decode_row_limit(T, S, p.D, kv_dtype);
+  p.mfma_path = (!tun.force_generic && rpa::decode_supported(p)) ? 1 : 0;
+  if (!p.mfma_path) p.D = D;
 
   hipStream_t s = (hipStream_t)stream;
-  const int stages = g_stages.load();
+  const int stages = tun.stages;
   if (new_key) {  // fused write + attention: the new rows go into the pages before any kernel reads them
     if (p.mfma_path && (stages & 1)) {
       p.new_k = new_key;  // copied by extra blocks of the decode plan kernel's launch
       p.new_v = new_value;
     } else {
       const int err = rpa::launch_scatter_ragged(s, new_key, new_value, const_cast<void*>(k_pages), context_lens, block_tables,
-                                                 query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, rpa::elem_bytes(kv_dtype));
+                                                 query_start_loc, num_seqs, T, S, M, P, page_size, Hkv, D, C, Dp, rpa::elem_bytes(kv_dtype));
       if (err) return hip_fail(err, "page scatter launch");
     }
   }
   if (p.mfma_path) {
+    const int Dc = p.D;  // head size the partial rows are laid out with
     const int td = decode_token_bound(T, S, Hq, Hkv, p.dec_rows);
     p.t_dec_max = td;
-    const size_t po = part_o_bytes(td, Hq, D), pml = part_ml_bytes(td, Hq), pb = plan_bytes(S);
-    int splits = static_splits(td, M, page_size, Hq, D);
+    const size_t po = part_o_bytes(td, Hq, Dc), pml = part_ml_bytes(td, Hq), pb = plan_bytes(S);
+    int splits = static_splits(td, M, page_size, Hq, Dc);
     int pre_keys, pre_chunks;
-    prefill_split(T, S, M, page_size, Hq, Hkv, D, &pre_keys, &pre_chunks);
-    const size_t pre_po = part_o_bytes(T, Hq, D), pre_pml = part_ml_bytes(T, Hq);
+    prefill_split(T, S, M, page_size, Hq, Hkv, Dc, &pre_keys, &pre_chunks);
+    const size_t pre_po = part_o_bytes(T, Hq, Dc), pre_pml = part_ml_bytes(T, Hq);
     size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (pre_po + pre_pml) : 0;
     size_t usable = workspace_bytes > 256 + pb ? workspace_bytes - 256 - pb : 0;
     if (!workspace || usable < 2 * (po + pml))
@@ -367,16 +402,16 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
                                const int32_t* context_lens, const int32_t* block_tables,
                                const int32_t* query_start_loc, const int32_t* num_seqs, void* out, void* workspace,
                                size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq, int Hkv,
-                               int D, int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
+                               int D, int Dp, int C, int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
                                float logits_soft_cap, const float* softmax_aux) {
   if (Hkv > 0 && C < 2 * Hkv)
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention: C=%d combined heads < 2*Hkv=%d", C, 2 * Hkv);
-  // interleaved pages: K of head h in combined head 2h, V in 2h+1, one row of D elements each
-  const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
+  // interleaved pages: K of head h in combined head 2h, V in 2h+1, one stored row of Dp elements each
+  const int64_t row = (int64_t)Dp * rpa::elem_bytes(kv_dtype);
   const void* v_pages = kv_pages ? (const char*)kv_pages + row : nullptr;
   return attention_impl("rpa_ragged_paged_attention", stream, q, kv_pages, v_pages, (int64_t)C * row, 2 * row, kv_scales,
                         context_lens, block_tables, query_start_loc, num_seqs, false, out, workspace, workspace_bytes, T, S,
-                        M, P, page_size, Hq, Hkv, D, C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap,
+                        M, P, page_size, Hq, Hkv, D, Dp, C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap,
                         softmax_aux);
 }
 
@@ -390,7 +425,7 @@ int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_ca
   const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
   return attention_impl("rpa_unified_attention", stream, q, key_cache, value_cache, (int64_t)Hkv * row, row, kv_scales,
                         context_lens, block_tables, query_start_loc, num_seqs, true, out, workspace, workspace_bytes, T, S, M,
-                        P, page_size, Hq, Hkv, D, 2 * Hkv, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap,
+                        P, page_size, Hq, Hkv, D, D, 2 * Hkv, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap,
                         softmax_aux);
 }
 
@@ -398,20 +433,19 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
                                   const int32_t* query_start_loc, const int32_t* distribution, void* out,
                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P, int page_size,
-                                  int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype, float softmax_scale,
+                                  int Hq, int Hkv, int D, int Dp, int C, int q_dtype, int kv_dtype, float softmax_scale,
                                   int sliding_window, float logits_soft_cap, const float* softmax_aux) {
   const char* who = "rpa_ragged_paged_attention_v3";
-  if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16)
-    return fail(RPA_ERR_UNSUPPORTED, "%s: quantised pages are read-only (kv_dtype %d)", who, kv_dtype);
   if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null distribution", who);
   if (Hkv > 0 && C < 2 * Hkv) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: C=%d combined heads < 2*Hkv=%d", who, C, 2 * Hkv);
   if (T > 0 && (!key || !value)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null key / value", who);
   const int32_t* n_live = distribution + 2;
-  const int64_t row = (int64_t)D * rpa::elem_bytes(kv_dtype);
+  const int64_t row = (int64_t)Dp * rpa::elem_bytes(kv_dtype);
   const void* v_pages = kv_pages ? (const char*)kv_pages + row : nullptr;
+  // 8-bit pages here are unscaled: key / value hold the cast codes, which are copied and later read as the values
   return attention_impl(who, stream, q, kv_pages, v_pages, (int64_t)C * row, 2 * row, nullptr, context_lens, block_tables,
-                        query_start_loc, n_live, false, out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C,
-                        q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux, key, value);
+                        query_start_loc, n_live, false, out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, Dp,
+                        C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux, key, value);
 }
 
 int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, const void* key, const void* value,
@@ -419,16 +453,16 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
                                             const int32_t* block_tables, const int32_t* query_start_loc,
                                             const int32_t* distribution, void* out, void* workspace,
                                             size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq,
-                                            int Hkv, int D, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
+                                            int Hkv, int D, int Dp, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
                                             float softmax_scale, int sliding_window, float logits_soft_cap,
                                             const float* softmax_aux) {
   if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_ragged_paged_attention_v3_quantised: null distribution");
   const int32_t* n_live = distribution + 2;
   int err = rpa_page_scatter_ragged_quantised(stream, key, value, kv_pages, kv_scales, context_lens, block_tables,
-                                              query_start_loc, n_live, T, S, M, P, page_size, Hkv, D, C, kv_src_dtype, kv_dtype);
+                                              query_start_loc, n_live, T, S, M, P, page_size, Hkv, D, Dp, C, kv_src_dtype, kv_dtype);
   if (err) return err;
   return rpa_ragged_paged_attention(stream, q, kv_pages, kv_scales, context_lens, block_tables, query_start_loc, n_live,
-                                    out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, C, q_dtype,
+                                    out, workspace, workspace_bytes, T, S, M, P, page_size, Hq, Hkv, D, Dp, C, q_dtype,
                                     kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux);
 }
 
@@ -514,7 +548,7 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.window = sliding_window > 0 ? sliding_window : 0;
   p.softcap = logits_soft_cap > 0.f ? logits_soft_cap : 0.f;
-  p.mfma = (!g_force_generic.load() && rpa::mla_mfma_supported(p)) ? 1 : 0;
+  p.mfma = (!g_tun.force_generic && rpa::mla_mfma_supported(p)) ? 1 : 0;
   hipStream_t s = (hipStream_t)stream;
   if (keys_values && !p.mfma) {  // on the matrix-core path the write rides along with the plan kernel's launch
     const int err = rpa::launch_mla_scatter(s, p);

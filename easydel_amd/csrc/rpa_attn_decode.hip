@@ -21,6 +21,7 @@
 // LDS tiles are wave-private and LDS operations of one wave execute in order, so no barrier is needed for
 // correctness; one every few tiles keeps the workgroup's waves on the same token rows, which keeps its
 // outstanding loads inside the same DRAM rows.
+#include <atomic>
 #include <type_traits>
 
 #include "rpa_mfma.h"
@@ -139,7 +140,10 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 #pragma unroll
     for (int u = 0; u < NLD; ++u) stage[B][u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
     // a vector load on purpose: a scalar load would be waited for together with the next LDS read
-    if constexpr (EB == 1) sc_stage[B] = *(const u32x2*)(p.kv_scales + (int64_t)page * p.C + 2 * h);
+    if constexpr (EB == 1) {
+      if (p.kv_scales) sc_stage[B] = *(const u32x2*)(p.kv_scales + (int64_t)page * p.C + 2 * h);
+      else sc_stage[B] = (u32x2){0x3f800000u, 0x3f800000u};  // unscaled 8-bit pages: the codes are the values
+    }
   };
   using Buf0 = std::integral_constant<int, 0>;
   using Buf1 = std::integral_constant<int, DEPTH - 1>;
@@ -198,14 +202,14 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   bf16x8 qf[RB][NKK];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok[rb]) * p.Hq + (h * G + r_head[rb])) * D * 2;
+    const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok[rb]) * p.Hq + (h * G + r_head[rb])) * p.Dq * 2;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
       // bf16 pages: step kk covers dims 32kk + 8g4 + e.  8-bit pages: a 16-byte K chunk holds 16
       // dims, so steps (2j, 2j+1) cover dims 64j + 16g4 + 8b + e.
       const int d0 = (EB == 2) ? (kk * 32 + 8 * g4) : ((kk >> 1) * 64 + 16 * g4 + 8 * (kk & 1));
       u32x4 v = {0u, 0u, 0u, 0u};
-      if (n + 16 * rb < rows) v = *(const u32x4*)(qrow + d0 * 2);
+      if (n + 16 * rb < rows && d0 < p.Dq) v = *(const u32x4*)(qrow + d0 * 2);  // dims past Dq: zero padding
       qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
     }
   }
@@ -428,20 +432,21 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
       if (cur.single) {
         const float l_fin = with_sink(p, head_out, m_run[rb], l_tot);
         const float inv = (l_fin > 0.f ? 1.f / l_fin : 0.f) * v_unit;
-        uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * D;
+        uint16_t* orow = (uint16_t*)p.out + ((int64_t)tok_out * p.Hq + head_out) * p.Dq;
         if constexpr (EB == 2) {
 #pragma unroll
           for (int rt = 0; rt < DPL; ++rt) {
             const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
                              pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
-            *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
+            if (16 * rt + 4 * g4 < p.Dq) *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
           }
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int rt = 0; rt < DPL; rt += 2)
-              *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
+              if (DPL * (4 * g4 + j) + rt < p.Dq)
+                *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
         }
       } else {
         const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok[rb]) * p.Hq + head_out;
@@ -478,8 +483,8 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     const int t = ((int)blockIdx.x - 1) * kScatterTokensPerBlock + (int)(threadIdx.x >> 6);
     if (t < p.T)
       scatter_token((const char*)p.new_k, (const char*)p.new_v, (char*)p.k_pages, (char*)p.v_pages, p.context_lens,
-                    p.block_tables, p.qsl, live_rows(p), p.M, p.P, p.page_size, p.Hkv, p.D * elem_bytes_dev(p.kv_dtype),
-                    p.head_stride, p.token_stride, p.page_stride, t, threadIdx.x & 63, 64);
+                    p.block_tables, p.qsl, live_rows(p), p.M, p.P, p.page_size, p.Hkv, p.Dq * elem_bytes_dev(p.kv_dtype),
+                    p.head_stride, p.token_stride, p.page_stride, t, threadIdx.x & 63, 64, p.kv_pad_bytes);
     return;
   }
   __shared__ int part[1024], part2[1024];
@@ -570,15 +575,20 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 static int launch_rb(hipStream_t stream, AttnParams p) {
   constexpr bool PACE = ElemBytes<KVT>::v == 2 && WPB == 8;
-  // persistent grid: as many workgroups as are resident at once, per KV-head group
-  static int resident = 0;
+  // persistent grid: as many workgroups as are resident at once, per KV-head group.  The figure belongs to the device
+  // the call runs on; it is looked up once per device and kernel (a racing first call computes the same value).
+  static std::atomic<int> resident_of[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
+  if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  int resident = resident_of[dev].load(std::memory_order_relaxed);
   if (resident == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return (int)hipGetLastError();
+    int cus = 0, per_cu = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP, RB, PACE>, 64 * WPB, 0) != hipSuccess)
       return (int)hipGetLastError();
     resident = max(1, cus * max(1, per_cu));
+    resident_of[dev].store(resident, std::memory_order_relaxed);
   }
   const int head_groups = (p.Hkv + WPB - 1) / WPB;
   int n_wg = resident / head_groups;
@@ -647,9 +657,10 @@ int decode_row_limit(int T, int S, int D, int kv_dtype) {
 
 bool decode_supported(const AttnParams& p) {
   if (p.q_dtype != RPA_BF16 || p.kv_dtype == RPA_F32) return false;
+  if (p.kv_dtype == RPA_F16) return false;
   if (p.D != 64 && p.D != 128 && p.D != 256) return false;
+  if (p.Dq > p.D || p.Dq % 8 != 0) return false;  // a q row is read in 16-byte chunks, whole chunks inside or outside Dq
   if (p.page_size % 16 != 0) return false;
-  if (p.kv_dtype != RPA_BF16 && p.kv_scales == nullptr) return false;
   if (!(p.scale > 0.f)) return false;  // the MFMA kernels take the running max before scaling
   return true;
 }

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
   if (!sp.live) return;
   if (p.mfma_path && sp.small_rows) return;  // the MFMA decode kernel owns these rows
 
-  const int D = p.D;
+  const int D = p.Dq;  // q / out row length; the pages are addressed through the strides
   const int h = hq / p.group;
   const int pos = sp.ctx - sp.q_len + (t - sp.q0);
   int k_hi = pos + 1;
@@ -96,10 +96,7 @@ __global__ __launch_bounds__(64) void attn_generic_kernel(AttnParams p) {
   for (int k = 0; k < 4; ++k) {
     const int d = lane + 64 * k;
     if (d < D) {
-      const int64_t o = ((int64_t)t * p.Hq + hq) * D + d;
-      const float r = acc[k] * inv;
-      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
-      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
+      store_out<QT>(p.out, ((int64_t)t * p.Hq + hq) * D + d, acc[k] * inv);
     }
   }
 }
@@ -112,14 +109,17 @@ static int launch_generic_q(hipStream_t stream, const AttnParams& p) {
     case RPA_BF16: hipLaunchKernelGGL((attn_generic_kernel<QT, RPA_BF16>), grid, block, 0, stream, p); break;
     case RPA_FP8_E4M3: hipLaunchKernelGGL((attn_generic_kernel<QT, RPA_FP8_E4M3>), grid, block, 0, stream, p); break;
     case RPA_INT8: hipLaunchKernelGGL((attn_generic_kernel<QT, RPA_INT8>), grid, block, 0, stream, p); break;
+    case RPA_F16: hipLaunchKernelGGL((attn_generic_kernel<QT, RPA_F16>), grid, block, 0, stream, p); break;
     default: return (int)hipErrorInvalidValue;
   }
   return (int)hipGetLastError();
 }
 
 int launch_attn_generic(hipStream_t stream, const AttnParams& p) {
-  if (p.D > 256) return (int)hipErrorInvalidValue;
-  return p.q_dtype == RPA_F32 ? launch_generic_q<RPA_F32>(stream, p) : launch_generic_q<RPA_BF16>(stream, p);
+  if (p.Dq > 256) return (int)hipErrorInvalidValue;
+  if (p.q_dtype == RPA_F32) return launch_generic_q<RPA_F32>(stream, p);
+  if (p.q_dtype == RPA_F16) return launch_generic_q<RPA_F16>(stream, p);
+  return launch_generic_q<RPA_BF16>(stream, p);
 }
 
 }  // namespace rpa

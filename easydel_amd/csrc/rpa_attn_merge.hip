@@ -110,12 +110,7 @@ __global__ __launch_bounds__(256, 8) void attn_merge_kernel(AttnParams p) {
 #pragma unroll
   for (int k = 0; k < NK; ++k) {
     const int d = lane + 64 * k;
-    if (d < D) {
-      const int64_t o = ((int64_t)t * p.Hq + hq) * D + d;
-      const float r = acc[k] * inv;
-      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
-      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
-    }
+    if (d < p.Dq) store_out<QT>(p.out, ((int64_t)t * p.Hq + hq) * p.Dq + d, acc[k] * inv);  // partial rows are D wide, out rows Dq
   }
 }
 
@@ -240,10 +235,8 @@ __global__ __launch_bounds__(256, 4) void attn_merge_wide_kernel(AttnParams p) {
 #pragma unroll
   for (int k = 0; k < NKT; ++k) {
     if (!zero && n_p[k / NK] == 0) continue;
-    const int64_t o = ((int64_t)t * p.Hq + hq0) * D + lane + 64 * k;
-    const float r = acc[k] * inv[k / NK];
-    if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
-    else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
+    const int d = (lane + 64 * k) % D;  // dim inside head k / NK (partial rows are D wide, out rows Dq)
+    if (d < p.Dq) store_out<QT>(p.out, ((int64_t)t * p.Hq + hq0 + k / NK) * p.Dq + d, acc[k] * inv[k / NK]);
   }
 }
 
@@ -264,6 +257,7 @@ static void launch_merge_q(hipStream_t stream, const AttnParams& p, int blocks) 
 int launch_attn_merge(hipStream_t stream, const AttnParams& p) {
   const int blocks = (p.T * p.Hq + 3) / 4;
   if (p.q_dtype == RPA_F32) launch_merge_q<RPA_F32>(stream, p, blocks);
+  else if (p.q_dtype == RPA_F16) launch_merge_q<RPA_F16>(stream, p, blocks);
   else launch_merge_q<RPA_BF16>(stream, p, blocks);
   return (int)hipGetLastError();
 }

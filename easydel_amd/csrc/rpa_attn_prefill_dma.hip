@@ -88,7 +88,15 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
 
   // ---- key range of the workgroup: one chunk of the row tile's range ----------------------------
   const PrefillTile pt = prefill_tile(p, sp, R0);
-  if (chunk >= pt.n_chunks) return;  // also: queries before position 0 have no keys; such rows stay unwritten
+  if (pt.n_chunks == 0 && chunk == 0) {  // every row of the tile lies before position 0 and sees no key: zeros
+    for (int e = tid; e < ROWS * (p.Dq / 4); e += 64 * NW) {
+      const int row = R0 + e / (p.Dq / 4), d4 = e % (p.Dq / 4);
+      if (row < rows_total)
+        *(u32x2*)((uint16_t*)p.out + ((int64_t)(sp.q0 + row / G) * p.Hq + h * G + row % G) * p.Dq + 4 * d4) = (u32x2){0u, 0u};
+    }
+    return;
+  }
+  if (chunk >= pt.n_chunks) return;
   const int base_pos = sp.ctx - sp.q_len;  // position of the sequence's first query token
   const int vis_lo = pt.vis_lo;
   // the first tile must hold vis_lo, so that rows of it that nobody may see can borrow a visible row's address
@@ -114,11 +122,11 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
     out_tok[rb] = sp.q0 + r_tok;
     out_head[rb] = h * G + r_head;
-    const char* qrow = (const char*)p.q + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D * 2;
+    const char* qrow = (const char*)p.q + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * p.Dq * 2;
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {
       u32x4 v = {0u, 0u, 0u, 0u};
-      if (row_ok[rb]) v = *(const u32x4*)(qrow + (kk * 32 + 8 * g4) * 2);
+      if (row_ok[rb] && kk * 32 + 8 * g4 < p.Dq) v = *(const u32x4*)(qrow + (kk * 32 + 8 * g4) * 2);  // dims past Dq: zero padding
       qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
     }
   }
@@ -452,12 +460,12 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       if (single) {
         const float l_fin = with_sink(p, out_head[rb], m_run[rb], l_tot);
         const float inv = l_fin > 0.f ? 1.f / l_fin : 0.f;
-        uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * D + 4 * g4;
+        uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * p.Dq + 4 * g4;
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
           const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
                            pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
-          *(u32x2*)(orow + 16 * rt) = w;
+          if (16 * rt + 4 * g4 < p.Dq) *(u32x2*)(orow + 16 * rt) = w;
         }
       } else {
         const int64_t pslot = ((int64_t)chunk * p.T + out_tok[rb]) * p.Hq + out_head[rb];

@@ -14,6 +14,7 @@ constexpr int kPlanHeader = 16;      // ints before the prefix array in the deco
 constexpr int kMaxDecodeWgs = 4096;  // persistent decode workgroups per KV-head group
 constexpr int kPrefillRows = 128;    // query rows (token x group head) one prefill workgroup owns
 constexpr int kMaxPrefillChunks = 8; // key chunks one prefill row tile may be split into
+constexpr int kMaxDevices = 64;      // devices of one process the per-device caches hold
 
 // Everything a kernel needs, passed by value.
 struct AttnParams {
@@ -39,9 +40,12 @@ struct AttnParams {
                    // P[S+1] exclusive prefix of per-sequence key spans, R[S+1] exclusive prefix of
                    // decode-class query tokens (row of a token in the partial buffers), first_seq[n_wg]
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
+  int Dq;                // elements of a q / out row.  D is the head size the kernels compute with: Dq itself, or -- on the
+                         // MFMA path over padded head storage -- the stored row width (128 / 256), whose padding holds zeros
   int64_t token_stride;  // bytes between consecutive tokens of a page = C*D*elem
   int64_t page_stride;   // bytes between pages
   int64_t head_stride;   // bytes between KV heads inside a token
+  int kv_pad_bytes;      // bytes of zero padding behind a head's Dq elements in the pages (padded head storage), else 0
   int q_dtype, kv_dtype;
   float scale;       // softmax scale
   float scale_log2;  // softmax scale * log2(e)
@@ -165,7 +169,7 @@ __device__ __forceinline__ void scatter_token(const char* __restrict__ key, cons
                                               const int32_t* __restrict__ block_tables, const int32_t* __restrict__ qsl,
                                               int n_live, int M, int P, int page_size, int Hkv, int head_bytes,
                                               int64_t head_stride, int64_t token_stride, int64_t page_stride, int t,
-                                              int tid, int nthreads) {
+                                              int tid, int nthreads, int pad_bytes = 0) {
   if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
   const int i = find_seq_wave(qsl, n_live, t);
   const int q0 = qsl[i], q_len = qsl[i + 1] - q0;
@@ -198,6 +202,14 @@ __device__ __forceinline__ void scatter_token(const char* __restrict__ key, cons
       dst[w] = src[w];
     }
   }
+  // padded head storage: the bytes between a head's head_bytes and its stored row width are written as zeros
+  if (pad_bytes > 0) {
+    const int n = 2 * Hkv * pad_bytes;
+    for (int k = tid; k < n; k += nthreads) {
+      const int ch = k / pad_bytes, w = k - ch * pad_bytes;
+      (((ch & 1) ? vdst : kdst) + (int64_t)(ch >> 1) * head_stride + head_bytes)[w] = 0;
+    }
+  }
 }
 
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
@@ -218,16 +230,26 @@ template <> struct ElemBytes<RPA_F32> { static constexpr int v = 4; };
 template <> struct ElemBytes<RPA_BF16> { static constexpr int v = 2; };
 template <> struct ElemBytes<RPA_FP8_E4M3> { static constexpr int v = 1; };
 template <> struct ElemBytes<RPA_INT8> { static constexpr int v = 1; };
+template <> struct ElemBytes<RPA_F16> { static constexpr int v = 2; };
 
-inline int elem_bytes(int dt) { return dt == RPA_F32 ? 4 : dt == RPA_BF16 ? 2 : 1; }
-__device__ __forceinline__ int elem_bytes_dev(int dt) { return dt == RPA_F32 ? 4 : dt == RPA_BF16 ? 2 : 1; }
+inline int elem_bytes(int dt) { return dt == RPA_F32 ? 4 : (dt == RPA_BF16 || dt == RPA_F16) ? 2 : 1; }
+__device__ __forceinline__ int elem_bytes_dev(int dt) { return dt == RPA_F32 ? 4 : (dt == RPA_BF16 || dt == RPA_F16) ? 2 : 1; }
 
 template <int DT>
 __device__ __forceinline__ float load_elem(const void* base, int64_t idx) {
   if constexpr (DT == RPA_F32) return ((const float*)base)[idx];
   else if constexpr (DT == RPA_BF16) return bf16_bits_to_float(((const uint16_t*)base)[idx]);
   else if constexpr (DT == RPA_FP8_E4M3) return fp8_e4m3_to_float(((const uint8_t*)base)[idx]);
+  else if constexpr (DT == RPA_F16) return (float)((const _Float16*)base)[idx];
   else return (float)((const int8_t*)base)[idx];
+}
+
+// One result element in the q / out element type (round to nearest even).
+template <int QT>
+__device__ __forceinline__ void store_out(void* base, int64_t idx, float r) {
+  if constexpr (QT == RPA_F32) ((float*)base)[idx] = r;
+  else if constexpr (QT == RPA_F16) ((_Float16*)base)[idx] = (_Float16)r;
+  else ((uint16_t*)base)[idx] = float_to_bf16_bits(r);
 }
 
 // Launchers (one per translation unit); all return a hipError_t as int.

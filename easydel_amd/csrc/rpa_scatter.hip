@@ -75,11 +75,12 @@ __global__ __launch_bounds__(256) void scatter_ragged_kernel(const char* __restr
                                                              const int32_t* __restrict__ block_tables,
                                                              const int32_t* __restrict__ qsl,
                                                              const int32_t* __restrict__ num_seqs, int S, int M, int P,
-                                                             int page_size, int Hkv, int head_bytes,
+                                                             int page_size, int Hkv, int head_bytes, int row_bytes,
                                                              int64_t token_stride, int64_t page_stride) {
-  // interleaved pages: V of a head one row behind its K, heads two rows apart
-  scatter_token(key, value, pages, pages + head_bytes, context_lens, block_tables, qsl, min(num_seqs[0], S), M, P, page_size, Hkv,
-                head_bytes, 2 * (int64_t)head_bytes, token_stride, page_stride, blockIdx.x, threadIdx.x, blockDim.x);
+  // interleaved pages: V of a head one stored row (row_bytes >= head_bytes) behind its K, heads two rows apart
+  scatter_token(key, value, pages, pages + row_bytes, context_lens, block_tables, qsl, min(num_seqs[0], S), M, P, page_size, Hkv,
+                head_bytes, 2 * (int64_t)row_bytes, token_stride, page_stride, blockIdx.x, threadIdx.x, blockDim.x,
+                row_bytes - head_bytes);
 }
 
 // ---- quantising ragged write ---------------------------------------------------------------------------
@@ -136,7 +137,7 @@ __global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __
                                                                   const int32_t* __restrict__ block_tables,
                                                                   const int32_t* __restrict__ qsl,
                                                                   const int32_t* __restrict__ num_seqs, int S, int M, int P,
-                                                                  int page_size, int Hkv, int D, int C) {
+                                                                  int page_size, int Hkv, int D, int C, int Dp) {
   const int t = blockIdx.x, c = blockIdx.y, lane = threadIdx.x;
   const int n_live = min(num_seqs[0], S);  // never more than the rows the metadata arrays hold
   if (n_live <= 0 || t < qsl[0] || t >= qsl[n_live]) return;
@@ -158,8 +159,8 @@ __global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __
   const void* src = (c & 1) ? value : key;
   const int64_t src0 = ((int64_t)t * Hkv + (c >> 1)) * D;  // element index of the first new token's head row
   const int64_t src_row = (int64_t)Hkv * D;
-  unsigned char* dst = pages + ((int64_t)page * page_size * C + c) * D;  // token row r of this head: dst + r*C*D
-  const int64_t dst_row = (int64_t)C * D;
+  unsigned char* dst = pages + ((int64_t)page * page_size * C + c) * Dp;  // token row r of this head: dst + r*C*Dp
+  const int64_t dst_row = (int64_t)C * Dp;  // stored rows are Dp >= D codes wide; the padding is written as zero codes
 
   float amax = 0.f;
   for (int idx = lane; idx < n * D4; idx += 64) {
@@ -190,17 +191,22 @@ __global__ __launch_bounds__(64) void scatter_ragged_quant_kernel(const void* __
     load4_src<SRC>(src, src0 + r * src_row + c4 * 4, f);
     *(uint32_t*)(dst + (first + r) * dst_row + c4 * 4) = quant4<KVT>(f[0] / new_scale, f[1] / new_scale, f[2] / new_scale, f[3] / new_scale);
   }
+  const int P4 = (Dp - D) >> 2;
+  for (int idx = lane; idx < n * P4; idx += 64) {
+    const int r = idx / P4, c4 = idx - r * P4;
+    *(uint32_t*)(dst + (first + r) * dst_row + D + c4 * 4) = 0u;
+  }
   if (lane == 0) scales[(int64_t)page * C + c] = new_scale;
 }
 
 int launch_scatter_ragged_quant(hipStream_t stream, const void* key, const void* value, void* pages, float* scales,
                                 const int32_t* context_lens, const int32_t* block_tables, const int32_t* qsl,
                                 const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int Hkv, int D, int C,
-                                int src_dtype, int kv_dtype) {
+                                int Dp, int src_dtype, int kv_dtype) {
   const dim3 grid(T, 2 * Hkv), block(64);
 #define RPA_QSCATTER(SRC, KVT)                                                                                        \
   hipLaunchKernelGGL((scatter_ragged_quant_kernel<SRC, KVT>), grid, block, 0, stream, key, value, (unsigned char*)pages, \
-                     scales, context_lens, block_tables, qsl, num_seqs, S, M, P, page_size, Hkv, D, C)
+                     scales, context_lens, block_tables, qsl, num_seqs, S, M, P, page_size, Hkv, D, C, Dp)
   if (src_dtype == RPA_F32 && kv_dtype == RPA_FP8_E4M3) RPA_QSCATTER(RPA_F32, RPA_FP8_E4M3);
   else if (src_dtype == RPA_F32 && kv_dtype == RPA_INT8) RPA_QSCATTER(RPA_F32, RPA_INT8);
   else if (src_dtype == RPA_BF16 && kv_dtype == RPA_FP8_E4M3) RPA_QSCATTER(RPA_BF16, RPA_FP8_E4M3);
@@ -271,11 +277,11 @@ int launch_scatter_slices(hipStream_t stream, const void* new_kv, const int32_t*
 int launch_scatter_ragged(hipStream_t stream, const void* key, const void* value, void* pages,
                           const int32_t* context_lens, const int32_t* block_tables, const int32_t* qsl,
                           const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int Hkv, int D, int C,
-                          int elem_bytes) {
-  const int head_bytes = D * elem_bytes;
-  const int64_t token_stride = (int64_t)C * head_bytes;
+                          int Dp, int elem_bytes) {
+  const int head_bytes = D * elem_bytes, row_bytes = Dp * elem_bytes;
+  const int64_t token_stride = (int64_t)C * row_bytes;
   hipLaunchKernelGGL(scatter_ragged_kernel, dim3(T), dim3(256), 0, stream, (const char*)key, (const char*)value,
-                     (char*)pages, context_lens, block_tables, qsl, num_seqs, S, M, P, page_size, Hkv, head_bytes,
+                     (char*)pages, context_lens, block_tables, qsl, num_seqs, S, M, P, page_size, Hkv, head_bytes, row_bytes,
                      token_stride, token_stride * page_size);
   return (int)hipGetLastError();
 }

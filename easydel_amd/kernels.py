@@ -18,6 +18,7 @@ _DTYPE_TAG = {
     torch.bfloat16: _lib.RPA_BF16,
     torch.float8_e4m3fn: _lib.RPA_FP8_E4M3,
     torch.int8: _lib.RPA_INT8,
+    torch.float16: _lib.RPA_F16,
 }
 
 _workspaces: dict[tuple, torch.Tensor] = {}
@@ -50,20 +51,23 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-def page_geometry(kv_pages: torch.Tensor, head_dim: int) -> tuple[int, int, int]:
-    """(P, page_size, C) of a v2 ``[P, pg, 2*Hkv, D]`` or v3 ``[P, pg, groups, packing, Dp]`` page buffer.
+def page_geometry(kv_pages: torch.Tensor, head_dim: int) -> tuple[int, int, int, int]:
+    """(P, page_size, C, Dp) of a v2 ``[P, pg, 2*Hkv, D]`` or v3 ``[P, pg, groups, packing, Dp]`` page buffer.
 
-    Both have token rows of ``C`` combined heads of ``head_dim`` elements, K at even and V at odd
-    combined heads; the v3 shape for ``head_dim == 64`` packs K_h|V_h into one 128-wide row, which
-    is the same bytes.  A padded head (``Dp > head_dim`` otherwise) is not supported.
+    Both have token rows of ``C`` combined heads of ``Dp`` stored elements, K at even and V at odd
+    combined heads.  The v3 shape for ``head_dim == 64`` packs K_h|V_h into one 128-wide row, which
+    is the same bytes as rows of 64 (``Dp = 64``); any other head size is stored padded to a multiple
+    of 128 (easydel/caching/ragged_page/cache.py:640-647), ``Dp > head_dim`` with zeros in the padding.
     """
     if kv_pages.ndim not in (4, 5):
         raise ValueError(f"kv_pages must be 4-D (v2) or 5-D (v3), got shape {tuple(kv_pages.shape)}")
     stored = kv_pages.shape[-1]
-    if stored != head_dim and not (head_dim == 64 and stored == 128):
-        raise NotImplementedError(f"padded head storage (stored {stored}, head_dim {head_dim}) is not supported")
+    if stored < head_dim:
+        raise ValueError(f"kv_pages rows hold {stored} elements, fewer than head_dim {head_dim}")
+    if head_dim == 64 and stored == 128 and kv_pages.ndim == 5:
+        stored = 64  # K_h | V_h share one 128-wide row
     per_token = math.prod(kv_pages.shape[2:])
-    return kv_pages.shape[0], kv_pages.shape[1], per_token // head_dim
+    return kv_pages.shape[0], kv_pages.shape[1], per_token // stored, stored
 
 
 def workspace_bytes(T, S, M, page_size, Hq, Hkv, D, q_dtype: torch.dtype, kv_dtype: torch.dtype) -> int:
@@ -107,7 +111,7 @@ def page_scatter_ragged(key, value, kv_pages, context_lens, block_tables, query_
     if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
         raise TypeError(f"key/value dtype {key.dtype}/{value.dtype} must equal the cache dtype {kv_pages.dtype}")
     T, Hkv, D = key.shape
-    P, pg, C = page_geometry(kv_pages, D)
+    P, pg, C, Dp = page_geometry(kv_pages, D)
     S = context_lens.shape[0]
     M = block_tables.numel() // S
     if T == 0:
@@ -117,7 +121,7 @@ def page_scatter_ragged(key, value, kv_pages, context_lens, block_tables, query_
         _lib.check(lib.rpa_page_scatter_ragged(
             _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
             _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, key.element_size()))
+            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, Dp, C, key.element_size()))
     return kv_pages
 
 
@@ -130,7 +134,7 @@ def page_scatter_ragged_quantised(key, value, kv_pages, kv_scales, context_lens,
     if kv_pages.dtype not in (torch.float8_e4m3fn, torch.int8):
         raise TypeError(f"kv_pages must be float8_e4m3fn or int8 for the quantising write, got {kv_pages.dtype}")
     T, Hkv, D = key.shape
-    P, pg, C = page_geometry(kv_pages, D)
+    P, pg, C, Dp = page_geometry(kv_pages, D)
     if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
         raise ValueError(f"kv_scales must be float32 [P={P}, C={C}]")
     S = context_lens.shape[0]
@@ -142,7 +146,7 @@ def page_scatter_ragged_quantised(key, value, kv_pages, kv_scales, context_lens,
         _lib.check(lib.rpa_page_scatter_ragged_quantised(
             _stream(kv_pages), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"), _dev(kv_scales, "kv_scales"),
             _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
-            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, C, dtype_tag(key.dtype), dtype_tag(kv_pages.dtype)))
+            _i32(num_seqs, "num_seqs"), T, S, M, P, pg, Hkv, D, Dp, C, dtype_tag(key.dtype), dtype_tag(kv_pages.dtype)))
     return kv_pages, kv_scales
 
 
@@ -163,7 +167,7 @@ def _sinks(softmax_aux, num_q_heads: int, device):
 
 def _attn_common(query, kv_pages, context_lens, block_tables, num_kv_heads, softmax_scale, sliding_window, logits_soft_cap):
     T, Hq, D = query.shape
-    P, pg, C = page_geometry(kv_pages, D)
+    P, pg, C, Dp = page_geometry(kv_pages, D)
     S = context_lens.shape[0]
     if block_tables.numel() % S:
         raise ValueError("block_tables size is not a multiple of the number of sequence rows")
@@ -172,7 +176,7 @@ def _attn_common(query, kv_pages, context_lens, block_tables, num_kv_heads, soft
     scale = float(D) ** -0.5 if softmax_scale is None else float(softmax_scale)
     window = int(sliding_window) if sliding_window else 0
     cap = float(logits_soft_cap) if logits_soft_cap else 0.0
-    return T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap
+    return T, Hq, D, Dp, P, pg, C, S, M, Hkv, scale, window, cap
 
 
 def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *,
@@ -180,7 +184,7 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
                            num_kv_heads=None, softmax_aux=None, out=None):
     """Read-only ragged paged attention; returns ``[T, Hq, D]`` in the query dtype."""
     lib = _lib.load()
-    T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+    T, Hq, D, Dp, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
         query, kv_pages, context_lens, block_tables, num_kv_heads, softmax_scale, sliding_window, logits_soft_cap)
     if out is None:
         out = torch.empty_like(query)
@@ -190,7 +194,7 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
     for name, t in (("query", query), ("kv_pages", kv_pages), ("out", out)):
         _dev(t, name)
     aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
-    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, Dp, qd, kd)))
     scales_ptr = None
     if kv_scales is not None:
         if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
@@ -201,7 +205,7 @@ def ragged_paged_attention(query, kv_pages, context_lens, block_tables, query_st
             _stream(query), _dev(query, "query"), _dev(kv_pages, "kv_pages"), scales_ptr,
             _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
             _i32(num_seqs, "num_seqs"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-            T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
+            T, S, M, P, pg, Hq, Hkv, D, Dp, C, qd, kd, scale, window, cap, aux_ptr))
     return out
 
 
@@ -257,7 +261,7 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
     lib = _lib.load()
     if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
         raise TypeError(f"key/value dtype {key.dtype}/{value.dtype} must equal the cache dtype {kv_pages.dtype}")
-    T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+    T, Hq, D, Dp, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
         query, kv_pages, context_lens, block_tables, key.shape[1] if num_kv_heads is None else num_kv_heads,
         softmax_scale, sliding_window, logits_soft_cap)
     if out is None:
@@ -268,13 +272,13 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
     for name, t in (("query", query), ("key", key), ("value", value), ("kv_pages", kv_pages), ("out", out)):
         _dev(t, name)
     aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
-    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, Dp, qd, kd)))
     with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
         _lib.check(lib.rpa_ragged_paged_attention_v3(
             _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
             _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
             _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(), ws.numel(),
-            T, S, M, P, pg, Hq, Hkv, D, C, qd, kd, scale, window, cap, aux_ptr))
+            T, S, M, P, pg, Hq, Hkv, D, Dp, C, qd, kd, scale, window, cap, aux_ptr))
     return out, kv_pages
 
 
@@ -286,7 +290,7 @@ def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, 
     lib = _lib.load()
     if key.dtype != value.dtype or key.dtype not in (torch.float32, torch.bfloat16):
         raise TypeError(f"key/value must both be float32 or bfloat16, got {key.dtype}/{value.dtype}")
-    T, Hq, D, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+    T, Hq, D, Dp, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
         query, kv_pages, context_lens, block_tables, key.shape[1] if num_kv_heads is None else num_kv_heads,
         softmax_scale, sliding_window, logits_soft_cap)
     if kv_scales.dtype != torch.float32 or kv_scales.numel() != P * C:
@@ -299,13 +303,13 @@ def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, 
     for name, t in (("query", query), ("key", key), ("value", value), ("kv_pages", kv_pages), ("kv_scales", kv_scales), ("out", out)):
         _dev(t, name)
     aux, aux_ptr = _sinks(softmax_aux, Hq, query.device)
-    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, D, qd, kd)))
+    ws = _workspace(query.device, int(lib.rpa_attention_workspace_bytes(T, S, M, pg, Hq, Hkv, Dp, qd, kd)))
     with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
         _lib.check(lib.rpa_ragged_paged_attention_v3_quantised(
             _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
             _dev(kv_scales, "kv_scales"), _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"),
             _i32(query_start_loc, "query_start_loc"), _i32(distribution, "distribution"), _dev(out, "out"), ws.data_ptr(),
-            ws.numel(), T, S, M, P, pg, Hq, Hkv, D, C, qd, dtype_tag(key.dtype), kd, scale, window, cap, aux_ptr))
+            ws.numel(), T, S, M, P, pg, Hq, Hkv, D, Dp, C, qd, dtype_tag(key.dtype), kd, scale, window, cap, aux_ptr))
     return out, kv_pages, kv_scales
 
 

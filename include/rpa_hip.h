@@ -11,12 +11,22 @@
  * negative value is one of the RPA_ERR_* codes.  rpa_last_error() returns a thread-local,
  * human-readable description of the most recent failure on the calling thread.
  *
- * KV page layout (all entry points): kv_pages[P][page_size][C][D] elements, where combined
+ * The entry points keep no state between calls and may be called from any number of threads at
+ * once (device properties are cached per device; the knobs of rpa_hip_probe.h, for tests and
+ * measurement, belong to the thread that sets them).  HIP's current device must be the one the
+ * pointers live on.
+ *
+ * KV page layout (all entry points): kv_pages[P][page_size][C][Dp] elements, where combined
  * head 2h holds K of KV head h and 2h+1 holds V (reference: easydel/caching/ragged_page/
  * cache.py:719-726 for the v2 shape, :711-718 for the v3 shape, :954-973 for the K-even /
  * V-odd interleave).  The reference's v3 storage [P][page][groups][packing][Dp] has the same
  * bytes as [P][page][C = groups*packing][Dp]; for head_dim 64 it stores K_h|V_h in one
- * 128-wide row, which is again the same bytes as C = 2*Hkv rows of 64.  C >= 2*Hkv.
+ * 128-wide row, which is again the same bytes as C = 2*Hkv rows of Dp = 64.  C >= 2*Hkv.
+ * Dp >= D is the stored width of a head row: the reference pads head sizes that are neither 64
+ * nor a multiple of 128 up to the next multiple of 128 (cache.py:640-647: 80 / 96 / 112 -> 128,
+ * 192 -> 256); Dp = D without padding.  The write entry points store zeros in the padding and
+ * the attention over bf16 / 8-bit pages relies on finite values there (a pool that starts as
+ * zeros, as the reference's does, and is written through these entry points qualifies).
  */
 #ifndef RPA_HIP_H_
 #define RPA_HIP_H_
@@ -28,12 +38,14 @@
 extern "C" {
 #endif
 
-/* Element formats of q / out (F32, BF16) and of KV pages (all four). */
+/* Element formats of q / out (F32, BF16, F16) and of KV pages (all five). */
 typedef enum rpa_dtype {
   RPA_F32 = 0,
   RPA_BF16 = 1,
-  RPA_FP8_E4M3 = 2, /* OCP e4m3fn codes, value = code * kv_scales[page][combined head] */
-  RPA_INT8 = 3      /* signed 8-bit codes, value = code * kv_scales[page][combined head] */
+  RPA_FP8_E4M3 = 2, /* OCP e4m3fn codes; value = code * kv_scales[page][combined head], or the code's own value
+                       when no scales are passed (the reference's cast-only 8-bit cache, cache.py:143-158) */
+  RPA_INT8 = 3,     /* signed 8-bit codes, scaled likewise */
+  RPA_F16 = 4       /* IEEE half: served by the float32 kernel */
 } rpa_dtype;
 
 #define RPA_OK 0
@@ -78,7 +90,7 @@ int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32
  * block_tables[i][*]; K of head h goes to combined head 2h, V to 2h+1.
  *
  *   key, value    device, [T][Hkv][D] in the cache element type (elem_bytes each)
- *   kv_pages      device, [P][page_size][C][D], updated in place
+ *   kv_pages      device, [P][page_size][C][Dp], updated in place (elements D..Dp-1 of a written row become zero)
  *   block_tables  device, int32 [S][M] (the flattened [S*M] form is the same bytes)
  *   num_seqs      device, int32 [1]: number of live rows (pass distribution + 2 for v3 metadata)
  * Bit-exact.  Positions < 0 and padded tokens (t >= qsl[num_seqs]) are skipped.
@@ -86,7 +98,7 @@ int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32
 int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
                             const int32_t* context_lens, const int32_t* block_tables,
                             const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M,
-                            int P, int page_size, int Hkv, int D, int C, int elem_bytes);
+                            int P, int page_size, int Hkv, int D, int Dp, int C, int elem_bytes);
 
 /*
  * Page scatter, ragged form, into scaled 8-bit pages (RPA_FP8_E4M3 or RPA_INT8).  No counterpart in the
@@ -104,12 +116,16 @@ int rpa_page_scatter_ragged(rpa_stream_t stream, const void* key, const void* va
 int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, const void* value, void* kv_pages,
                                       float* kv_scales, const int32_t* context_lens, const int32_t* block_tables,
                                       const int32_t* query_start_loc, const int32_t* num_seqs, int T, int S, int M, int P,
-                                      int page_size, int Hkv, int D, int C, int src_dtype, int kv_dtype);
+                                      int page_size, int Hkv, int D, int Dp, int C, int src_dtype, int kv_dtype);
 
 /*
  * Bytes of scratch rpa_ragged_paged_attention needs for these static bounds (split-K
  * partial outputs and their running max / sum).  The caller owns the buffer (under XLA it
- * is an extra result of the custom call), 256-byte aligned.
+ * is an extra result of the custom call), 256-byte aligned.  D is the stored head width Dp when
+ * the pages are padded.  The figure is what lets every sequence and row tile be split as finely
+ * as the kernels would like; an attention call accepts any workspace that holds two partial
+ * slots (it reports RPA_ERR_WORKSPACE below that), lays the buffer out from the bytes it is
+ * given and splits less when they are fewer, so the two calls cannot disagree.
  */
 size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D,
                                      int q_dtype, int kv_dtype);
@@ -120,9 +136,10 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
  * easydel/operations/kernels/ragged_page_attention.py:281-313, and the attention half of
  * ragged_page_attention_v3 (:684-695, :732-746).
  *
- *   q             device, [T][Hq][D]          q_dtype in {RPA_F32, RPA_BF16}
- *   kv_pages      device, [P][page_size][C][D] kv_dtype
- *   kv_scales     device, float [P][C] or NULL; required for RPA_FP8_E4M3 / RPA_INT8 pages
+ *   q             device, [T][Hq][D]          q_dtype in {RPA_F32, RPA_BF16, RPA_F16}
+ *   kv_pages      device, [P][page_size][C][Dp] kv_dtype
+ *   kv_scales     device, float [P][C] or NULL; 8-bit pages only.  NULL with 8-bit pages: the codes are the values
+ *                 (scale 1), which is how the reference stores an fp8 cache (a bare cast, ragged_page_attention.py:570-580)
  *   context_lens  device, int32 [S]           tokens in the cache per sequence, new ones included
  *   block_tables  device, int32 [S][M]
  *   query_start_loc device, int32 [S+1]
@@ -144,7 +161,7 @@ int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* k
                                const float* kv_scales, const int32_t* context_lens,
                                const int32_t* block_tables, const int32_t* query_start_loc,
                                const int32_t* num_seqs, void* out, void* workspace, size_t workspace_bytes,
-                               int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int C,
+                               int T, int S, int M, int P, int page_size, int Hq, int Hkv, int D, int Dp, int C,
                                int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
                                float logits_soft_cap, const float* softmax_aux);
 
@@ -172,14 +189,15 @@ int rpa_unified_attention(rpa_stream_t stream, const void* q, const void* key_ca
  * Fused v3 form: rpa_page_scatter_ragged followed by rpa_ragged_paged_attention on the
  * same stream, pages updated in place (the reference returns (out, kv_pages) and the
  * caller stores the pages back, ragged_page_attention.py:747).  key/value must already be
- * in the cache element type (the reference casts them first, :570-580); kv_dtype must be
- * RPA_F32 or RPA_BF16 (scaled 8-bit pages have rpa_ragged_paged_attention_v3_quantised).
+ * in the cache element type (the reference casts them first, :570-580), whatever that type is:
+ * for an 8-bit cache they hold the cast codes, which are copied bit for bit and read back as
+ * their own values (scaled 8-bit pages have rpa_ragged_paged_attention_v3_quantised).
  */
 int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void* key, const void* value,
                                   void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
                                   const int32_t* query_start_loc, const int32_t* distribution, void* out,
                                   void* workspace, size_t workspace_bytes, int T, int S, int M, int P,
-                                  int page_size, int Hq, int Hkv, int D, int C, int q_dtype, int kv_dtype,
+                                  int page_size, int Hq, int Hkv, int D, int Dp, int C, int q_dtype, int kv_dtype,
                                   float softmax_scale, int sliding_window, float logits_soft_cap,
                                   const float* softmax_aux);
 
@@ -192,7 +210,7 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
                                             const int32_t* block_tables, const int32_t* query_start_loc,
                                             const int32_t* distribution, void* out, void* workspace,
                                             size_t workspace_bytes, int T, int S, int M, int P, int page_size, int Hq,
-                                            int Hkv, int D, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
+                                            int Hkv, int D, int Dp, int C, int q_dtype, int kv_src_dtype, int kv_dtype,
                                             float softmax_scale, int sliding_window, float logits_soft_cap,
                                   const float* softmax_aux);
 
@@ -244,46 +262,6 @@ int rpa_mla_page_scatter(rpa_stream_t stream, const void* keys_values, const voi
                          const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,
                          const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int kv_lora_rank,
                          int qk_rope_head_dim, int row_elems, int elem_bytes);
-
-/*
- * Measurement aid with no counterpart in the reference: copies `bytes` (a multiple of 16, both
- * pointers 16-byte aligned) with a plain vector copy kernel.  Profiling a known-size copy next to
- * the attention kernels gives the factor that turns raw HBM traffic counters into bytes.
- */
-int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t bytes);
-
-/*
- * Measurement aid with no counterpart in the reference: a read-only kernel that says what the memory system gives
- * a streaming reader.  `workgroups` workgroups of eight wavefronts (one per CU: each holds 96 KiB of LDS) read `src`
- * once, every wavefront its own contiguous share with 16-byte loads, `kib_in_flight_per_wave` (2, 4, 8, 16 or 32) KiB
- * of them in flight.  Returns the bytes the launch reads (the share of each wavefront is rounded down to whole rounds
- * of loads), 0 on bad arguments; time the launch with events on `stream`.  `sink` is one device word, never written in
- * practice.  The decode kernel's bandwidth is judged against this probe's at the same number of workgroups.
- */
-size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
-                      void* sink);
-
-/*
- * Tuning knobs (process-wide, read at call time).  Returns the previous value.
- *   "max_splits"     partial-output slots per sequence the decode kernel may use (2..256, 0 = sized
- *                    from the shapes); set it before sizing the workspace
- *   "decode_wgs"     persistent decode workgroups per KV-head group (0 = as many as are resident at once)
- *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
- *   "decode_pace"    1 (default): in the bf16 eight-wave decode kernel a wave that finds four or more of its workgroup's
- *                    tiles in flight pauses once (512 clocks) before issuing its own; 0: never
- *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
- *                    set it before sizing the workspace
- *   "prefill_dma"    1 (default): bf16 prefill tiles are loaded global -> LDS by the load unit where that kernel
- *                    applies (page_size % 32 == 0); 0: every prefill tile is staged through registers
- *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
- *                    the shapes); set it before sizing the workspace
- *   "mla_min_chunk"  fewest keys of such a chunk (rounded up to 64; 0 = default: 1024 at 64 heads and more, else 512)
- *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
- *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
- *                    1 = decode plan kernel, 2 = decode kernel, 4 = prefill / large-row kernel,
- *                    8 = merge (default 15)
- */
-int rpa_set_tunable(const char* name, int value);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,59 @@
+/*
+ * rpa_hip_probe.h -- test and measurement aids of librpa_hip.so, kept apart from the operator entry points of
+ * rpa_hip.h.  Nothing here has a counterpart in the reference and a serving runtime needs none of it.
+ */
+#ifndef RPA_HIP_PROBE_H_
+#define RPA_HIP_PROBE_H_
+
+#include "rpa_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/*
+ * Measurement aid with no counterpart in the reference: copies `bytes` (a multiple of 16, both
+ * pointers 16-byte aligned) with a plain vector copy kernel.  Profiling a known-size copy next to
+ * the attention kernels gives the factor that turns raw HBM traffic counters into bytes.
+ */
+int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t bytes);
+
+/*
+ * Measurement aid with no counterpart in the reference: a read-only kernel that says what the memory system gives
+ * a streaming reader.  `workgroups` workgroups of eight wavefronts (one per CU: each holds 96 KiB of LDS) read `src`
+ * once, every wavefront its own contiguous share with 16-byte loads, `kib_in_flight_per_wave` (2, 4, 8, 16 or 32) KiB
+ * of them in flight.  Returns the bytes the launch reads (the share of each wavefront is rounded down to whole rounds
+ * of loads), 0 on bad arguments; time the launch with events on `stream`.  `sink` is one device word, never written in
+ * practice.  The decode kernel's bandwidth is judged against this probe's at the same number of workgroups.
+ */
+size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
+                      void* sink);
+
+/*
+ * Knobs for tests and measurement.  They belong to the calling thread: a value set here is seen only by entry points
+ * the same thread calls afterwards (each call reads them once, when it starts), so threads that never call this function
+ * always run with the defaults.  Returns the previous value, -1 for an unknown name.
+ *   "max_splits"     partial-output slots per sequence the decode kernel may use (2..256, 0 = sized
+ *                    from the shapes); set it before sizing the workspace
+ *   "decode_wgs"     persistent decode workgroups per KV-head group (0 = as many as are resident at once)
+ *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
+ *   "decode_pace"    1 (default): in the bf16 eight-wave decode kernel a wave that finds four or more of its workgroup's
+ *                    tiles in flight pauses once (512 clocks) before issuing its own; 0: never
+ *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
+ *                    set it before sizing the workspace
+ *   "prefill_dma"    1 (default): bf16 prefill tiles are loaded global -> LDS by the load unit where that kernel
+ *                    applies (page_size % 32 == 0); 0: every prefill tile is staged through registers
+ *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
+ *                    the shapes); set it before sizing the workspace
+ *   "mla_min_chunk"  fewest keys of such a chunk (rounded up to 64; 0 = default: 1024 at 64 heads and more, else 512)
+ *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
+ *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
+ *                    1 = decode plan kernel, 2 = decode kernel, 4 = prefill / large-row kernel,
+ *                    8 = merge (default 15)
+ */
+int rpa_set_tunable(const char* name, int value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RPA_HIP_PROBE_H_ */

@@ -121,7 +121,19 @@ def f32_to_e4m3fn_bits(x: np.ndarray) -> np.ndarray:
 
 
 # dtype tags shared with the C ABI (include/rpa_hip.h: rpa_dtype)
-F32, BF16, FP8_E4M3, INT8 = 0, 1, 2, 3
+def cast_e4m3fn_ref(x: np.ndarray) -> np.ndarray:
+    """The plain cast to e4m3fn codes the reference applies to K/V headed for an fp8 cache
+    (``key.astype(kv_cache_dtype)``, operations/kernels/ragged_page_attention.py:570-580): round to nearest
+    even, and -- the format has no infinity -- whatever rounds beyond +-448 (|x| > 464; the tie at 464 goes to the
+    even code, 448) becomes NaN; nothing saturates.  jax's cast runs in ml_dtypes / XLA, neither present here: "parity unpinned" against them; pinned
+    against torch's CPU cast (same documented rule) in tests/test_oracle_formats.py."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    code = f32_to_e4m3fn_bits(x)
+    over = np.abs(x.astype(np.float64)) > 464.0  # 464 is halfway between 448 and the (absent) 480
+    return np.where(over, code | np.uint8(0x7F), code).astype(np.uint8)
+
+
+F32, BF16, FP8_E4M3, INT8, F16 = 0, 1, 2, 3, 4
 
 
 def decode_array(raw: np.ndarray, dtype_tag: int) -> np.ndarray:
@@ -134,6 +146,8 @@ def decode_array(raw: np.ndarray, dtype_tag: int) -> np.ndarray:
         return e4m3fn_bits_to_f32(raw).astype(np.float64)
     if dtype_tag == INT8:
         return np.asarray(raw, dtype=np.int8).astype(np.float64)
+    if dtype_tag == F16:
+        return np.asarray(raw, dtype=np.float16).astype(np.float64)
     raise ValueError(f"unknown dtype tag {dtype_tag}")
 
 

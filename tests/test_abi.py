@@ -1,4 +1,4 @@
-"""The C-ABI library loads and exports every symbol include/rpa_hip.h declares (no compute calls: no GPU here)."""
+"""The C-ABI library loads and exports every symbol include/rpa_hip.h and include/rpa_hip_probe.h declare (no compute calls: no GPU here)."""
 
 import ctypes
 import os
@@ -12,9 +12,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "rpa_hip.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(rpa_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in ("rpa_hip.h", "rpa_hip_probe.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(rpa_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_header_symbols_are_exported_and_bound():
@@ -33,26 +36,30 @@ def test_host_only_entry_points():
     assert re.fullmatch(r"\d+\.\d+\.\d+", lib.rpa_version().decode())
     # argument validation happens before any device work
     rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
-                                        4, 1, 1, 1, 16, 8, 3, 64, 6, 1, 1, 1.0, 0, 0.0, None)
+                                        4, 1, 1, 1, 16, 8, 3, 64, 64, 6, 1, 1, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"multiple of Hkv" in lib.rpa_last_error()
     rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
-                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 5, 1, 1.0, 0, 0.0, None)
+                                        4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 9, 1, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_UNSUPPORTED
+    a = 0x7000_0000_0000
+    rc = lib.rpa_ragged_paged_attention(None, None, None, a, None, None, None, None, None, None, 0,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"kv_scales" in lib.rpa_last_error()  # scales with 16-bit pages
     rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
-                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 2, 1.0, 0, 0.0, None)
-    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"kv_scales" in lib.rpa_last_error()
+                                        4, 1, 1, 1, 16, 8, 2, 96, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"Dp" in lib.rpa_last_error()  # stored rows narrower than the head
     with pytest.raises(_lib.RpaError):
         _lib.check(rc)
     # pointers are checked for null and alignment before anything is launched (the values below are never dereferenced)
     a = 0x7000_0000_0000
     rc = lib.rpa_ragged_paged_attention(None, a + 8, a, None, a, a, a, a, a, a, 1 << 20,
-                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+                                        4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 1, 1, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"16-byte aligned" in lib.rpa_last_error()
     rc = lib.rpa_ragged_paged_attention(None, a, a, None, a, a, a, a, a, a, 1 << 20,
-                                        4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 1, 1.0, 0, 0.0, a + 2)
+                                        4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 1, 1, 1.0, 0, 0.0, a + 2)
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"softmax_aux" in lib.rpa_last_error()
     rc = lib.rpa_ragged_paged_attention_v3(None, a, None, a, a, a, a, a, a, a, a, 1 << 20,
-                                           4, 1, 1, 1, 16, 8, 2, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+                                           4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 1, 1, 1.0, 0, 0.0, None)
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"null key" in lib.rpa_last_error()
     assert lib.rpa_page_scatter_slices(None, None, None, None, None, 0, 0, 0, 4, 16, 0) == 0  # empty input is a no-op
     assert lib.rpa_page_scatter_slices(None, None, None, None, None, 4, 4, 64, 0, 16, 0) == _lib.RPA_ERR_INVALID_ARGUMENT

@@ -18,7 +18,11 @@ def check(b, what, *, fused=True, softmax_aux=None, **kw):
     want, want_pages = mla_oracle(b, fused=fused, softmax_aux=softmax_aux, **kw)
     got, got_pages = run_gpu_mla(b, fused=fused, softmax_aux=softmax_aux, **kw)
     np.testing.assert_array_equal(got_pages, want_pages, err_msg=f"{what}: pages after the write")
-    return tl.assert_close(got, want, b, what)
+    # latent rows are N(0,1) in 512 dims and a row with one dominant key returns them: outputs beyond 4 do occur here
+    r = tl.assert_close(got, want, b, what, one_ulp_above_4=True)
+    if tl.last_widened:
+        print(f"  {tl.last_widened} element(s) with |want| >= 4 judged by one bf16 step instead of 2e-2", flush=True)
+    return r
 
 
 SCALE = (128 + 64) ** -0.5  # what the caller passes for DeepSeek-V3: (qk_nope_head_dim + qk_rope_head_dim) ** -0.5

@@ -58,5 +58,7 @@ def test_random_mla_batch(gpu, seed):
     want, want_pages = mla_oracle(b, fused=fused, softmax_aux=aux, **kw)
     got, got_pages = run_gpu_mla(b, fused=fused, softmax_aux=aux, **kw)
     np.testing.assert_array_equal(got_pages, want_pages, err_msg=f"{what}: pages after the call")
-    tl.assert_close(got, want, b, what)
+    tl.assert_close(got, want, b, what, one_ulp_above_4=True)
+    if tl.last_widened:
+        print(f"  {tl.last_widened} element(s) with |want| >= 4 judged by one bf16 step instead of 2e-2", flush=True)
     assert np.all(got[int(b.query_start_loc[b.n]):] == 0.0), "padded token rows must be written as zeros"

@@ -124,7 +124,8 @@ def test_quantised_view_is_read_through_scales(gpu):
     d = tl.device_batch(b, gpu)
     cfg = RaggedPagesCacheConfig.create(torch.float8_e4m3fn, num_hidden_layers=1, num_kv_heads=8, max_model_length=b.M * 64,
                                         kv_head_dim_size=128, page_size=64, num_pages=b.P)
-    view = RaggedPagesCacheView.init(cfg, device=gpu)
+    assert RaggedPagesCacheView.init(cfg, device=gpu).kv_scales is None  # the reference's fp8 cache: plain casts, no scales
+    view = RaggedPagesCacheView.init(cfg, device=gpu, scaled=True)
     assert tuple(view.kv_scales.shape) == (b.P, 16)
     view.kv_pages.copy_(d["kv_pages"].view(view.kv_pages.shape))
     view.kv_scales.copy_(d["kv_scales"])

@@ -98,7 +98,7 @@ def test_fused_quantised_v3_operation(gpu, kv_dtype):
     P = S * M + 1
     cfg = RaggedPagesCacheConfig.create(TORCH_KV[kv_dtype], num_hidden_layers=1, num_kv_heads=Hkv, max_model_length=M * pg,
                                         kv_head_dim_size=D, page_size=pg, num_pages=P)
-    view = RaggedPagesCacheView.init(cfg, device=gpu)
+    view = RaggedPagesCacheView.init(cfg, device=gpu, scaled=True)
     bt = _tables(rng, S, M, P)
     op = OperationRegistry.create("ragged_page_attention_v3", OperationMetadata())
     codes = np.zeros((P, pg, 2 * Hkv, D), np.uint8)

@@ -54,7 +54,9 @@ def test_random_batch(gpu, seed):
     what = f"seed {seed}: D{D} pg{page_size} {Hq}/{Hkv} kv{kv_dtype} ctx {ctx} q {q_lens} {sorted(kw)}"
     print(what, flush=True)
     got = tl.run_gpu_attention(b, **kw)
-    tl.assert_close(got, tl.oracle_out(b, **kw), b, what)
+    tl.assert_close(got, tl.oracle_out(b, **kw), b, what, one_ulp_above_4=True)
+    if tl.last_widened:
+        print(f"  {tl.last_widened} element(s) with |want| >= 4 judged by one bf16 step instead of 2e-2", flush=True)
     assert np.all(got[int(b.query_start_loc[b.n]):] == 0.0), "padded token rows must be written as zeros"
     same = tl.run_gpu_unified_attention(b, **kw)
     assert np.array_equal(got, same), "separate K and V pools must give the same bits"

@@ -157,13 +157,17 @@ def test_product_path_refuses_cpu_tensors():
 
 
 def test_page_geometry_views():
-    assert kernels.page_geometry(torch.empty((5, 64, 16, 128), dtype=torch.bfloat16), 128) == (5, 64, 16)
-    assert kernels.page_geometry(torch.empty((5, 64, 8, 2, 128), dtype=torch.bfloat16), 128) == (5, 64, 16)
-    assert kernels.page_geometry(torch.empty((5, 16, 2, 1, 128)), 64) == (5, 16, 4)  # v3 storage of head_dim 64
+    assert kernels.page_geometry(torch.empty((5, 64, 16, 128), dtype=torch.bfloat16), 128) == (5, 64, 16, 128)
+    assert kernels.page_geometry(torch.empty((5, 64, 8, 2, 128), dtype=torch.bfloat16), 128) == (5, 64, 16, 128)
+    assert kernels.page_geometry(torch.empty((5, 16, 2, 1, 128)), 64) == (5, 16, 4, 64)  # v3 storage of head_dim 64: K_h | V_h per row
+    # padded head storage (reference cache.py:640-647): head sizes 96 and 192 live in rows of 128 and 256
+    assert kernels.page_geometry(torch.empty((5, 16, 4, 2, 128), dtype=torch.bfloat16), 96) == (5, 16, 8, 128)
+    assert kernels.page_geometry(torch.empty((5, 16, 2, 4, 256), dtype=torch.float8_e4m3fn), 192) == (5, 16, 8, 256)
+    with pytest.raises(ValueError, match="fewer than head_dim"):
+        kernels.page_geometry(torch.empty((5, 16, 4, 2, 128), dtype=torch.bfloat16), 192)
+    assert kernels.dtype_tag(torch.float16) == 4
     with pytest.raises(NotImplementedError):
-        kernels.page_geometry(torch.empty((5, 16, 4, 2, 128), dtype=torch.bfloat16), 96)
-    with pytest.raises(NotImplementedError):
-        kernels.dtype_tag(torch.float16)
+        kernels.dtype_tag(torch.float64)
 
 
 def test_unified_attention_registry_requirements_and_config():

@@ -118,3 +118,19 @@ def test_quantised_write_places_tokens_like_the_plain_ragged_write():
     codes, _ = orc.page_scatter_ragged_quantised_ref(k, v, zero_codes, np.zeros((P, 2 * Hkv), np.float32), ctx, bt, qsl, [3], kv_dtype=orc.INT8)
     plain = orc.page_scatter_ragged_ref(k, v, np.zeros((P, pg, 2 * Hkv, D), np.float32), ctx, bt, qsl, [3])
     assert np.array_equal(codes.any(axis=(2, 3)), (plain != 0).any(axis=(2, 3)))
+
+
+def test_plain_e4m3fn_cast_matches_torch_incl_overflow_to_nan():
+    """The cast-only fp8 cache of the reference: round to nearest even, overflow -> NaN (no saturation)."""
+    import torch
+
+    rng = np.random.default_rng(5)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * np.float32(40.0),
+                        np.array([0.0, -0.0, 447.9, 448.0, 463.9, 464.0, 464.1, 480.0, 1e6, -464.0, -464.1, -1e9, np.inf, -np.inf,
+                                  2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -10, 2.0 ** -10 * 1.01], np.float32),
+                        orc.e4m3fn_decode_table()[np.arange(256) % 128 != 127]])
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    got = orc.cast_e4m3fn_ref(x)
+    nan_w, nan_g = (want & 0x7F) == 0x7F, (got & 0x7F) == 0x7F
+    assert np.array_equal(nan_w, nan_g) and nan_w.sum() == 7
+    assert np.array_equal(want[~nan_w], got[~nan_g])
