@@ -108,13 +108,22 @@ def make_batch(seed, ctx_lens, q_lens, *, Hq, Hkv, D, page_size, num_pages=None,
         b.kv_scales = scales
     else:
         raise ValueError(kv_dtype)
-    b.Dp = D
-    b.kv_dev = b.kv_raw  # what the device gets: the same pool, or its padded copy
-    if stored_dim is not None and stored_dim > D:
-        b.Dp = stored_dim
-        b.kv_dev = np.zeros((P, page_size, C, stored_dim), dtype=b.kv_raw.dtype)
-        b.kv_dev[..., :D] = b.kv_raw
+    b.Dp = stored_dim if stored_dim is not None and stored_dim > D else D
+    b.kv_dev = None  # set to hand the device a pool of the caller's making instead of device_pool(b)
     return b
+
+
+def device_pool(b) -> np.ndarray:
+    """The pool as the device gets it: ``kv_raw``, or -- padded head storage -- its copy in rows of ``Dp`` elements
+    with zeros behind the first D."""
+    if b.kv_dev is not None:
+        return b.kv_dev
+    if b.Dp == b.D:
+        return b.kv_raw
+    P, pg, C, D = b.kv_raw.shape
+    pool = np.zeros((P, pg, C, b.Dp), dtype=b.kv_raw.dtype)
+    pool[..., :D] = b.kv_raw
+    return pool
 
 
 def oracle_out(b, *, softmax_scale=None, sliding_window=None, logits_soft_cap=None, kv_val=None, softmax_aux=None):
@@ -153,7 +162,7 @@ def device_batch(b, device="cuda:0"):
 
     d = {
         "query": to_torch(b.q_raw, b.q_dtype, device),
-        "kv_pages": to_torch(b.kv_dev, b.kv_dtype, device),
+        "kv_pages": to_torch(device_pool(b), b.kv_dtype, device),
         "context_lens": torch.from_numpy(b.context_lens).to(device),
         "block_tables": torch.from_numpy(b.block_tables).to(device),
         "query_start_loc": torch.from_numpy(b.query_start_loc).to(device),
