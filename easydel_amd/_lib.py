@@ -44,6 +44,10 @@ SIGNATURES = {
         _c_int,
         [_c_vp] * 11 + [_c_sz] + [_c_int] * 12 + [_c_f32, _c_int, _c_f32, _c_vp],
     ),
+    "rpa_ragged_paged_attention_v3_static": (
+        _c_int,
+        [_c_vp] * 10 + [_c_int] * 12 + [_c_f32, _c_int, _c_f32, _c_vp],
+    ),
     "rpa_mla_ragged_paged_attention": (
         _c_int,
         [_c_vp] * 12 + [_c_sz] + [_c_int] * 11 + [_c_f32, _c_int, _c_f32, _c_vp],

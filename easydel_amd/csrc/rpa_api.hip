@@ -448,6 +448,57 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                         C, q_dtype, kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux, key, value);
 }
 
+// ---- the entry point that allocates nothing ----------------------------------------------------------------
+// Its workspace (decode plan, split-K partial slots, key-chunk partials) is this file-scope device array: every GPU
+// the library runs on holds its own copy, at its own address, until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress: the address is looked up once per device (with that device current) and
+// kept in scratch_ptr; kernels, like the ones behind the other entry points, get the pointer as an argument.
+static __device__ __align__(256) unsigned char scratch[RPA_STATIC_WORKSPACE_BYTES];
+
+static int static_workspace(void** ptr) {
+  static std::mutex mu;
+  static void* scratch_ptr[rpa::kMaxDevices];  // per device; null = not looked up yet
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return hip_fail((int)err, "hipGetDevice");
+  if (dev < 0 || dev >= rpa::kMaxDevices) return fail(RPA_ERR_UNSUPPORTED, "device %d: the static workspace is kept for devices 0..%d", dev, rpa::kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !p) return hip_fail(err != hipSuccess ? (int)err : (int)hipErrorInvalidSymbol, "hipGetSymbolAddress(scratch)");
+    scratch_ptr[dev] = p;
+  }
+  *ptr = scratch_ptr[dev];
+  return RPA_OK;
+}
+
+int rpa_ragged_paged_attention_v3_static(rpa_stream_t stream, const void* q, const void* key, const void* value,
+                                         void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
+                                         const int32_t* query_start_loc, const int32_t* distribution, void* out, int T,
+                                         int S, int M, int P, int page_size, int Hq, int Hkv, int D, int Dp, int C,
+                                         int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
+                                         float logits_soft_cap, const float* softmax_aux) {
+  const char* who = "rpa_ragged_paged_attention_v3_static";
+  // The smallest layout the attention accepts: plan + two partial slots of the decode-class tokens.  Checked here, from
+  // the shapes alone, so that a batch too large for the array is refused by name instead of as a generic workspace error.
+  if (T > 0 && S > 0 && M > 0 && page_size > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && D > 0 && Dp >= D) {
+    const int Dc = Dp;  // partial rows are at most the stored width
+    const int td = decode_token_bound(T, S, Hq, Hkv, rpa::decode_row_limit(T, S, Dc, kv_dtype));
+    const size_t need = 2 * (part_o_bytes(td, Hq, Dc) + part_ml_bytes(td, Hq)) + plan_bytes(S) + 256;
+    if (need > (size_t)RPA_STATIC_WORKSPACE_BYTES)
+      return fail(RPA_ERR_WORKSPACE, "%s: these shapes need at least %zu bytes of workspace, the built-in array holds %u; "
+                  "use rpa_ragged_paged_attention_v3 with a caller-owned workspace", who, need, (unsigned)RPA_STATIC_WORKSPACE_BYTES);
+  }
+  void* ws = nullptr;
+  if (T > 0) {
+    if (const int rc = static_workspace(&ws)) return rc;
+  }
+  return rpa_ragged_paged_attention_v3(stream, q, key, value, kv_pages, context_lens, block_tables, query_start_loc, distribution,
+                                       out, ws, RPA_STATIC_WORKSPACE_BYTES, T, S, M, P, page_size, Hq, Hkv, D, Dp, C, q_dtype,
+                                       kv_dtype, softmax_scale, sliding_window, logits_soft_cap, softmax_aux);
+}
+
 int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, const void* key, const void* value,
                                             void* kv_pages, float* kv_scales, const int32_t* context_lens,
                                             const int32_t* block_tables, const int32_t* query_start_loc,

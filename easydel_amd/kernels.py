@@ -282,6 +282,35 @@ def ragged_paged_attention_v3(query, key, value, kv_pages, context_lens, block_t
     return out, kv_pages
 
 
+def ragged_paged_attention_v3_static(query, key, value, kv_pages, context_lens, block_tables, query_start_loc, distribution, *,
+                                     softmax_scale=None, sliding_window=None, logits_soft_cap=None, num_kv_heads=None,
+                                     softmax_aux=None, out):
+    """``ragged_paged_attention_v3`` through the entry point that allocates nothing: the caller passes ``out``, the
+    scratch memory is the library's built-in per-GPU array (64 MiB; larger needs raise ``RpaError``).  Calls that
+    overlap on one GPU share that array and race."""
+    lib = _lib.load()
+    if key.dtype != kv_pages.dtype or value.dtype != kv_pages.dtype:
+        raise TypeError(f"key/value dtype {key.dtype}/{value.dtype} must equal the cache dtype {kv_pages.dtype}")
+    T, Hq, D, Dp, P, pg, C, S, M, Hkv, scale, window, cap = _attn_common(
+        query, kv_pages, context_lens, block_tables, key.shape[1] if num_kv_heads is None else num_kv_heads,
+        softmax_scale, sliding_window, logits_soft_cap)
+    if T == 0:
+        return out, kv_pages
+    qd, kd = dtype_tag(query.dtype), dtype_tag(kv_pages.dtype)
+    aux_ptr = None
+    if softmax_aux is not None:  # no conversion here: that would allocate
+        if softmax_aux.dtype != torch.float32 or tuple(softmax_aux.shape) != (Hq,):
+            raise ValueError(f"softmax_aux must be float32 [{Hq}] for the call that allocates nothing")
+        aux_ptr = _dev(softmax_aux, "softmax_aux")
+    with torch.cuda.device(query.device):  # the library queries and launches on HIP's current device
+        _lib.check(lib.rpa_ragged_paged_attention_v3_static(
+            _stream(query), _dev(query, "query"), _dev(key, "key"), _dev(value, "value"), _dev(kv_pages, "kv_pages"),
+            _i32(context_lens, "context_lens"), _i32(block_tables, "block_tables"), _i32(query_start_loc, "query_start_loc"),
+            _i32(distribution, "distribution"), _dev(out, "out"), T, S, M, P, pg, Hq, Hkv, D, Dp, C, qd, kd, scale, window, cap,
+            aux_ptr))
+    return out, kv_pages
+
+
 def ragged_paged_attention_v3_quantised(query, key, value, kv_pages, kv_scales, context_lens, block_tables,
                                         query_start_loc, distribution, *, softmax_scale=None, sliding_window=None,
                                         logits_soft_cap=None, num_kv_heads=None, softmax_aux=None, out=None):

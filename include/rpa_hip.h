@@ -202,6 +202,25 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
                                   const float* softmax_aux);
 
 /*
+ * rpa_ragged_paged_attention_v3 for callers that cannot allocate or hand over scratch memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same operands and
+ * results; the split-K partials and the decode plan live in a 64 MiB device array inside the library
+ * (RPA_STATIC_WORKSPACE_BYTES, one copy per GPU, held until the process ends) instead of a caller's workspace, and the
+ * call allocates nothing.  Shapes whose smallest layout (two partial slots + plan) exceeds the array are rejected with
+ * RPA_ERR_WORKSPACE; shapes that fit but would like more run with fewer partial slots / key chunks than a caller-sized
+ * workspace would allow.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race --
+ * serialise them.  Nothing in the array has to survive or be cleared between calls (each call writes what it reads).
+ */
+#define RPA_STATIC_WORKSPACE_BYTES (64u << 20)
+int rpa_ragged_paged_attention_v3_static(rpa_stream_t stream, const void* q, const void* key, const void* value,
+                                         void* kv_pages, const int32_t* context_lens, const int32_t* block_tables,
+                                         const int32_t* query_start_loc, const int32_t* distribution, void* out, int T,
+                                         int S, int M, int P, int page_size, int Hq, int Hkv, int D, int Dp, int C,
+                                         int q_dtype, int kv_dtype, float softmax_scale, int sliding_window,
+                                         float logits_soft_cap, const float* softmax_aux);
+
+/*
  * Fused v3 form over scaled 8-bit pages: rpa_page_scatter_ragged_quantised followed by
  * rpa_ragged_paged_attention on the same stream; pages and scales updated in place.  key/value in kv_src_dtype.
  */
