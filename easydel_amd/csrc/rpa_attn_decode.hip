@@ -24,6 +24,7 @@
 #include <atomic>
 #include <type_traits>
 
+#include "rpa_attn_decode_dma.h"
 #include "rpa_mfma.h"
 
 namespace rpa {
@@ -572,9 +573,18 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   }
 }
 
+// The kernel that serves these template arguments: the LDS-direct one where it applies and the call asks for it.
+template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
+static bool use_dma(const AttnParams& p) {
+  if constexpr (KVT == RPA_BF16 && WPB >= 4 && TT == (D == 64 ? 32 : 16)) return p.decode_dma != 0 && decode_dma_supported(p);
+  else return false;
+}
+
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 static int launch_rb(hipStream_t stream, AttnParams p) {
   constexpr bool PACE = ElemBytes<KVT>::v == 2 && WPB == 8;
+  constexpr int TTD = D == 64 ? 32 : 16;  // keys per tile of the LDS-direct kernel (its pages hold multiples of 64 tokens)
+  const bool dma = use_dma<D, KVT, TT, WPB, CAP, RB>(p);
   // persistent grid: as many workgroups as are resident at once, per KV-head group.  The figure belongs to the device
   // the call runs on; it is looked up once per device and kernel (a racing first call computes the same value).
   static std::atomic<int> resident_of[kMaxDevices];
@@ -587,7 +597,7 @@ static int launch_rb(hipStream_t stream, AttnParams p) {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return (int)hipGetLastError();
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<D, KVT, TT, WPB, CAP, RB, PACE>, 64 * WPB, 0) != hipSuccess)
       return (int)hipGetLastError();
-    resident = max(1, cus * max(1, per_cu));
+    resident = max(1, cus * max(1, per_cu));  // one workgroup per CU for either kernel (registers here, LDS there)
     resident_of[dev].store(resident, std::memory_order_relaxed);
   }
   const int head_groups = (p.Hkv + WPB - 1) / WPB;
@@ -596,8 +606,15 @@ static int launch_rb(hipStream_t stream, AttnParams p) {
   n_wg = max(1, min(n_wg, kMaxDecodeWgs));
   p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + (p.T + kScatterTokensPerBlock - 1) / kScatterTokensPerBlock : 1), dim3(1024), 0, stream, p);
-  if (p.decode_which & 2)
+  if (p.decode_which & 2) {
+    if constexpr (KVT == RPA_BF16 && WPB >= 4 && TT == TTD) {
+      if (dma) {
+        hipLaunchKernelGGL((attn_decode_dma_kernel<D, TTD, WPB, CAP, RB>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+        return (int)hipGetLastError();
+      }
+    }
     hipLaunchKernelGGL((attn_decode_kernel<D, KVT, TT, WPB, CAP, RB, PACE>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+  }
   return (int)hipGetLastError();
 }
 

@@ -24,18 +24,6 @@
 
 namespace rpa {
 
-// One LDS DMA of 1 KiB: every lane fetches 16 bytes from base + voff; lane L's bytes land at LDS byte
-// address lds_addr + 16 L.  (An instruction offset would move the LDS address as well, so none is used.)
-__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
-}
-
-// Waits until at most N of this wave's loads are in flight, then joins the workgroup barrier.
-template <int N>
-__device__ __forceinline__ void wait_loads_and_barrier() {
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
-}
-
 template <int D, int NW, int RB, bool CAP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams p) {
   constexpr int TT = 32;                 // keys per tile

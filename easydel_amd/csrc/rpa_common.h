@@ -60,6 +60,7 @@ struct AttnParams {
   int pre_max_chunks;  // chunks the prefill partial buffers hold; 1 = never split
   int decode_sync;   // decode workgroups re-align their waves with a barrier every this many tiles (power of two), 0 = never
   int decode_pace;   // 0: the decode kernel never pauses a wave (see PACE there); default 1
+  int decode_dma;    // 1: bf16 decode tiles go global -> LDS directly where that kernel applies; 0: always through registers
   int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel
   int prefill_dma;   // 1: bf16 prefill tiles go global -> LDS directly where that kernel applies; 0: always through registers
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row

@@ -86,6 +86,26 @@ __device__ __forceinline__ float xor32_max(float v) {
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
+// One LDS DMA of 1 KiB (global_load_lds_dwordx4): every lane fetches 16 bytes from base + voff; lane L's bytes land at
+// LDS byte address lds_addr + 16 L.  (An instruction offset would move the LDS address as well, so none is used.)
+// Issued through inline assembly: the compiler neither tracks these loads nor orders its own waits around them, the
+// kernels that use them state their waits themselves (wait_loads).
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
+// Waits until at most N of this wave's vector-memory loads are in flight (they complete in issue order).
+template <int N>
+__device__ __forceinline__ void wait_loads() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// ... and then joins the workgroup barrier.
+template <int N>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
 // tanh through the hardware exp2: tanh(x) = 1 - 2 / (exp(2x) + 1).  Good to ~1e-6 relative, far inside
 // the bf16 tolerance of the MFMA kernels (the fp32 kernel uses tanhf).
 __device__ __forceinline__ float fast_tanh(float x) {

@@ -39,6 +39,9 @@ size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int wo
  *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
  *   "decode_pace"    1 (default): in the bf16 eight-wave decode kernel a wave that finds four or more of its workgroup's
  *                    tiles in flight pauses once (512 clocks) before issuing its own; 0: never
+ *   "decode_dma"     which bf16 decode batches (pages of a multiple of 64 tokens, four or more KV heads) run on the
+ *                    LDS-direct decode kernel, two tiles in flight per wave: -1 (default) those of head size 256,
+ *                    where it measured faster; 0 none; 1 all; 2 all, with one tile in flight
  *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
  *                    set it before sizing the workspace
  *   "prefill_dma"    1 (default): bf16 prefill tiles are loaded global -> LDS by the load unit where that kernel
