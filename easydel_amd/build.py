@@ -25,6 +25,7 @@ SOURCES = [
     "rpa_attn_decode.hip",
     "rpa_attn_prefill.hip",
     "rpa_attn_prefill_dma.hip",
+    "rpa_attn_prefill_dma8.hip",
     "rpa_attn_merge.hip",
     "rpa_mla.hip",
 ]

@@ -364,6 +364,7 @@ bool prefill_supported(const AttnParams& p) { return decode_supported(p); }
 
 int launch_attn_prefill(hipStream_t stream, const AttnParams& p) {
   if (p.prefill_dma && prefill_dma_supported(p)) return launch_attn_prefill_dma(stream, p);
+  if (p.prefill_dma && prefill_dma8_supported(p)) return launch_attn_prefill_dma8(stream, p);
   switch (p.kv_dtype) {
     case RPA_BF16: return launch_kvt<RPA_BF16>(stream, p);
     case RPA_FP8_E4M3: return launch_kvt<RPA_FP8_E4M3>(stream, p);

@@ -263,5 +263,7 @@ bool decode_supported(const AttnParams& p);
 int decode_row_limit(int T, int S, int D, int kv_dtype);
 bool prefill_supported(const AttnParams& p);
 bool prefill_dma_supported(const AttnParams& p);
+int launch_attn_prefill_dma8(hipStream_t stream, const AttnParams& p);  // 8-bit pages: codes loaded straight into LDS, widened there
+bool prefill_dma8_supported(const AttnParams& p);
 
 }  // namespace rpa

@@ -182,6 +182,18 @@ def llama_long_prefill(seed: int = 0, n_seqs: int = 8, q_len: int = 2048, num_pa
                     block_tables=_tables(rng, ctx, 64, num_pages, 576), softmax_scale=128.0 ** -0.5)
 
 
+def quantised_long_prefill(seed: int = 0, kv_dtype: str = "fp8", n_seqs: int = 4, q_len: int = 2048, num_pages: int = 2000) -> Workload:
+    """Not one of the five benchmark shapes: chunked prefill over scaled 8-bit pages at the heads of the quantised decode
+    configuration (40 query heads, 8 KV heads, head size 128, 64-token pages): ``n_seqs`` chunks of ``q_len`` tokens
+    appended to 8192..16384 tokens of context.  Used to measure the 8-bit prefill kernel."""
+    rng = np.random.default_rng(seed)
+    prior = rng.integers(8192 - q_len, 16385 - q_len, size=n_seqs)
+    ctx = (prior + q_len).astype(np.int32)
+    return Workload(f"Qwen2.5-32B-shaped {kv_dtype}-KV chunked prefill (tuning shape)", Hq=40, Hkv=8, D=128, page_size=64,
+                    num_pages=num_pages, max_pages_per_seq=256, context_lens=ctx, q_lens=np.full(n_seqs, q_len, dtype=np.int32),
+                    block_tables=_tables(rng, ctx, 64, num_pages, 256), kv_dtype=kv_dtype, softmax_scale=128.0 ** -0.5)
+
+
 # ---- device side ---------------------------------------------------------------------------------
 
 

@@ -14,9 +14,11 @@ from rpa_testlib import BF16, F16, F32, FP8, orc
 pytestmark = pytest.mark.gpu
 
 
-def _check(b, what, **kw):
+def _check(b, what, above_4=False, **kw):
     got = tl.run_gpu_attention(b, **kw)
-    mx, mean = tl.assert_close(got, tl.oracle_out(b, **kw), b, what)
+    mx, mean = tl.assert_close(got, tl.oracle_out(b, **kw), b, what, one_ulp_above_4=above_4)
+    if tl.last_widened:
+        print(f"  {tl.last_widened} element(s) with |want| >= 4 judged by one bf16 step instead of 2e-2", flush=True)
     print(f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
     return got
 
@@ -230,3 +232,37 @@ def test_rows_before_position_zero_are_zeros_on_every_kernel(gpu, kv_dtype, dma)
     assert not want[:300].any() and not want[401:405].any()
     tl.assert_close(got, want, b, "rows before position 0")
     assert not got[:300].any() and not got[401:405].any()
+
+
+# ---- 8-bit pages on the LDS-direct prefill pipeline ------------------------------------------------------------------
+@pytest.mark.parametrize("kv_dtype", [FP8, tl.INT8])
+@pytest.mark.parametrize("D,page_size,Hq,Hkv", [(128, 64, 32, 8), (256, 32, 8, 4), (128, 128, 40, 8)])
+def test_8bit_prefill_on_the_lds_direct_pipeline(gpu, kv_dtype, D, page_size, Hq, Hkv):
+    """Chunked prefill over scaled 8-bit pages: the kernel that loads codes straight into LDS and widens them there,
+    against the oracle and against the register-staged kernel; with a window whose left edge falls inside a tile, a
+    soft cap, a row tile split over key chunks, and NaN codes in the slots past the context."""
+    b = tl.make_batch(400 + D + page_size, [3000, 700, 9300, 40], [300, 1, 520, 40], Hq=Hq, Hkv=Hkv, D=D, page_size=page_size,
+                      kv_dtype=kv_dtype, pad_rows=1, pad_tokens=3)
+    if kv_dtype == FP8:  # slots past each context hold NaN codes: nobody may read them as data
+        for i, c in enumerate(b.context_lens[:b.n]):
+            if c % page_size:
+                b.kv_raw[b.block_tables[i, c // page_size], c % page_size:] = 0x7F
+    for kw in ({}, dict(sliding_window=777, logits_soft_cap=30.0)):
+        # (scales up to 2 on N(0,1) codes: rows that see a handful of keys return values beyond 4, where a bf16 result
+        # cannot keep 2e-2)
+        got = _check(b, f"8-bit prefill kv{kv_dtype} D{D} pg{page_size} {sorted(kw)}", above_4=True, **kw)
+        prev = _lib.set_tunable("prefill_dma", 0)
+        try:
+            staged = tl.run_gpu_attention(b, **kw)
+        finally:
+            _lib.set_tunable("prefill_dma", prev)
+        tl.assert_close(staged, tl.oracle_out(b, **kw), b, "register-staged kernel")
+        # (the two kernels round V differently -- bf16(code x scale) here, code x scale in float32 there -- so they
+        # agree with each other only as closely as each agrees with the oracle)
+        assert np.abs(got - staged)[tl.valid_rows(b)].max() <= 2 * tl.TOL_BF16_MAX
+    prev = _lib.set_tunable("prefill_chunks", 8)
+    try:
+        b2 = tl.make_batch(401 + D, [20000], [200], Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype)
+        _check(b2, "8-bit prefill, row tiles split over key chunks", above_4=True)
+    finally:
+        _lib.set_tunable("prefill_chunks", prev)
