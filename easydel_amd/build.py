@@ -75,5 +75,26 @@ def build_library(verbose: bool = True, extra_flags: list[str] | None = None, jo
     return LIB_PATH
 
 
+def build_ffi(verbose: bool = True) -> Path | None:
+    """Compile csrc/rpa_ffi.cc (the XLA FFI handlers over the C ABI) into lib/librpa_ffi.so.  It needs jaxlib's
+    ``xla/ffi/api`` headers: where ``jax.ffi`` does not import, nothing is built and None is returned."""
+    try:
+        import jax.ffi as jax_ffi
+    except Exception:  # jax is not installed on this host
+        if verbose:
+            print("jax.ffi is not importable here: librpa_ffi.so is not built")
+        return None
+    out = OUT_DIR / "librpa_ffi.so"
+    cmd = [_hipcc(), "-shared", "-fPIC", "-std=c++17", "-O2", f"-I{jax_ffi.include_dir()}", str(CSRC / "rpa_ffi.cc"),
+           f"-L{OUT_DIR}", "-lrpa_hip", "-Wl,-rpath,$ORIGIN", "-o", str(out)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on rpa_ffi.cc:\n{res.stderr[-6000:]}")
+    if verbose:
+        print(f"built {out}")
+    return out
+
+
 if __name__ == "__main__":
     build_library(extra_flags=sys.argv[1:])
+    build_ffi()
