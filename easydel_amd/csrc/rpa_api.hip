@@ -93,10 +93,12 @@ int device_cus() {
   return cus;
 }
 
-// How a prefill row tile's key range is cut into chunks (each a workgroup of its own, merged afterwards).
-// Cutting pays when a batch holds few row tiles (a couple of long prompts): it fills the chip and evens out the
-// workgroups' lengths.  It costs a float32 partial per chunk and row, written and read back by the merge, so a batch
-// whose bounds already allow many times more row tiles than workgroups fit on the chip is not cut at all.
+// How many chunks a prefill row tile's key range may be cut into (each a workgroup of its own, merged afterwards),
+// and, when the caller fixed that number, the keys of one chunk.  Cutting pays when a batch holds few row tiles (a
+// couple of long prompts): it fills the chip and evens out the workgroups' lengths.  It costs a float32 partial per
+// chunk and row, written and read back by the merge, so a batch whose bounds already allow many times more row tiles
+// than workgroups fit on the chip is not cut at all.  Otherwise this only sizes the partial buffers: the plan kernel
+// picks the chunk length from the lengths of the batch it finds on the device.
 void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int* chunk_keys, int* max_chunks) {
   const long span = (long)M * page_size;
   int chunks = g_tun.prefill_chunks > 0 ? g_tun.prefill_chunks : rpa::kMaxPrefillChunks;
@@ -104,15 +106,13 @@ void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, i
   if (g_tun.prefill_chunks <= 0 && Hkv > 0) {
     const long row_tiles = ((long)T * (Hq / Hkv) / rpa::kPrefillRows + S) * Hkv;  // the prefill grid's bound without cutting
     const int cus = device_cus();
-    if (cus > 0) {  // about eight units per CU fill the chip evenly; more chunks than that only add partials
-      const long want = (8L * cus + row_tiles - 1) / row_tiles;
-      if (want < chunks) chunks = (int)(want < 1 ? 1 : want);
-    }
+    if (cus > 0 && row_tiles >= 8L * cus) chunks = 1;  // eight units per CU even out by themselves
   }
   const size_t per = part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq);
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   long keys = (span + chunks - 1) / chunks;
-  if (keys < 8192) keys = 8192;
+  const long min_keys = g_tun.prefill_chunks > 0 ? 8192 : rpa::kMinPrefillChunk;
+  if (keys < min_keys) keys = min_keys;
   keys = (keys + 63) & ~63L;
   chunks = (int)((span + keys - 1) / keys);
   if (chunks < 1) chunks = 1;
@@ -371,15 +371,18 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     if (!workspace || usable < 2 * (po + pml))
       return fail(RPA_ERR_WORKSPACE, "%s: workspace %zu bytes < %zu needed for two partial slots", who,
                   workspace_bytes, 2 * (po + pml) + pb + 256);
-    if (usable < pre + 2 * (po + pml)) {  // a small workspace: prefill rows are not split over keys
-      pre = 0;
-      pre_chunks = 1;
+    if (usable < pre + 2 * (po + pml)) {  // a small workspace: prefill rows are split into fewer chunks, or not at all
+      pre_chunks = (int)((usable - 2 * (po + pml)) / (pre_po + pre_pml));
+      if (pre_chunks < 2) pre_chunks = 1;
+      pre = pre_chunks > 1 ? (size_t)pre_chunks * (pre_po + pre_pml) : 0;
     }
     usable -= pre;
     if ((size_t)splits * (po + pml) > usable) splits = (int)(usable / (po + pml));
     p.max_splits = splits;
     p.pre_chunk = pre_keys;
     p.pre_max_chunks = pre_chunks;
+    p.pre_auto = tun.prefill_chunks <= 0 ? 1 : 0;
+    p.pre_slots = device_cus() * (Dc <= 128 ? 2 : 1);  // resident workgroups of the large-row kernels
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     p.plan = (int32_t*)base;
     p.part_o = (float*)(base + pb);

@@ -495,9 +495,15 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   const int S = p.S, tid = threadIdx.x;
   const int per = (S + 1023) / 1024;
   const int i0 = min(S, tid * per), i1 = min(S, i0 + per);
-  __shared__ int s_large, s_merge;
+  __shared__ int s_large, s_merge, s_reach, s_span_min, s_span_max, s_tiles;
+  __shared__ unsigned long long s_work;
   if (tid == 0) {
     s_large = 0;
+    s_reach = 0;
+    s_work = 0;
+    s_span_min = 0x7fffffff;
+    s_span_max = 0;
+    s_tiles = 0;
     // Does the merge kernel have anything to do?  Rows of padded tokens to zero ...
     const int n_live = live_rows(p);
     s_merge = (n_live <= 0 || p.qsl[0] > 0 || p.qsl[n_live] < p.T) ? 1 : 0;
@@ -507,24 +513,38 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     const SeqPlan sp = seq_plan(p, i);
     toks = 0;
     if (sp.live && !sp.small_rows) s_large = 1;  // benign race: every writer stores 1
-    // ... rows of sequences with tokens but no context to zero, partial rows of the decode kernel (any sequence of its
-    // class may be cut by a span boundary), or row tiles of the large-row kernel cut into key chunks (a bound on the
-    // keys one tile visits, not the exact count: a flag that is set without need only costs the merge kernel's look)
-    if (i < live_rows(p) && sp.q_len > 0) {
-      if (!sp.live || sp.small_rows) s_merge = 1;
-      else if (p.pre_max_chunks > 1) {
-        const int reach = p.window > 0 ? min(sp.ctx, p.window + kPrefillRows / p.group + 64) : sp.ctx;
-        if (reach > p.pre_chunk) s_merge = 1;
-      }
-    }
+    // ... rows of sequences with tokens but no context to zero, or partial rows of the decode kernel (any sequence of
+    // its class may be cut by a span boundary); row tiles of the large-row kernel cut into key chunks are added below
+    if (i < live_rows(p) && sp.q_len > 0 && (!sp.live || sp.small_rows)) s_merge = 1;
     if (!sp.live || !sp.small_rows) return 0;
     toks = sp.q_len;
     return (sp.hi - sp.lo + 63) & ~63;
   };
   int sum = 0, tsum = 0, toks;
+  unsigned long long work = 0;  // keys the large-row kernel visits per KV head, over its row tiles (an estimate)
+  int reach = 0;                // a bound on the keys one of its row tiles visits
+  int span_min = 0x7fffffff, span_max = 0, n_tiles = 0;  // of a sequence's average row tile
   for (int i = i0; i < i1; ++i) {
     sum += span_of(i, toks);
     tsum += toks;
+    const SeqPlan sp = seq_plan(p, i);
+    if (sp.live && !sp.small_rows && sp.q_len > 0) {
+      const int tile_reach = p.window > 0 ? min(sp.ctx, p.window + kPrefillRows / p.group + 64) : sp.ctx;
+      const int tiles = (sp.q_len * p.group + kPrefillRows - 1) / kPrefillRows;
+      const int span = max(min(tile_reach, sp.ctx - sp.q_len / 2), 1);  // causal: half the new keys on average
+      work += (unsigned long long)tiles * (unsigned)span;
+      reach = max(reach, tile_reach);
+      span_min = min(span_min, span);
+      span_max = max(span_max, span);
+      n_tiles += tiles;
+    }
+  }
+  if (work) atomicAdd(&s_work, work);
+  if (reach) {
+    atomicMax(&s_reach, reach);
+    atomicMin(&s_span_min, span_min);
+    atomicMax(&s_span_max, span_max);
+    atomicAdd(&s_tiles, n_tiles);
   }
   part[tid] = sum;
   part2[tid] = tsum;
@@ -553,8 +573,29 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     q = max(max(q, q_min), 256);
     plan[0] = W;
     plan[1] = q;
+    // Keys per split-K chunk of the large-row kernel.  Its workgroups are dealt to the chip in grid order as others
+    // finish, so the last ones leave part of the chip idle for up to one chunk's time: about four chunks per resident
+    // workgroup keep that within a few percent.  Row tiles of (nearly) one length need no more than a whole number
+    // of rounds: they are cut into the fewest equal parts that give one, often not at all.
+    long long chunk = (long long)1 << 30;
+    if (p.pre_max_chunks > 1) {
+      chunk = p.pre_chunk;
+      if (p.pre_auto) {
+        const int slots = max(p.pre_slots, 1);
+        chunk = (long long)((s_work * (unsigned)p.Hkv / (unsigned)slots / 4 + 63) & ~63ull);
+        if (s_tiles > 0 && 4ll * s_span_max <= 5ll * s_span_min) {
+          const long long units = (long long)s_tiles * p.Hkv;
+          int parts = 1;  // rounds * slots <= 1.08 units * parts
+          while (parts < p.pre_max_chunks && ((units * parts + slots - 1) / slots) * slots * 100 > units * parts * 108) ++parts;
+          chunk = parts == 1 ? (long long)1 << 30 : ((s_reach + parts - 1) / parts + 63) & ~63;
+        }
+      }
+      chunk = min(max(chunk, (long long)kMinPrefillChunk), (long long)1 << 30);
+      if (2ll * s_reach >= 3 * chunk) s_merge = 1;  // a row tile is cut in two from 1.5 chunks on (prefill_tile)
+    }
     plan[2] = s_large;  // any sequence for the large-row (prefill) kernel?
     plan[3] = s_merge;  // anything for the merge kernel?
+    plan[4] = (int)chunk;
     s_Q = q;
   }
   __threadfence_block();

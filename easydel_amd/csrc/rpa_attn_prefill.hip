@@ -76,8 +76,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
   if (chunk >= pt.n_chunks) return;
   const int base_pos = sp.ctx - sp.q_len;  // position of the sequence's first query token
   const int vis_lo = pt.vis_lo;
-  const int kv_lo = pt.kv_lo + chunk * p.pre_chunk;
-  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : kv_lo + p.pre_chunk;
+  const int kv_lo = pt.kv_lo + chunk * pt.chunk_len;
+  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : kv_lo + pt.chunk_len;
   const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
   const bool single = pt.n_chunks == 1;
 

@@ -92,8 +92,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma8_kernel(AttnParam
   const int base_pos = sp.ctx - sp.q_len;  // position of the sequence's first query token
   const int vis_lo = pt.vis_lo;
   // the first tile must hold vis_lo, so that rows of it that nobody may see can borrow a visible row's address
-  const int kv_lo = max(pt.kv_lo + chunk * p.pre_chunk, vis_lo & ~(TT - 1));
-  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : pt.kv_lo + (chunk + 1) * p.pre_chunk;
+  const int kv_lo = max(pt.kv_lo + chunk * pt.chunk_len, vis_lo & ~(TT - 1));
+  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : pt.kv_lo + (chunk + 1) * pt.chunk_len;
   const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
   const bool single = pt.n_chunks == 1;
 

@@ -14,6 +14,7 @@ constexpr int kPlanHeader = 16;      // ints before the prefix array in the deco
 constexpr int kMaxDecodeWgs = 4096;  // persistent decode workgroups per KV-head group
 constexpr int kPrefillRows = 128;    // query rows (token x group head) one prefill workgroup owns
 constexpr int kMaxPrefillChunks = 8; // key chunks one prefill row tile may be split into
+constexpr int kMinPrefillChunk = 2048; // fewest keys of such a chunk
 constexpr int kMaxDevices = 64;      // devices of one process the per-device caches hold
 
 // Everything a kernel needs, passed by value.
@@ -36,7 +37,8 @@ struct AttnParams {
   float* pre_o;    // prefill split-K partials [pre_max_chunks][T][Hq][D]
   float* pre_ml;   // [pre_max_chunks][T][Hq][2]
   int32_t* plan;   // decode plan: [0] = W (flattened keys), [1] = Q (keys per workgroup), [2] = 1 if any sequence needs
-                   // the large-row kernel, then at kPlanHeader:
+                   // the large-row kernel, [3] = 1 if the merge kernel has work, [4] = keys per split-K chunk of the
+                   // large-row kernel, then at kPlanHeader:
                    // P[S+1] exclusive prefix of per-sequence key spans, R[S+1] exclusive prefix of
                    // decode-class query tokens (row of a token in the partial buffers), first_seq[n_wg]
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
@@ -56,8 +58,10 @@ struct AttnParams {
   int t_dec_max;     // static bound on decode-class query tokens = rows of one partial slot
   int n_wg;          // persistent decode workgroups per KV-head group
   int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
-  int pre_chunk;     // keys per prefill split-K chunk (multiple of 64)
+  int pre_chunk;     // keys per prefill split-K chunk (multiple of 64) when pre_auto is 0
   int pre_max_chunks;  // chunks the prefill partial buffers hold; 1 = never split
+  int pre_auto;        // 1: the plan kernel sets the chunk length from the batch's lengths; 0: pre_chunk as given
+  int pre_slots;       // workgroups of the prefill kernel the chip holds at once
   int decode_sync;   // decode workgroups re-align their waves with a barrier every this many tiles (power of two), 0 = never
   int decode_pace;   // 0: the decode kernel never pauses a wave (see PACE there); default 1
   int decode_dma;    // 1: bf16 decode tiles go global -> LDS directly where that kernel applies; 0: always through registers
@@ -108,9 +112,11 @@ __device__ __forceinline__ float with_sink(const AttnParams& p, int hq, float m_
 }
 
 // Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + kPrefillRows) of a sequence) must visit, kv_lo
-// rounded down to 64, and the number of split-K chunks the prefill kernel cuts it into.
+// rounded down to 64, and the split-K chunks the prefill kernel cuts it into: the range over the chunk length the
+// plan kernel chose (plan[4]), rounded to the nearest count the partial buffers hold, all chunks of one length (a
+// multiple of 64; the last one holds what is left), so that the workgroups of a sequence finish together.
 struct PrefillTile {
-  int kv_lo, kv_hi, vis_lo, n_chunks;
+  int kv_lo, kv_hi, vis_lo, n_chunks, chunk_len;
 };
 __device__ __forceinline__ PrefillTile prefill_tile(const AttnParams& p, const SeqPlan& sp, int R0) {
   PrefillTile t;
@@ -121,7 +127,13 @@ __device__ __forceinline__ PrefillTile prefill_tile(const AttnParams& p, const S
   t.vis_lo = (p.window > 0) ? max(base_pos + R0 / p.group - p.window + 1, 0) : 0;
   t.kv_lo = t.vis_lo & ~63;
   const int span = t.kv_hi - t.kv_lo;
-  t.n_chunks = span <= 0 ? 0 : min((span + p.pre_chunk - 1) / p.pre_chunk, p.pre_max_chunks);
+  const int target = p.plan[4];  // >= 64
+  t.n_chunks = span <= 0 ? 0 : min(max((int)(((int64_t)span + target / 2) / target), 1), p.pre_max_chunks);
+  t.chunk_len = target;
+  if (t.n_chunks > 1) {
+    t.chunk_len = ((span + t.n_chunks - 1) / t.n_chunks + 63) & ~63;
+    t.n_chunks = (span + t.chunk_len - 1) / t.chunk_len;  // rounding up to 64 may have emptied the last one
+  }
   return t;
 }
 
