@@ -46,6 +46,7 @@ def parse_args():
     ap.add_argument("--decode-wgs", type=int, default=0)
     ap.add_argument("--prefill-chunks", type=int, default=0)
     ap.add_argument("--decode-sync", type=int, default=-1)
+    ap.add_argument("--decode-dma", type=int, default=-1, help="LDS-direct decode kernel: -1 the library's choice, 0 never, 1 wherever built")
     ap.add_argument("--max-splits", type=int, default=0)
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
@@ -312,6 +313,8 @@ def main():
         _lib.set_tunable("decode_wgs", args.decode_wgs)
     if args.decode_sync >= 0:
         _lib.set_tunable("decode_sync", args.decode_sync)
+    if args.decode_dma >= 0:
+        _lib.set_tunable("decode_dma", args.decode_dma)
     if args.prefill_chunks:
         _lib.set_tunable("prefill_chunks", args.prefill_chunks)
     if args.max_splits:

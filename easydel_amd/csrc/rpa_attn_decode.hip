@@ -615,16 +615,19 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
 }
 
 // The kernel that serves these template arguments: the LDS-direct one where it applies and the call asks for it.
+// It is built for bf16 pages (every head size, four or eight waves) and for 8-bit pages at head size 128 with eight waves.
+template <int D, int KVT, int TT, int WPB>
+constexpr bool kHasDecodeDma = (KVT == RPA_BF16 && WPB >= 4 && TT == (D == 64 ? 32 : 16)) ||
+                               (ElemBytes<KVT>::v == 1 && D == 128 && TT == 32 && WPB == 8);
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 static bool use_dma(const AttnParams& p) {
-  if constexpr (KVT == RPA_BF16 && WPB >= 4 && TT == (D == 64 ? 32 : 16)) return p.decode_dma != 0 && decode_dma_supported(p);
+  if constexpr (kHasDecodeDma<D, KVT, TT, WPB>) return p.decode_dma != 0 && decode_dma_supported(p);
   else return false;
 }
 
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 static int launch_rb(hipStream_t stream, AttnParams p) {
   constexpr bool PACE = ElemBytes<KVT>::v == 2 && WPB == 8;
-  constexpr int TTD = D == 64 ? 32 : 16;  // keys per tile of the LDS-direct kernel (its pages hold multiples of 64 tokens)
   const bool dma = use_dma<D, KVT, TT, WPB, CAP, RB>(p);
   // persistent grid: as many workgroups as are resident at once, per KV-head group.  The figure belongs to the device
   // the call runs on; it is looked up once per device and kernel (a racing first call computes the same value).
@@ -648,9 +651,9 @@ static int launch_rb(hipStream_t stream, AttnParams p) {
   p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + (p.T + kScatterTokensPerBlock - 1) / kScatterTokensPerBlock : 1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2) {
-    if constexpr (KVT == RPA_BF16 && WPB >= 4 && TT == TTD) {
+    if constexpr (kHasDecodeDma<D, KVT, TT, WPB>) {
       if (dma) {
-        hipLaunchKernelGGL((attn_decode_dma_kernel<D, TTD, WPB, CAP, RB>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
+        hipLaunchKernelGGL((attn_decode_dma_kernel<D, KVT, TT, WPB, CAP, RB>), dim3(n_wg, head_groups), dim3(64 * WPB), 0, stream, p);
         return (int)hipGetLastError();
       }
     }

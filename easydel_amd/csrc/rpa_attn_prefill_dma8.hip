@@ -20,11 +20,6 @@ namespace rpa {
 // Two floats of ones: what unscaled 8-bit pages use in place of a page's (K scale, V scale).
 __device__ const float ones2[2] = {1.f, 1.f};
 
-// One LDS DMA of 256 bytes (global_load_lds_dword): every lane fetches 4 bytes from base + voff; lane L's bytes land
-// at LDS byte address lds_addr + 4 L.
-__device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const void* base) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
-}
 
 template <int D, int KVT, int NW, int RB, bool CAP>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma8_kernel(AttnParams p) {

@@ -94,6 +94,12 @@ __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const vo
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
+// One LDS DMA of 256 bytes (global_load_lds_dword): every lane fetches 4 bytes from base + voff; lane L's bytes land
+// at LDS byte address lds_addr + 4 L.
+__device__ __forceinline__ void dma4(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
 // Waits until at most N of this wave's vector-memory loads are in flight (they complete in issue order).
 template <int N>
 __device__ __forceinline__ void wait_loads() {
