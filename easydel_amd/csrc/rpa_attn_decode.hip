@@ -75,6 +75,8 @@ constexpr int kPaceCrowd = 4, kPacePause = 8;
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB, bool PACE>
 __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
+  constexpr int HT = KVT == RPA_F16 ? RPA_F16 : RPA_BF16;  // 16-bit float type of the MFMA operands
+  using H = Half16<HT>;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
   constexpr int HB = 2 * RK;           // K_h | V_h span of one token
   constexpr int NCH = RK / 16;         // 16-byte chunks per row
@@ -200,7 +202,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   const int all_hi = cur.ctx - cur.q_len + 1;
 
   // ---- Q as B operands -----------------------------------------------------------------
-  bf16x8 qf[RB][NKK];
+  u32x4 qf[RB][NKK];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok[rb]) * p.Hq + (h * G + r_head[rb])) * p.Dq * 2;
@@ -211,7 +213,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
       const int d0 = (EB == 2) ? (kk * 32 + 8 * g4) : ((kk >> 1) * 64 + 16 * g4 + 8 * (kk & 1));
       u32x4 v = {0u, 0u, 0u, 0u};
       if (n + 16 * rb < rows && d0 < p.Dq) v = *(const u32x4*)(qrow + d0 * 2);  // dims past Dq: zero padding
-      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+      qf[rb][kk] = v;
     }
   }
 
@@ -273,17 +275,17 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
           const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb)
-            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
+            s_acc[rb][st] = H::mfma32(a, qf[rb][kk], s_acc[rb][st]);
         }
       } else {
 #pragma unroll
         for (int j = 0; j < NKK / 2; ++j) {
           const u32x4 a = *(const u32x4*)(krow + (((j * 4 + g4) ^ key) << 4));
-          const bf16x8 a_lo = codes8_to_bf16x8<KVT>(a[0], a[1]), a_hi = codes8_to_bf16x8<KVT>(a[2], a[3]);
+          const u32x4 a_lo = codes8_to_bf16x8<KVT>(a[0], a[1]), a_hi = codes8_to_bf16x8<KVT>(a[2], a[3]);
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb) {
-            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, qf[rb][2 * j], s_acc[rb][st], 0, 0, 0);
-            s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, qf[rb][2 * j + 1], s_acc[rb][st], 0, 0, 0);
+            s_acc[rb][st] = H::mfma32(a_lo, qf[rb][2 * j], s_acc[rb][st]);
+            s_acc[rb][st] = H::mfma32(a_hi, qf[rb][2 * j + 1], s_acc[rb][st]);
           }
         }
       }
@@ -304,9 +306,9 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     for (int rb = 0; rb < RB; ++rb) {
       float alpha;
       if (inside)
-        alpha = softmax_step<false, CAP, NS>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+        alpha = softmax_step<false, CAP, NS, HT>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
       else
-        alpha = softmax_step<true, CAP, NS>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+        alpha = softmax_step<true, CAP, NS, HT>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
       const float o_mul = (EB == 1) ? alpha * unit_mul : alpha;
       if (__any(o_mul != 1.f)) {
 #pragma unroll
@@ -320,11 +322,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
     // 8-bit pages: each lane reads 4 keys x 4 consecutive dims of codes and widens them while transposing.
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-      s16x4 pb[RB];
+      u32x2 pb[RB];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const u32x2 pb2 = {pfrag[rb][st][0], pfrag[rb][st][1]};
-        pb[rb] = __builtin_bit_cast(s16x4, pb2);
+        pb[rb] = pb2;
       }
       if constexpr (EB == 2) {
         const int tk = st * 16 + 4 * g4 + (n >> 2);
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
           const unsigned char* ptr = vrow + (((off >> 4) ^ key) << 4) + (off & 15);
           const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr);
 #pragma unroll
-          for (int rb = 0; rb < RB; ++rb) o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[rb], o_acc[rb][rt], 0, 0, 0);
+          for (int rb = 0; rb < RB; ++rb) o_acc[rb][rt] = H::mfma16(__builtin_bit_cast(u32x2, a), pb[rb], o_acc[rb][rt]);
         }
       } else {
         // lane (n, g4) reads DPL consecutive dims (DPL*n ..) of keys 4g4..4g4+3 and widens them; row tile rt
@@ -368,7 +370,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
           const u32x2 a2 = {pack_bf16(vf[0][rt], vf[1][rt]), pack_bf16(vf[2][rt], vf[3][rt])};
 #pragma unroll
           for (int rb = 0; rb < RB; ++rb)
-            o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), pb[rb], o_acc[rb][rt], 0, 0, 0);
+            o_acc[rb][rt] = H::mfma16(a2, pb[rb], o_acc[rb][rt]);
         }
       }
     }
@@ -437,8 +439,8 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
         if constexpr (EB == 2) {
 #pragma unroll
           for (int rt = 0; rt < DPL; ++rt) {
-            const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
-                             pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+            const u32x2 w = {H::pack(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                             H::pack(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
             if (16 * rt + 4 * g4 < p.Dq) *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
           }
         } else {
@@ -447,7 +449,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 #pragma unroll
             for (int rt = 0; rt < DPL; rt += 2)
               if (DPL * (4 * g4 + j) + rt < p.Dq)
-                *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
+                *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = H::pack(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
         }
       } else {
         const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok[rb]) * p.Hq + head_out;
@@ -615,9 +617,9 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
 }
 
 // The kernel that serves these template arguments: the LDS-direct one where it applies and the call asks for it.
-// It is built for bf16 pages (every head size, four or eight waves) and for 8-bit pages at head size 128 with eight waves.
+// It is built for bf16 / float16 pages (every head size, four or eight waves) and for 8-bit pages at head size 128 with eight waves.
 template <int D, int KVT, int TT, int WPB>
-constexpr bool kHasDecodeDma = (KVT == RPA_BF16 && WPB >= 4 && TT == (D == 64 ? 32 : 16)) ||
+constexpr bool kHasDecodeDma = (ElemBytes<KVT>::v == 2 && WPB >= 4 && TT == (D == 64 ? 32 : 16)) ||
                                (ElemBytes<KVT>::v == 1 && D == 128 && TT == 32 && WPB == 8);
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 static bool use_dma(const AttnParams& p) {
@@ -712,13 +714,16 @@ static int launch_kvt(hipStream_t stream, const AttnParams& p) {
 // call with T query tokens over S sequence rows.  A call that cannot hold a multi-token row (T <= S leaves no room
 // for one unless other rows are empty) keeps the one-block kernel, which is the faster one on single-token rows.
 int decode_row_limit(int T, int S, int D, int kv_dtype) {
-  if (kv_dtype == RPA_BF16 && D <= 128 && T > S) return 2 * kRowBlock;
+  if ((kv_dtype == RPA_BF16 || kv_dtype == RPA_F16) && D <= 128 && T > S) return 2 * kRowBlock;
   return kRowBlock;
 }
 
 bool decode_supported(const AttnParams& p) {
-  if (p.q_dtype != RPA_BF16 || p.kv_dtype == RPA_F32) return false;
-  if (p.kv_dtype == RPA_F16) return false;
+  // bf16 queries over bf16 / fp8 / int8 pages, or float16 queries over float16 pages (the MFMA operands of a kernel
+  // are of one 16-bit type); float16 pages also need the LDS-direct prefill kernel's page sizes, the only large-row
+  // kernel built for them
+  if (p.kv_dtype == RPA_F32) return false;
+  if (p.kv_dtype == RPA_F16 ? (p.q_dtype != RPA_F16 || p.page_size % 32 != 0) : p.q_dtype != RPA_BF16) return false;
   if (p.D != 64 && p.D != 128 && p.D != 256) return false;
   if (p.Dq > p.D || p.Dq % 8 != 0) return false;  // a q row is read in 16-byte chunks, whole chunks inside or outside Dq
   if (p.page_size % 16 != 0) return false;
@@ -731,6 +736,7 @@ int launch_attn_decode(hipStream_t stream, const AttnParams& p_in, int which) {
   p.decode_which = which;
   switch (p.kv_dtype) {
     case RPA_BF16: return launch_kvt<RPA_BF16>(stream, p);
+    case RPA_F16: return launch_kvt<RPA_F16>(stream, p);
     case RPA_FP8_E4M3: return launch_kvt<RPA_FP8_E4M3>(stream, p);
     case RPA_INT8: return launch_kvt<RPA_INT8>(stream, p);
     default: return (int)hipErrorInvalidValue;

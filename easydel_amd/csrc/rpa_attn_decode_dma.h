@@ -65,6 +65,8 @@ __device__ const float decode_dma_unit_scales[2] = {1.f, 1.f};  // what unscaled
 template <int D, int KVT, int TT, int WPB, bool CAP, int RB>
 __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams p) {
   constexpr int EB = ElemBytes<KVT>::v;
+  constexpr int HT = KVT == RPA_F16 ? RPA_F16 : RPA_BF16;  // 16-bit float type of the MFMA operands
+  using H = Half16<HT>;
   constexpr int RK = D * EB;           // bytes of one K (or V) row
   constexpr int NCH = RK / 16;         // 16-byte chunks per row
   constexpr int RPI = 64 / NCH;        // rows one DMA instruction covers
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
     const int all_hi = cur.ctx - cur.q_len + 1;
 
     // ---- Q as B operands: step kk covers dims 32kk + 8g4 + e
-    bf16x8 qf[RB][NKK];
+    u32x4 qf[RB][NKK];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const char* qrow = (const char*)p.q + ((int64_t)(cur.q0 + r_tok[rb]) * p.Hq + (h * G + r_head[rb])) * p.Dq * 2;
@@ -232,7 +234,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
         const int d0 = (EB == 2) ? (kk * 32 + 8 * g4) : ((kk >> 1) * 64 + 16 * g4 + 8 * (kk & 1));
         u32x4 v = {0u, 0u, 0u, 0u};
         if (n + 16 * rb < rows && d0 < p.Dq) v = *(const u32x4*)(qrow + d0 * 2);  // dims past Dq: zero padding
-        qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+        qf[rb][kk] = v;
       }
     }
 
@@ -277,17 +279,17 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
             const u32x4 a = *(const u32x4*)(krow + (((kk * 4 + g4) ^ key) << 4));
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
-              s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][kk], s_acc[rb][st], 0, 0, 0);
+              s_acc[rb][st] = H::mfma32(a, qf[rb][kk], s_acc[rb][st]);
           }
         } else {
 #pragma unroll
           for (int j = 0; j < NKK / 2; ++j) {
             const u32x4 a = *(const u32x4*)(krow + (((j * 4 + g4) ^ key) << 4));
-            const bf16x8 a_lo = codes8_to_bf16x8<KVT>(a[0], a[1]), a_hi = codes8_to_bf16x8<KVT>(a[2], a[3]);
+            const u32x4 a_lo = codes8_to_bf16x8<KVT>(a[0], a[1]), a_hi = codes8_to_bf16x8<KVT>(a[2], a[3]);
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb) {
-              s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, qf[rb][2 * j], s_acc[rb][st], 0, 0, 0);
-              s_acc[rb][st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, qf[rb][2 * j + 1], s_acc[rb][st], 0, 0, 0);
+              s_acc[rb][st] = H::mfma32(a_lo, qf[rb][2 * j], s_acc[rb][st]);
+              s_acc[rb][st] = H::mfma32(a_hi, qf[rb][2 * j + 1], s_acc[rb][st]);
             }
           }
         }
@@ -315,9 +317,9 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
       for (int rb = 0; rb < RB; ++rb) {
         float alpha;
         if (inside)
-          alpha = softmax_step<false, CAP, NS>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+          alpha = softmax_step<false, CAP, NS, HT>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
         else
-          alpha = softmax_step<true, CAP, NS>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
+          alpha = softmax_step<true, CAP, NS, HT>(s_acc[rb], sc_mul, cap_in * k_scale, tb, g4, row_lo[rb], row_hi[rb], m_run[rb], l_run[rb], pfrag[rb]);
         const float o_mul = (EB == 1) ? alpha * unit_mul : alpha;
         if (__any(o_mul != 1.f)) {
 #pragma unroll
@@ -329,11 +331,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
       wait_half(v_half, 2 * tg + 1);
 #pragma unroll
       for (int st = 0; st < NS; ++st) {
-        s16x4 pb[RB];
+        u32x2 pb[RB];
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           const u32x2 pb2 = {pfrag[rb][st][0], pfrag[rb][st][1]};
-          pb[rb] = __builtin_bit_cast(s16x4, pb2);
+          pb[rb] = pb2;
         }
         if constexpr (EB == 2) {
           const int tk = st * 16 + 4 * g4 + (n >> 2);
@@ -345,7 +347,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
             const unsigned char* ptr = vrow + (((off >> 4) ^ key) << 4) + (off & 15);
             const s16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)ptr);
 #pragma unroll
-            for (int rb = 0; rb < RB; ++rb) o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pb[rb], o_acc[rb][rt], 0, 0, 0);
+            for (int rb = 0; rb < RB; ++rb) o_acc[rb][rt] = H::mfma16(__builtin_bit_cast(u32x2, a), pb[rb], o_acc[rb][rt]);
           }
         } else {
           // lane (n, g4) reads DPL consecutive dims (DPL*n ..) of keys 4g4..4g4+3 and widens them; row tile rt of this
@@ -378,7 +380,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
             const u32x2 a2 = {pack_bf16(vf[0][rt], vf[1][rt]), pack_bf16(vf[2][rt], vf[3][rt])};
 #pragma unroll
             for (int rb = 0; rb < RB; ++rb)
-              o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a2), pb[rb], o_acc[rb][rt], 0, 0, 0);
+              o_acc[rb][rt] = H::mfma16(a2, pb[rb], o_acc[rb][rt]);
           }
         }
       }
@@ -404,8 +406,8 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
           if constexpr (EB == 2) {
 #pragma unroll
             for (int rt = 0; rt < DPL; ++rt) {
-              const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
-                               pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+              const u32x2 w = {H::pack(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                               H::pack(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
               if (16 * rt + 4 * g4 < p.Dq) *(u32x2*)(orow + 16 * rt + 4 * g4) = w;
             }
           } else {
@@ -414,7 +416,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
 #pragma unroll
               for (int rt = 0; rt < DPL; rt += 2)
                 if (DPL * (4 * g4 + j) + rt < p.Dq)
-                  *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = pack_bf16(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
+                  *(uint32_t*)(orow + DPL * (4 * g4 + j) + rt) = H::pack(o_acc[rb][rt][j] * inv, o_acc[rb][rt + 1][j] * inv);
           }
         } else {
           const int64_t slot = ((int64_t)cur.slot * p.t_dec_max + cur.part_row + r_tok[rb]) * p.Hq + head_out;
@@ -440,11 +442,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
   }  // pieces
 }
 
-// bf16 or 8-bit pages whose size is a multiple of 64 tokens (a tile's unseen rows borrow a visible row of the same page,
+// 16-bit or 8-bit pages whose size is a multiple of 64 tokens (a tile's unseen rows borrow a visible row of the same page,
 // and the lowest visible key of a sequence lies in the 64-token group its first tile starts), four or more KV heads,
 // and tiles that a 32-bit byte offset can address.
 inline bool decode_dma_supported(const AttnParams& p) {
-  return p.kv_dtype != RPA_F32 && p.kv_dtype != RPA_F16 && p.page_size % 64 == 0 && p.Hkv >= 4 && (int64_t)64 * p.token_stride < ((int64_t)1 << 31);
+  return p.kv_dtype != RPA_F32 && p.page_size % 64 == 0 && p.Hkv >= 4 && (int64_t)64 * p.token_stride < ((int64_t)1 << 31);
 }
 
 }  // namespace rpa

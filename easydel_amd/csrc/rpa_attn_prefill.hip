@@ -176,10 +176,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_kernel(AttnParams p) 
       if constexpr (EB == 2) {
         *(u32x4*)(row + ((st_cc[u] ^ key) << 4)) = v;
       } else {  // 16 codes -> 16 bf16 = two LDS chunks
-        const bf16x8 a = codes8_to_bf16x8<KVT>(v[0], v[1]);
-        const bf16x8 b = codes8_to_bf16x8<KVT>(v[2], v[3]);
-        *(u32x4*)(row + (((2 * st_cc[u]) ^ key) << 4)) = __builtin_bit_cast(u32x4, a);
-        *(u32x4*)(row + (((2 * st_cc[u] + 1) ^ key) << 4)) = __builtin_bit_cast(u32x4, b);
+        *(u32x4*)(row + (((2 * st_cc[u]) ^ key) << 4)) = codes8_to_bf16x8<KVT>(v[0], v[1]);
+        *(u32x4*)(row + (((2 * st_cc[u] + 1) ^ key) << 4)) = codes8_to_bf16x8<KVT>(v[2], v[3]);
       }
     }
   };

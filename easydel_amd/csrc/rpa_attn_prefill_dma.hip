@@ -24,8 +24,9 @@
 
 namespace rpa {
 
-template <int D, int NW, int RB, bool CAP>
+template <int D, int NW, int RB, bool CAP, int HT>
 __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams p) {
+  using H = Half16<HT>;  // bf16, or half for float16 queries over float16 pages
   constexpr int TT = 32;                 // keys per tile
   constexpr int RKL = D * 2;             // bytes of one K (or V) row
   constexpr int CPR = RKL / 16;          // 16-byte chunks per row
@@ -97,7 +98,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   int row_lo[RB], row_hi[RB];
   bool row_ok[RB];
   int out_tok[RB], out_head[RB];
-  bf16x8 qf[RB][NKK];
+  u32x4 qf[RB][NKK];
   int wave_lo, wave_hi;          // keys every row of the wave sees: [max row_lo, min row_hi)
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
@@ -115,7 +116,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     for (int kk = 0; kk < NKK; ++kk) {
       u32x4 v = {0u, 0u, 0u, 0u};
       if (row_ok[rb] && kk * 32 + 8 * g4 < p.Dq) v = *(const u32x4*)(qrow + (kk * 32 + 8 * g4) * 2);  // dims past Dq: zero padding
-      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+      qf[rb][kk] = v;
     }
   }
   // Use the query registers once here, so that the compiler waits for these loads now and not at their first use
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     for (int kk = 0; kk < NKK; ++kk) {
       u32x4 v = __builtin_bit_cast(u32x4, qf[rb][kk]);
       asm volatile("" : "+v"(v));
-      qf[rb][kk] = __builtin_bit_cast(bf16x8, v);
+      qf[rb][kk] = v;
     }
   {
     int lo_max = 0, hi_min = 0x7fffffff;
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
       const u32x4 a = kp[i % KPD];
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb)
-        sa[rb][i / NKK] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), qf[rb][i % NKK], sa[rb][i / NKK], 0, 0, 0);
+        sa[rb][i / NKK] = H::mfma32(a, qf[rb][i % NKK], sa[rb][i / NKK]);
       if (i + KPD < NKO) kp[i % KPD] = read_k(lds_k, i + KPD);
     }
   };
@@ -311,8 +312,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
         float pr[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sa[rb][st][j], sc_mul, -m_use));
-        pfrag[rb][st][0] = pack_bf16(pr[0], pr[1]);
-        pfrag[rb][st][1] = pack_bf16(pr[2], pr[3]);
+        pfrag[rb][st][0] = H::pack(pr[0], pr[1]);
+        pfrag[rb][st][1] = H::pack(pr[2], pr[3]);
       }
     }
   };
@@ -322,11 +323,11 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
     // element of column n, the sum of row n's probabilities over all 32 keys (as rounded to bf16, i.e. exactly the
     // weights the PV product uses).  Two MFMAs replace 16 additions per lane and the cross-lane sum at the end.
     {
-      const u32x4 ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+      const u32x4 ones = {H::kOnes, H::kOnes, H::kOnes, H::kOnes};
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
-        l_acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ones), __builtin_bit_cast(bf16x8, b4), l_acc[rb], 0, 0, 0);
+        l_acc[rb] = H::mfma32(ones, b4, l_acc[rb]);
       }
     }
     // ds_read_b64_tr_b16: inside a 16-lane group, lane l supplies the address of 4 consecutive bf16
@@ -355,8 +356,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const u32x4 b4 = {pfrag[rb][0][0], pfrag[rb][0][1], pfrag[rb][1][0], pfrag[rb][1][1]};
-        o_acc[rb][rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a4), __builtin_bit_cast(bf16x8, b4),
-                                                                o_acc[rb][rt], 0, 0, 0);
+        o_acc[rb][rt] = H::mfma32(a4, b4, o_acc[rb][rt]);
       }
       if (rt + PD < DPL) av[rt % PD] = read_v(rt + PD);
     }
@@ -451,8 +451,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
         uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * p.Dq + 4 * g4;
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) {  // accumulator column j of row tile rt is dim 16rt + 4g4 + j
-          const u32x2 w = {pack_bf16(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
-                           pack_bf16(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
+          const u32x2 w = {H::pack(o_acc[rb][rt][0] * inv, o_acc[rb][rt][1] * inv),
+                           H::pack(o_acc[rb][rt][2] * inv, o_acc[rb][rt][3] * inv)};
           if (16 * rt + 4 * g4 < p.Dq) *(u32x2*)(orow + 16 * rt) = w;
         }
       } else {
@@ -469,32 +469,37 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma_kernel(AttnParams
   }
 }
 
-template <int D, int NW, int RB>
+template <int D, int NW, int RB, int HT>
 static int launch_dma(hipStream_t stream, const AttnParams& p) {
   constexpr int ROWS = NW * RB * 16;
   const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
   const int64_t blocks = slots * p.Hkv * p.pre_max_chunks;
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
   if (p.softcap > 0.f)
-    hipLaunchKernelGGL((attn_prefill_dma_kernel<D, NW, RB, true>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+    hipLaunchKernelGGL((attn_prefill_dma_kernel<D, NW, RB, true, HT>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
   else
-    hipLaunchKernelGGL((attn_prefill_dma_kernel<D, NW, RB, false>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+    hipLaunchKernelGGL((attn_prefill_dma_kernel<D, NW, RB, false, HT>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
   return (int)hipGetLastError();
 }
 
-// bf16 pages whose size is a multiple of the 32-key tile, and page rows that a 32-bit byte offset can address
+// bf16 (or float16) pages whose size is a multiple of the 32-key tile, and page rows that a 32-bit byte offset can address
 bool prefill_dma_supported(const AttnParams& p) {
-  return p.kv_dtype == RPA_BF16 && p.page_size % 32 == 0 && (p.D == 64 || p.D == 128 || p.D == 256) &&
+  return (p.kv_dtype == RPA_BF16 || p.kv_dtype == RPA_F16) && p.page_size % 32 == 0 && (p.D == 64 || p.D == 128 || p.D == 256) &&
          (int64_t)32 * p.token_stride < ((int64_t)1 << 31);
 }
 
-int launch_attn_prefill_dma(hipStream_t stream, const AttnParams& p) {
+template <int HT>
+static int launch_dma_d(hipStream_t stream, const AttnParams& p) {
   switch (p.D) {
-    case 64: return launch_dma<64, 4, 2>(stream, p);
-    case 128: return launch_dma<128, 4, 2>(stream, p);
-    case 256: return launch_dma<256, 8, 1>(stream, p);
+    case 64: return launch_dma<64, 4, 2, HT>(stream, p);
+    case 128: return launch_dma<128, 4, 2, HT>(stream, p);
+    case 256: return launch_dma<256, 8, 1, HT>(stream, p);
     default: return (int)hipErrorInvalidValue;
   }
+}
+
+int launch_attn_prefill_dma(hipStream_t stream, const AttnParams& p) {
+  return p.kv_dtype == RPA_F16 ? launch_dma_d<RPA_F16>(stream, p) : launch_dma_d<RPA_BF16>(stream, p);
 }
 
 }  // namespace rpa

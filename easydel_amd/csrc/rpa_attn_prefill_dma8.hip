@@ -209,7 +209,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma8_kernel(AttnParam
     const int kkey = swz_key<RKL>(dma_row), vkey = swz_key_v<RKL>(dma_row);
 #pragma unroll
     for (int e = 0; e < 2; ++e) {  // codes 8e .. 8e + 7 of the lane's sixteen: chunk 2 dma_chunk + e of the bf16 row
-      *(u32x4*)(krow + (((2 * dma_chunk + e) ^ kkey) << 4)) = __builtin_bit_cast(u32x4, codes8_to_bf16x8<KVT>(ck[2 * e], ck[2 * e + 1]));
+      *(u32x4*)(krow + (((2 * dma_chunk + e) ^ kkey) << 4)) = codes8_to_bf16x8<KVT>(ck[2 * e], ck[2 * e + 1]);
       *(u32x4*)(vrow + (((2 * dma_chunk + e) ^ vkey) << 4)) = __builtin_bit_cast(u32x4, codes8_to_bf16x8<KVT>(cv[2 * e], cv[2 * e + 1]));
     }
     cv_rs = (cv_rs == RN - 1) ? 0 : cv_rs + 1;

@@ -24,6 +24,44 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, r);
 }
 
+// The 16-bit float type of a kernel's MFMA operands: bfloat16 (bf16 queries over bf16, fp8 or int8 pages), or IEEE half
+// (float16 queries over float16 pages).  Same instruction shapes, operand layouts and accumulators either way; the
+// operands travel as raw dwords.
+template <int ET>
+struct Half16;
+template <>
+struct Half16<RPA_BF16> {
+  static constexpr uint32_t kOnes = 0x3F803F80u;  // (1, 1)
+  static __device__ __forceinline__ uint32_t pack(float a, float b) { return pack_bf16(a, b); }
+  static __device__ __forceinline__ f32x4 mfma32(u32x4 a, u32x4 b, f32x4 c) {  // 16x16x32
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(u32x2 a, u32x2 b, f32x4 c) {  // 16x16x16
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, a), __builtin_bit_cast(s16x4, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Half16<RPA_F16> {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+  typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+  static constexpr uint32_t kOnes = 0x3C003C00u;
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {  // round to nearest even
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+  }
+  static __device__ __forceinline__ f32x4 mfma32(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(u32x2 a, u32x2 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+  }
+};
+// ... as chosen by the page dtype of a kernel instance.
+template <int KVT>
+using HalfOf = Half16<KVT == RPA_F16 ? RPA_F16 : RPA_BF16>;
+
 // Four 8-bit codes in one dword -> four floats.
 template <int KVT>
 __device__ __forceinline__ void decode4(uint32_t w, float* f) {
@@ -39,14 +77,14 @@ __device__ __forceinline__ void decode4(uint32_t w, float* f) {
   }
 }
 
-// Eight 8-bit codes (two dwords) -> one bf16x8 MFMA operand (exact: both code sets fit bf16).
+// Eight 8-bit codes (two dwords) -> one bf16 MFMA operand of eight elements (exact: both code sets fit bf16).
 template <int KVT>
-__device__ __forceinline__ bf16x8 codes8_to_bf16x8(uint32_t w0, uint32_t w1) {
+__device__ __forceinline__ u32x4 codes8_to_bf16x8(uint32_t w0, uint32_t w1) {
   float f[8];
   decode4<KVT>(w0, f);
   decode4<KVT>(w1, f + 4);
-  u32x4 r = {pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7])};
-  return __builtin_bit_cast(bf16x8, r);
+  const u32x4 r = {pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7])};
+  return r;
 }
 
 // XOR swizzle of 16-byte chunks inside an LDS row of ROW_BYTES so that 16 consecutive token rows
@@ -122,10 +160,10 @@ __device__ __forceinline__ float fast_tanh(float x) {
 
 // Online-softmax step of one 16-row block over NS 16-key sub-tiles held as S^T accumulators (lane = query row
 // n, 4 keys 4*g4 + j per sub-tile).  Applies the soft cap if CAP, masks keys outside [row_lo, row_hi) if MASK,
-// updates the running max / sum, and leaves the probabilities as packed bf16 B operands.  The maximum is taken
+// updates the running max / sum, and leaves the probabilities as packed 16-bit B operands (bf16, or half if ET says so).  The maximum is taken
 // over the raw scores and scaled once (sc_mul > 0, so scaling commutes with max); each probability is then one
 // fused multiply-add and one exp2.  Returns the factor the output accumulators must be multiplied by.
-template <bool MASK, bool CAP, int NS>
+template <bool MASK, bool CAP, int NS, int ET = RPA_BF16>
 __device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, float cap_in, int tb, int g4,
                                               int row_lo, int row_hi, float& m_run, float& l_run,
                                               uint32_t (&pfrag)[NS][2]) {
@@ -158,8 +196,8 @@ __device__ __forceinline__ float softmax_step(f32x4 (&s_acc)[NS], float sc_mul, 
       pr[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[st][j], sc_mul, -m_use));
       psum += pr[j];
     }
-    pfrag[st][0] = pack_bf16(pr[0], pr[1]);
-    pfrag[st][1] = pack_bf16(pr[2], pr[3]);
+    pfrag[st][0] = Half16<ET>::pack(pr[0], pr[1]);
+    pfrag[st][1] = Half16<ET>::pack(pr[2], pr[3]);
   }
   l_run = l_run * alpha + psum;
   return alpha;

@@ -45,7 +45,7 @@ typedef enum rpa_dtype {
   RPA_FP8_E4M3 = 2, /* OCP e4m3fn codes; value = code * kv_scales[page][combined head], or the code's own value
                        when no scales are passed (the reference's cast-only 8-bit cache, cache.py:143-158) */
   RPA_INT8 = 3,     /* signed 8-bit codes, scaled likewise */
-  RPA_F16 = 4       /* IEEE half: served by the float32 kernel */
+  RPA_F16 = 4       /* IEEE half: half queries over half pages run on the matrix-core kernels, other mixes on the float32 kernel */
 } rpa_dtype;
 
 #define RPA_OK 0
