@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import rpa_testlib as tl
-from rpa_testlib import BF16, FP8, INT8
+from rpa_testlib import BF16, F16, FP8, INT8
 
 pytestmark = pytest.mark.gpu
 
@@ -39,9 +39,8 @@ def test_random_batch(gpu, seed):
         ctx.append(c); q_lens.append(q)
     if sum(q_lens) == 0:
         q_lens[0], ctx[0] = 1, max(ctx[0], 1)
-    b = tl.make_batch(2000 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype,
-                      pad_rows=int(rng.integers(0, 4)), pad_tokens=int(rng.integers(0, 6)),
-                      max_pages=-(-4000 // page_size), shared_prefix_pages=int(rng.integers(0, 3)))
+    shape_kw = dict(pad_rows=int(rng.integers(0, 4)), pad_tokens=int(rng.integers(0, 6)),
+                    max_pages=-(-4000 // page_size), shared_prefix_pages=int(rng.integers(0, 3)))
     kw = {}
     if rng.random() < 0.4:
         kw["sliding_window"] = int(rng.integers(1, 600))
@@ -51,6 +50,10 @@ def test_random_batch(gpu, seed):
         kw["softmax_aux"] = rng.uniform(-3.0, 7.0, size=Hq).astype(np.float32)
     if rng.random() < 0.3:
         kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * D ** -0.5
+    q_dtype = BF16
+    if rng.random() < 0.15:  # float16 queries over float16 pages (drawn last: the other draws of a seed stay what they were)
+        q_dtype = kv_dtype = F16
+    b = tl.make_batch(2000 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, q_dtype=q_dtype, kv_dtype=kv_dtype, **shape_kw)
     what = f"seed {seed}: D{D} pg{page_size} {Hq}/{Hkv} kv{kv_dtype} ctx {ctx} q {q_lens} {sorted(kw)}"
     print(what, flush=True)
     got = tl.run_gpu_attention(b, **kw)
