@@ -39,13 +39,15 @@ size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int wo
  *   "decode_sync"    decode workgroups re-align their waves every this many tiles (power of two, default 8, 0 = never)
  *   "decode_pace"    1 (default): in the bf16 eight-wave decode kernel a wave that finds four or more of its workgroup's
  *                    tiles in flight pauses once (512 clocks) before issuing its own; 0: never
- *   "decode_dma"     which bf16 decode batches (pages of a multiple of 64 tokens, four or more KV heads) run on the
- *                    LDS-direct decode kernel, two tiles in flight per wave: -1 (default) those of head size 256,
- *                    where it measured faster; 0 none; 1 all; 2 all, with one tile in flight
- *   "prefill_chunks" most key chunks one prefill row tile is split into (1..8, 0 = default 8; 1 = never split);
- *                    set it before sizing the workspace
- *   "prefill_dma"    1 (default): bf16 prefill tiles are loaded global -> LDS by the load unit where that kernel
- *                    applies (page_size % 32 == 0); 0: every prefill tile is staged through registers
+ *   "decode_dma"     which decode batches (bf16 / float16 pages, fp8 / int8 pages at head size 128; pages of a multiple
+ *                    of 64 tokens, four or more KV heads) run on the LDS-direct decode kernel, two tiles in flight per
+ *                    wave: -1 (default) 16-bit pages of head size 256, where it measured faster; 0 none; 1 all; 2 all,
+ *                    with one tile in flight
+ *   "prefill_chunks" 0 (default): the key chunks of a prefill row tile are sized on the device from the lengths in the
+ *                    batch (up to 8 per row tile); 1..8: a row tile is cut into at most this many chunks of a length
+ *                    fixed from the block-table bound (1 = never split); set it before sizing the workspace
+ *   "prefill_dma"    1 (default): prefill tiles are loaded global -> LDS by the load unit where those kernels apply
+ *                    (page_size % 32 == 0); 0: every prefill tile is staged through registers (bf16 / 8-bit pages only)
  *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
  *                    the shapes); set it before sizing the workspace
  *   "mla_min_chunk"  fewest keys of such a chunk (rounded up to 64; 0 = default: 1024 at 64 heads and more, else 512)
