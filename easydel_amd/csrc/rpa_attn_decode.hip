@@ -511,8 +511,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     s_merge = (n_live <= 0 || p.qsl[0] > 0 || p.qsl[n_live] < p.T) ? 1 : 0;
   }
   __syncthreads();
-  auto span_of = [&](int i, int& toks) -> int {
-    const SeqPlan sp = seq_plan(p, i);
+  auto span_of = [&](int i, const SeqPlan& sp, int& toks) -> int {
     toks = 0;
     if (sp.live && !sp.small_rows) s_large = 1;  // benign race: every writer stores 1
     // ... rows of sequences with tokens but no context to zero, or partial rows of the decode kernel (any sequence of
@@ -527,9 +526,9 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   int reach = 0;                // a bound on the keys one of its row tiles visits
   int span_min = 0x7fffffff, span_max = 0, n_tiles = 0;  // of a sequence's average row tile
   for (int i = i0; i < i1; ++i) {
-    sum += span_of(i, toks);
-    tsum += toks;
     const SeqPlan sp = seq_plan(p, i);
+    sum += span_of(i, sp, toks);
+    tsum += toks;
     if (sp.live && !sp.small_rows && sp.q_len > 0) {
       const int tile_reach = p.window > 0 ? min(sp.ctx, p.window + kPrefillRows / p.group + 64) : sp.ctx;
       const int tiles = (sp.q_len * p.group + kPrefillRows - 1) / kPrefillRows;
@@ -563,7 +562,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   for (int i = i0; i < i1; ++i) {
     P[i] = run;
     P[S + 1 + i] = min(trun, max(p.t_dec_max - 1, 0));
-    run += span_of(i, toks);
+    run += span_of(i, seq_plan(p, i), toks);
     trun += toks;
   }
   const int W = part[1023];
@@ -606,8 +605,16 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   const int Q = s_Q;
   for (int j = tid; j < p.n_wg; j += 1024) {
     const int64_t target = (int64_t)j * Q;
-    int lo = 0, hi = S;  // invariant: P[lo] <= target (P[0] = 0); answer in [lo, hi)
     if (target >= W) { plan[kPlanHeader + 2 * (S + 1) + j] = 0; continue; }
+    // First among the threads' groups of `per` sequences, whose running sums are still in LDS (part[c] = the sum up
+    // to and including group c; groups past S are empty and sit at W > target), then inside the group in the plan
+    // itself: with up to 1024 sequences the search never leaves LDS.
+    int clo = 0, chi = 1024;  // invariant: the sum before group clo is <= target; the answer's group is in [clo, chi)
+    while (chi - clo > 1) {
+      const int mid = (clo + chi) >> 1;
+      if (part[mid - 1] <= target) clo = mid; else chi = mid;
+    }
+    int lo = clo * per, hi = min(S, lo + per);  // invariant: P[lo] <= target; answer in [lo, hi)
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (P[mid] <= target) lo = mid; else hi = mid;
