@@ -7,6 +7,8 @@ import ast
 import os
 import re
 
+import pytest
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -82,3 +84,20 @@ def test_binding_arity_matches_the_handler_signatures():
         n_bound = len(re.findall(r"\.(?:Ctx|Arg|Ret|Attr)<", bind))
         params = _call_args(cc, "ffi::Error " + impl)[0]
         assert n_bound == len(params), f"{handler}: {n_bound} bound items, {impl} takes {len(params)} parameters"
+
+
+def test_shim_type_checks_against_a_stub_of_the_ffi_api():
+    """The handler file compiles (syntax and types only) against tests/ffi_api_stub, a stand-in with the shape of the
+    XLA FFI API the file uses: every handler's parameter list matches, type by type, what its binding declares.  This
+    is not a build against jaxlib's header, which the image does not have."""
+    import shutil
+    import subprocess
+
+    gxx = shutil.which("g++")
+    hip_include = "/opt/rocm/include"
+    if gxx is None or not os.path.exists(os.path.join(hip_include, "hip", "hip_runtime.h")):
+        pytest.skip("needs g++ and the HIP headers")
+    cmd = [gxx, "-fsyntax-only", "-std=c++17", "-D__HIP_PLATFORM_AMD__", "-I" + hip_include,
+           "-I" + os.path.join(ROOT, "tests", "ffi_api_stub"), os.path.join(ROOT, "easydel_amd", "csrc", "rpa_ffi.cc")]
+    done = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr[-3000:]
