@@ -84,3 +84,42 @@ def test_static_workspace_entry_point_rejects_shapes_beyond_its_array(gpu):
     assert rc == _lib.RPA_ERR_WORKSPACE and b"built-in array holds 67108864" in lib.rpa_last_error()
     assert lib.rpa_ragged_paged_attention_v3_static(None, a, a, a, a, a, a, a, a, a, 0, 4, 4, 10, 64, 8, 2, 128, 128, 4, 1, 1,
                                                     0.1, 0, 0.0, None) == 0  # an empty batch is a no-op
+
+
+def test_static_workspace_entry_point_replays_from_a_hip_graph(gpu):
+    """What the entry point is for: a caller that may not allocate.  After one eager call (which looks up the array's
+    address on this device) the call is captured into a HIP graph and replayed, with eager work and synchronisation
+    between replays; every replay gives the eager result, and new metadata in the same buffers is picked up."""
+    b, d, _ = _case(920, [3000, 700, 65, 1500, 300, 5000], [1, 1, 1, 2, 90, 1], gpu, Hq=32, Hkv=8, D=128, page_size=64)
+    pages, out = d["kv_pages"].clone(), torch.empty_like(d["query"])
+
+    def call():
+        kernels.ragged_paged_attention_v3_static(d["query"], d["key"], d["value"], pages, d["context_lens"], d["block_tables"].reshape(-1),
+                                                 d["query_start_loc"], d["dist"], out=out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    eager = out.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call()
+    for rep in range(3):
+        out.zero_()
+        d["query"].mul_(1.0)  # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
+    d["context_lens"][0] = 2900  # a shorter first sequence: its new token lands elsewhere and it sees fewer keys
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = out.clone()
+    call()
+    torch.cuda.synchronize()
+    assert torch.equal(replayed, out), "a replay with new metadata differs from the eager call on the same buffers"
+    assert not torch.equal(replayed[:1], eager[:1])
