@@ -30,7 +30,7 @@ thread_local char g_err[512] = "";
 // rpa_set_tunable always runs with the defaults below, whatever a profiling or test thread of the same process does.
 struct Tunables {
   int max_splits = 0;      // 0 = sized from the shapes
-  int prefill_chunks = 0;  // 0 = default (kMaxPrefillChunks)
+  int prefill_chunks = 0;  // 0 = chunk length chosen on the device per batch; n = at most n chunks of a fixed length
   int decode_sync = 8;     // workgroup barrier every this many decode tiles (power of two, 0 = never)
   int decode_wgs = 0;      // 0 = as many persistent workgroups as are resident at once
   int force_generic = 0;
