@@ -35,7 +35,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill", "fp8-prefill", "int8-prefill",
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill", "fp8-prefill", "int8-prefill", "gemma-decode",
                              "mla-decode-h128", "mla-decode-h16", "mla-prefill-h128"])
     ap.add_argument("--layout", default="interleaved", choices=["interleaved", "unified"],
                     help="interleaved: one pool [P, page, 2*Hkv, D], scatter fused with the attention call (v3); "
@@ -72,6 +72,8 @@ def build_workload(name, seed, sequential=False):
         return workloads.config4_quantised_decode(seed, "int8")
     if name in ("fp8-prefill", "int8-prefill"):  # tuning shape for the 8-bit prefill kernel
         return workloads.quantised_long_prefill(seed, name.split("-")[0])
+    if name == "gemma-decode":  # tuning shape: decode at head size 256, where the LDS-direct decode kernel is the default
+        return workloads.gemma_decode(seed)
     if name == "llama-prefill":  # tuning shape for the prefill kernel, not one of the benchmark configurations
         return workloads.llama_long_prefill(seed)
     return workloads.config5_gemma_long_prefill(seed, windowed=(name == "c5-window"))

@@ -182,6 +182,17 @@ def llama_long_prefill(seed: int = 0, n_seqs: int = 8, q_len: int = 2048, num_pa
                     block_tables=_tables(rng, ctx, 64, num_pages, 576), softmax_scale=128.0 ** -0.5)
 
 
+def gemma_decode(seed: int = 0, n_seqs: int = 256, num_pages: int = 12_000) -> Workload:
+    """Not one of the five benchmark shapes: pure decode at the heads of the long-context prefill configuration (16
+    query heads over 8 KV heads, head size 256, 128-token pages, soft cap 50), ``n_seqs`` sequences of 512..8192 tokens.
+    The decode shape on which the library picks its LDS-direct decode kernel."""
+    rng = np.random.default_rng(seed)
+    ctx = rng.integers(512, 8193, size=n_seqs).astype(np.int32)
+    return Workload("Gemma-2-9B-shaped pure decode (tuning shape)", Hq=16, Hkv=8, D=256, page_size=128, num_pages=num_pages,
+                    max_pages_per_seq=64, context_lens=ctx, q_lens=np.ones(n_seqs, dtype=np.int32),
+                    block_tables=_tables(rng, ctx, 128, num_pages, 64), softmax_scale=1.0 / 16.0, logits_soft_cap=50.0)
+
+
 def quantised_long_prefill(seed: int = 0, kv_dtype: str = "fp8", n_seqs: int = 4, q_len: int = 2048, num_pages: int = 2000) -> Workload:
     """Not one of the five benchmark shapes: chunked prefill over scaled 8-bit pages at the heads of the quantised decode
     configuration (40 query heads, 8 KV heads, head size 128, 64-token pages): ``n_seqs`` chunks of ``q_len`` tokens
