@@ -36,7 +36,7 @@ struct Tunables {
   int force_generic = 0;
   int prefill_dma = 1;
   int decode_pace = 1;
-  int decode_dma = -1;     // -1: where it measured faster (head size 256); 0: never; 1: wherever it applies; 2: same, one tile ahead
+  int decode_dma = -1;     // -1: where it measured faster (head size 256); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
   int mla_chunks = 0;      // 0 = sized from the shapes
   int mla_min_chunk = 0;   // 0 = default
   int stages = 15;         // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
@@ -175,7 +175,7 @@ int rpa_set_tunable(const char* name, int value) {
   if (!strcmp(name, "force_generic")) return swap(g_tun.force_generic, value != 0);
   if (!strcmp(name, "prefill_dma")) return swap(g_tun.prefill_dma, value != 0);
   if (!strcmp(name, "decode_pace")) return swap(g_tun.decode_pace, value != 0);
-  if (!strcmp(name, "decode_dma")) return swap(g_tun.decode_dma, value < 0 ? -1 : value > 2 ? 2 : value);
+  if (!strcmp(name, "decode_dma")) return swap(g_tun.decode_dma, value < 0 ? -1 : value > 3 ? 3 : value);
   if (!strcmp(name, "mla_min_chunk")) return swap(g_tun.mla_min_chunk, value <= 0 ? 0 : ((value + 63) & ~63));
   if (!strcmp(name, "mla_chunks")) return swap(g_tun.mla_chunks, value < 0 ? 0 : (value > rpa::kMlaMaxChunks ? rpa::kMlaMaxChunks : value));
   if (!strcmp(name, "stages")) return swap(g_tun.stages, value & 15);

@@ -300,7 +300,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int st = 0; st < NS; ++st) asm volatile("" : "+v"(s_acc[rb][st]));
-      issue_k();
+      if (p.decode_dma != 3) issue_k();
 
       // ---- online softmax (log2 domain) ---------------------------------------------------------------------
       const float sc_mul = CAP ? cap_out : p.scale_log2 * k_scale;
@@ -388,6 +388,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int rt = 0; rt < DPL; ++rt) asm volatile("" : "+v"(o_acc[rb][rt]));
+      if (p.decode_dma == 3) issue_k();  // a measurement setting: both halves of a tile asked for at the same moment
       issue_v();
     }
 
