@@ -19,6 +19,9 @@ def _both(b, **kw):
         staged = tl.run_gpu_attention(b, **kw)
         _lib.set_tunable("decode_dma", 1)
         direct = tl.run_gpu_attention(b, **kw)
+        _lib.set_tunable("decode_dma", 3)  # the K rows of a tile requested together with its V rows
+        other = tl.run_gpu_attention(b, **kw)
+        assert np.array_equal(other[tl.valid_rows(b)], direct[tl.valid_rows(b)]), "decode_dma 3 differs"
     finally:
         _lib.set_tunable("decode_dma", prev)
     return staged, direct
