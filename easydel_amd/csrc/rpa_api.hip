@@ -145,10 +145,6 @@ void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* min_chunk) {
   *min_chunk = g_tun.mla_min_chunk > 0 ? g_tun.mla_min_chunk : (Hq >= 64 ? 1024 : 512);
 }
 
-bool mla_shape_on_mfma(int page_size, int lkv, int rope, int row_elems, int q_dtype, int kv_dtype) {
-  return q_dtype == RPA_BF16 && kv_dtype == RPA_BF16 && lkv == 512 && rope == 64 && page_size % 32 == 0 && row_elems % 8 == 0;
-}
-
 }  // namespace
 
 extern "C" {
