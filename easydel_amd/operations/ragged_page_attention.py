@@ -93,6 +93,43 @@ class _RaggedPageAttn(OperationImpl):
         cache_view.kv_pages = kv_pages
         return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
 
+    # -- v3 on pages sharded over data-parallel ranks: one rank's share ------------------------------------------
+    def forward_v3_dp_local_shard(self, query, key, value, local_kv_pages, cache_metadata: RaggedPagesMetadata,
+                                  shard_index: int, num_shards: int, softmax_scale: float | None = None,
+                                  logits_soft_cap: float | None = None, sliding_window: int | None = None,
+                                  softmax_aux=None, **ignore):
+        """What one data-parallel rank computes when the page pool is sharded over ranks and every sequence's pages
+        live on the rank that owns its metadata row (the body of the reference's ``shard_map`` at :645-717, before the
+        sum over ranks): the rank takes its ``S / num_shards`` rows of ``context_lens``, ``pages_tables`` and
+        ``query_start_loc`` (token indices stay global: every rank holds the whole query), recomputes the request
+        distribution for them, rebases the page ids by ``shard_index * local_pages`` and clips them into the local
+        pool, runs the fused write + attention on its pages, and returns output rows that are zero for the tokens of
+        other ranks' sequences.  Returns ``(local_output, local_kv_pages)``; the ranks' outputs are then summed in
+        float32 (:699-717) -- ``dp_local_reduce`` does that for outputs gathered on one device.  Nothing here reads
+        device values on the host."""
+        S = int(cache_metadata.context_lens.shape[0])
+        if num_shards <= 0 or S % num_shards != 0:
+            raise ValueError(f"{S} metadata rows do not divide over {num_shards} shards")  # the reference falls back to the global path
+        if not 0 <= shard_index < num_shards:
+            raise ValueError(f"shard_index {shard_index} outside [0, {num_shards})")
+        rows = S // num_shards
+        row_start = shard_index * rows
+        max_pages = int(cache_metadata.pages_tables.shape[-1]) if cache_metadata.pages_tables.ndim == 2 else \
+            int(cache_metadata.pages_tables.numel()) // S
+        context_lens = cache_metadata.context_lens[row_start:row_start + rows].contiguous()
+        tables = cache_metadata.pages_tables.reshape(S, max_pages)[row_start:row_start + rows]
+        query_start_loc = cache_metadata.query_start_loc[row_start:row_start + rows + 1].contiguous()
+        distribution = _request_distribution_bounds(query_start_loc[1:] - query_start_loc[:-1], context_lens)
+        local_pages = int(local_kv_pages.shape[0])
+        tables = (tables - shard_index * local_pages).clamp(0, local_pages - 1).to(torch.int32).reshape(-1).contiguous()
+        if key.dtype != local_kv_pages.dtype or value.dtype != local_kv_pages.dtype:
+            key, value = key.to(local_kv_pages.dtype), value.to(local_kv_pages.dtype)
+        # tokens outside [query_start_loc[0], query_start_loc[total]) belong to other ranks: the kernels write zeros
+        # for them, which is the masking of :699-712
+        return kernels.ragged_paged_attention_v3(
+            query, key.contiguous(), value.contiguous(), local_kv_pages, context_lens, tables, query_start_loc, distribution,
+            softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, softmax_aux=softmax_aux)
+
     def forward_native(self, query, key, value, cache_view, cache_metadata, softmax_scale: float | None = None,
                        logits_soft_cap: float | None = None, sliding_window: int | None = None, softmax_aux=None,
                        vmem_limit_bytes: int | None = None, mask_value: float | None = None, compute_dtype=None,
@@ -126,6 +163,15 @@ class _RaggedPageAttn(OperationImpl):
         if is_4d:
             output.attention_outputs = output.attention_outputs.reshape(shape4)
         return output
+
+
+def dp_local_reduce(local_outputs) -> torch.Tensor:
+    """The sum over data-parallel ranks the reference performs on the shard outputs: in float32, cast back to the output
+    dtype (:713-717).  For outputs that already sit on one device; across GPUs it is an all-reduce of the same values."""
+    total = local_outputs[0].to(torch.float32)
+    for other in local_outputs[1:]:
+        total = total + other.to(torch.float32)
+    return total.to(local_outputs[0].dtype)
 
 
 def _num_kv_heads(cache_view) -> int | None:

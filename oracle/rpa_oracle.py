@@ -52,6 +52,11 @@ Pinning status
   then ordinary attention, ``layers/attention/_unified.py:1240-1248, 1380-1395``), i.e. to
   ``ragged_paged_attention_ref`` on decompressed pages, and to the reductions of that function's tests.
   ``mla_page_layout_ref`` is pinned by the shape arithmetic of ``caching/mla_ragged_page/cache.py:198-201``.
+* ``dp_local_shard_ref`` (one data-parallel rank's view of the metadata when pages are sharded over ranks): no
+  reference vector exists; pinned in ``tests/test_oracle_dp_local.py`` by what the scheme must guarantee -- every
+  scheduled token is owned by exactly one rank, a page id owned by the rank maps to itself minus the rank's first page
+  and any other id is clipped into the local pool, and the float32 sum over ranks of the ranks' masked attention
+  outputs equals the attention over the whole pool when every sequence's pages live on the rank of its row.
 """
 
 from __future__ import annotations
@@ -164,6 +169,33 @@ def request_distribution_ref(scheduled, context_lens) -> np.ndarray:
     dec = (scheduled == 1) & (context_lens > 1) & has
     n_dec = int(dec.sum())
     return np.array([n_dec, n_dec + int((has & ~dec).sum()), int(has.sum())], dtype=np.int32)
+
+
+def dp_local_shard_ref(shard_index: int, num_shards: int, context_lens, pages_tables, query_start_loc, local_num_pages: int,
+                       total_tokens: int) -> dict:
+    """One data-parallel rank's metadata when the page pool is sharded over ranks --
+    easydel/operations/kernels/ragged_page_attention.py:645-712 (the body of the shard_map before the sum over ranks).
+    The rank takes rows ``[shard * S/n, (shard + 1) * S/n)`` of the lengths and page tables and the matching
+    ``S/n + 1`` entries of ``query_start_loc`` (:650-672; token indices stay global), recomputes the request distribution
+    (:674-676), rebases page ids by ``shard * local_num_pages`` and clips them to ``[0, local_num_pages - 1]`` (:678-681),
+    and keeps the output rows of its own live requests only (:699-712: ``token_mask``)."""
+    context_lens = np.asarray(context_lens, dtype=np.int32)
+    S = context_lens.shape[0]
+    if S % num_shards:
+        raise ValueError("metadata rows do not divide over the shards")
+    rows = S // num_shards
+    r0 = shard_index * rows
+    local_ctx = context_lens[r0:r0 + rows].copy()
+    local_tables = np.asarray(pages_tables, dtype=np.int32).reshape(S, -1)[r0:r0 + rows]
+    local_qsl = np.asarray(query_start_loc, dtype=np.int32)[r0:r0 + rows + 1].copy()
+    dist = request_distribution_ref(local_qsl[1:] - local_qsl[:-1], local_ctx)
+    rebased = np.clip(local_tables - np.int32(shard_index * local_num_pages), 0, local_num_pages - 1).astype(np.int32)
+    mask = np.zeros(total_tokens, dtype=bool)
+    for r in range(rows):
+        if r < int(dist[2]):
+            mask[local_qsl[r]:local_qsl[r + 1]] = True
+    return dict(context_lens=local_ctx, block_tables=rebased.reshape(-1), query_start_loc=local_qsl, distribution=dist,
+                token_mask=mask)
 
 
 def storage_layout_ref(num_kv_heads: int, head_dim: int, bits: int) -> dict:

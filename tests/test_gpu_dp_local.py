@@ -1,0 +1,79 @@
+"""One data-parallel rank's share of the page-sharded attention (reference
+easydel/operations/kernels/ragged_page_attention.py:645-717) on one GPU: the ranks' calls run one after the other on
+their slices of the pool, their outputs are summed as the reference's psum does, and the result is compared with the
+oracle's statement of the same scheme and with one call over the whole pool."""
+
+import numpy as np
+import pytest
+import torch
+
+import rpa_testlib as tl
+from easydel_amd import kernels
+from easydel_amd.caching import RaggedPagesMetadata
+from easydel_amd.operations import OperationMetadata, OperationRegistry
+from easydel_amd.operations.ragged_page_attention import dp_local_reduce
+from rpa_testlib import BF16, orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _sharded_batch(seed, n_shards, rows_per_shard, local_pages, page_size, Hq, Hkv, D):
+    rng = np.random.default_rng(seed)
+    S, M = n_shards * rows_per_shard, 40
+    ctx, q_lens, tables = np.zeros(S, np.int32), np.zeros(S, np.int32), np.zeros((S, M), np.int32)
+    kinds = [(1, 1), (1, 1), (3, 3), (40, 200), (1, 1), (130, 700)]  # (q_len, least context)
+    for sh in range(n_shards):
+        live = int(rng.integers(2, rows_per_shard + 1))
+        free = list(rng.permutation(np.arange(1 if sh == 0 else 0, local_pages)) + sh * local_pages)
+        for r in range(live):
+            i = sh * rows_per_shard + r
+            ql, lo = kinds[int(rng.integers(0, len(kinds)))]
+            ctx[i] = int(rng.integers(max(lo, ql), M * page_size + 1))
+            q_lens[i] = ql
+            need = -(-int(ctx[i]) // page_size)
+            tables[i, :need] = [free.pop() for _ in range(need)]
+    qsl = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    T, P = int(qsl[-1]), n_shards * local_pages
+    raw = lambda *shape: orc.f32_to_bf16_bits(rng.standard_normal(shape, dtype=np.float32))  # noqa: E731
+    return dict(S=S, T=T, P=P, M=M, ctx=ctx, q_lens=q_lens, tables=tables, qsl=qsl, pages=raw(P, page_size, 2 * Hkv, D),
+                q=raw(T, Hq, D), k=raw(T, Hkv, D), v=raw(T, Hkv, D))
+
+
+@pytest.mark.parametrize("n_shards,page_size,Hq,Hkv,D", [(2, 64, 32, 8, 128), (4, 32, 8, 2, 64)])
+def test_dp_local_shards_sum_to_the_global_result(gpu, n_shards, page_size, Hq, Hkv, D):
+    local_pages = 400
+    b = _sharded_batch(70 + n_shards, n_shards, 5, local_pages, page_size, Hq, Hkv, D)
+    up = lambda a: torch.from_numpy(a).to(gpu)  # noqa: E731
+    meta = RaggedPagesMetadata(pages_tables=up(b["tables"]), context_lens=up(b["ctx"]), query_start_loc=up(b["qsl"]),
+                               num_seqs=torch.tensor([b["S"]], dtype=torch.int32, device=gpu),
+                               request_distribution=up(orc.request_distribution_ref(b["q_lens"], b["ctx"])), page_size=page_size)
+    q, k, v = (tl.to_torch(b[x], BF16, gpu) for x in ("q", "k", "v"))
+    pool = tl.to_torch(b["pages"], BF16, gpu)
+    op = OperationRegistry.create("ragged_page_attention_v3", OperationMetadata())
+    outs, new_pages = [], []
+    for sh in range(n_shards):
+        out, pages = op.forward_v3_dp_local_shard(q, k, v, pool[sh * local_pages:(sh + 1) * local_pages].clone(), meta, sh, n_shards)
+        torch.cuda.synchronize()
+        m = orc.dp_local_shard_ref(sh, n_shards, b["ctx"], b["tables"], b["qsl"], local_pages, b["T"])
+        got = tl.from_torch(out, BF16)
+        assert not np.abs(got[~m["token_mask"]]).any(), f"shard {sh}: rows of other ranks' tokens must be zero"
+        outs.append(out)
+        new_pages.append(pages)
+    total = tl.from_torch(dp_local_reduce(outs), BF16)
+    # the page write: every rank wrote its own sequences' tokens; together they are the global write
+    want_pages = orc.page_scatter_ragged_ref(b["k"], b["v"], b["pages"], b["ctx"], b["tables"], b["qsl"], [b["S"]])
+    got_pages = torch.cat(new_pages).view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got_pages, want_pages)
+    want = orc.ragged_paged_attention_ref(orc.bf16_bits_to_f32(b["q"]).astype(np.float64), orc.bf16_bits_to_f32(want_pages).astype(np.float64),
+                                          b["ctx"], b["tables"], b["qsl"], [b["S"]])
+    err = np.abs(total - want)
+    assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
+    # and one call over the whole pool gives the same rows within the same bound (every row counted: the live rows
+    # of the ranks are not contiguous in the global arrays, rows without tokens are skipped by their empty spans)
+    every_row = torch.tensor([0, 0, b["S"]], dtype=torch.int32, device=gpu)
+    out_global, _ = kernels.ragged_paged_attention_v3(q, k, v, pool.clone(), meta.context_lens, meta.pages_tables.reshape(-1),
+                                                      meta.query_start_loc, every_row)
+    torch.cuda.synchronize()
+    assert np.abs(tl.from_torch(out_global, BF16) - want).max() <= tl.TOL_BF16_MAX
+    with pytest.raises(ValueError):
+        op.forward_v3_dp_local_shard(q, k, v, pool[:local_pages], meta, 0, 3 if b["S"] % 3 else 7)
