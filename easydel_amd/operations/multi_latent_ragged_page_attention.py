@@ -135,6 +135,27 @@ class _MultiLatentRaggedPageAttn(OperationImpl):
             output = output.reshape(shape4)
         return AttentionOutput(attention_weights=None, attention_outputs=output, cache_view=cache_view)
 
+    def forward_core_dp_local_shard(self, queries_nope, queries_pe, keys_values, keys_pe, local_kv_pages, cache_metadata,
+                                    shard_index: int, num_shards: int, softmax_scale: float | None = None,
+                                    logits_soft_cap: float | None = None, sliding_window: int | None = None,
+                                    softmax_aux=None, **ignore):
+        """One data-parallel rank's share when the latent pages are sharded over ranks and every sequence's pages live
+        on the rank of its metadata row (the body of the reference's ``shard_map`` at :507-566, before the sum over
+        ranks): metadata rows sliced, page ids rebased and clipped, distribution recomputed, fused write + attention on
+        the rank's pages; the rows of other ranks' tokens come back as zeros.  Operands already flattened
+        (``[tokens, heads, dim]`` / ``[tokens, dim]``) and in the page dtype.  Returns ``(local_output, local_kv_pages)``;
+        the ranks' outputs are summed in float32 (``ragged_page_attention.dp_local_reduce``)."""
+        from .ragged_page_attention import dp_local_metadata
+
+        context_lens, tables, query_start_loc, distribution = dp_local_metadata(cache_metadata, shard_index, num_shards,
+                                                                                int(local_kv_pages.shape[0]))
+        distribution = torch.stack([torch.zeros_like(distribution[2]), torch.zeros_like(distribution[2]), distribution[2]])
+        return kernels.mla_ragged_paged_attention(
+            queries_nope.contiguous(), queries_pe.to(queries_nope.dtype).contiguous(), keys_values.to(local_kv_pages.dtype).contiguous(),
+            keys_pe.to(local_kv_pages.dtype).contiguous(), local_kv_pages, context_lens, tables, query_start_loc,
+            distribution.contiguous(), softmax_scale=softmax_scale, sliding_window=sliding_window,
+            logits_soft_cap=logits_soft_cap, softmax_aux=softmax_aux)
+
     def forward_native(self, *args, **kwargs) -> AttentionOutput:
         return self.forward_core(*args, **kwargs)
 

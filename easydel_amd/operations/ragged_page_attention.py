@@ -35,6 +35,28 @@ def _request_distribution_bounds(scheduled: torch.Tensor, context_lens: torch.Te
     return torch.stack((decode, decode + prefill, has_tokens.sum())).to(torch.int32)
 
 
+def dp_local_metadata(cache_metadata, shard_index: int, num_shards: int, local_pages: int):
+    """``(context_lens, flat block tables, query_start_loc, distribution)`` of one data-parallel rank when the page pool
+    is sharded over ranks (reference :650-681; the same lines serve the multi-latent operation,
+    multi_latent_ragged_page_attention.py:507-536): the rank's rows of the lengths and page tables, the matching
+    ``rows + 1`` entries of ``query_start_loc`` (token indices stay global), the request distribution recomputed for them,
+    page ids rebased by ``shard_index * local_pages`` and clipped into the local pool.  All on the device."""
+    S = int(cache_metadata.context_lens.shape[0])
+    if num_shards <= 0 or S % num_shards != 0:
+        raise ValueError(f"{S} metadata rows do not divide over {num_shards} shards")  # the reference falls back to the global path
+    if not 0 <= shard_index < num_shards:
+        raise ValueError(f"shard_index {shard_index} outside [0, {num_shards})")
+    rows = S // num_shards
+    row_start = shard_index * rows
+    max_pages = int(cache_metadata.pages_tables.numel()) // S
+    context_lens = cache_metadata.context_lens[row_start:row_start + rows].contiguous()
+    tables = cache_metadata.pages_tables.reshape(S, max_pages)[row_start:row_start + rows]
+    query_start_loc = cache_metadata.query_start_loc[row_start:row_start + rows + 1].contiguous()
+    distribution = _request_distribution_bounds(query_start_loc[1:] - query_start_loc[:-1], context_lens)
+    tables = (tables - shard_index * local_pages).clamp(0, local_pages - 1).to(torch.int32).reshape(-1).contiguous()
+    return context_lens, tables, query_start_loc, distribution
+
+
 class _RaggedPageAttn(OperationImpl):
     """Attention over a paged KV cache for ragged batches (prefill, chunked prefill and decode rows mixed)."""
 
@@ -107,21 +129,7 @@ class _RaggedPageAttn(OperationImpl):
         other ranks' sequences.  Returns ``(local_output, local_kv_pages)``; the ranks' outputs are then summed in
         float32 (:699-717) -- ``dp_local_reduce`` does that for outputs gathered on one device.  Nothing here reads
         device values on the host."""
-        S = int(cache_metadata.context_lens.shape[0])
-        if num_shards <= 0 or S % num_shards != 0:
-            raise ValueError(f"{S} metadata rows do not divide over {num_shards} shards")  # the reference falls back to the global path
-        if not 0 <= shard_index < num_shards:
-            raise ValueError(f"shard_index {shard_index} outside [0, {num_shards})")
-        rows = S // num_shards
-        row_start = shard_index * rows
-        max_pages = int(cache_metadata.pages_tables.shape[-1]) if cache_metadata.pages_tables.ndim == 2 else \
-            int(cache_metadata.pages_tables.numel()) // S
-        context_lens = cache_metadata.context_lens[row_start:row_start + rows].contiguous()
-        tables = cache_metadata.pages_tables.reshape(S, max_pages)[row_start:row_start + rows]
-        query_start_loc = cache_metadata.query_start_loc[row_start:row_start + rows + 1].contiguous()
-        distribution = _request_distribution_bounds(query_start_loc[1:] - query_start_loc[:-1], context_lens)
-        local_pages = int(local_kv_pages.shape[0])
-        tables = (tables - shard_index * local_pages).clamp(0, local_pages - 1).to(torch.int32).reshape(-1).contiguous()
+        context_lens, tables, query_start_loc, distribution = dp_local_metadata(cache_metadata, shard_index, num_shards, int(local_kv_pages.shape[0]))
         if key.dtype != local_kv_pages.dtype or value.dtype != local_kv_pages.dtype:
             key, value = key.to(local_kv_pages.dtype), value.to(local_kv_pages.dtype)
         # tokens outside [query_start_loc[0], query_start_loc[total]) belong to other ranks: the kernels write zeros

@@ -77,3 +77,48 @@ def test_dp_local_shards_sum_to_the_global_result(gpu, n_shards, page_size, Hq, 
     assert np.abs(tl.from_torch(out_global, BF16) - want).max() <= tl.TOL_BF16_MAX
     with pytest.raises(ValueError):
         op.forward_v3_dp_local_shard(q, k, v, pool[:local_pages], meta, 0, 3 if b["S"] % 3 else 7)
+
+
+def test_mla_dp_local_shards_sum_to_the_global_result(gpu):
+    """The same scheme for the multi-latent operation over latent pages
+    (easydel/operations/kernels/multi_latent_ragged_page_attention.py:507-566)."""
+    n_shards, local_pages, page_size, Hq, lkv, rope = 2, 120, 64, 16, 512, 64
+    row = orc.mla_page_layout_ref(lkv, rope, page_size)["kv_dim_padded"]
+    rng = np.random.default_rng(91)
+    S, M = n_shards * 4, 12
+    ctx, q_lens, tables = np.zeros(S, np.int32), np.zeros(S, np.int32), np.zeros((S, M), np.int32)
+    for sh in range(n_shards):
+        free = list(rng.permutation(np.arange(1 if sh == 0 else 0, local_pages)) + sh * local_pages)
+        for r, (ql, c) in enumerate([(1, 300), (2, 130), (40, 700)][:3 - sh]):
+            i = sh * 4 + r
+            ctx[i], q_lens[i] = c + int(rng.integers(0, 60)), ql
+            need = -(-int(ctx[i]) // page_size)
+            tables[i, :need] = [free.pop() for _ in range(need)]
+    qsl = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    T, P = int(qsl[-1]), n_shards * local_pages
+    raw = lambda *shape: orc.f32_to_bf16_bits((0.3 * rng.standard_normal(shape)).astype(np.float32))  # noqa: E731
+    pages = raw(P, page_size, row)
+    qn, qp, kvs, pe = raw(T, Hq, lkv), raw(T, Hq, rope), raw(T, lkv), raw(T, rope)
+    up = lambda a: torch.from_numpy(a).to(gpu)  # noqa: E731
+    meta = RaggedPagesMetadata(pages_tables=up(tables), context_lens=up(ctx), query_start_loc=up(qsl),
+                               num_seqs=torch.tensor([S], dtype=torch.int32, device=gpu),
+                               request_distribution=up(orc.request_distribution_ref(q_lens, ctx)), page_size=page_size)
+    op = OperationRegistry.create("multi_latent_ragged_page_attention_v1", OperationMetadata())
+    pool = tl.to_torch(pages, BF16, gpu)
+    scale = (128 + rope) ** -0.5
+    outs, new_pages = [], []
+    for sh in range(n_shards):
+        out, local = op.forward_core_dp_local_shard(tl.to_torch(qn, BF16, gpu), tl.to_torch(qp, BF16, gpu), tl.to_torch(kvs, BF16, gpu),
+                                                    tl.to_torch(pe, BF16, gpu), pool[sh * local_pages:(sh + 1) * local_pages].clone(),
+                                                    meta, sh, n_shards, softmax_scale=scale)
+        torch.cuda.synchronize()
+        m = orc.dp_local_shard_ref(sh, n_shards, ctx, tables, qsl, local_pages, T)
+        assert not np.abs(tl.from_torch(out, BF16)[~m["token_mask"]]).any(), f"shard {sh}: rows of other ranks' tokens must be zero"
+        outs.append(out)
+        new_pages.append(local)
+    want_pages = orc.mla_page_scatter_ref(kvs, pe, pages, ctx, tables, qsl, [S])
+    assert np.array_equal(torch.cat(new_pages).view(torch.int16).cpu().numpy().view(np.uint16), want_pages)
+    f = lambda a: orc.bf16_bits_to_f32(a).astype(np.float64)  # noqa: E731
+    want = orc.mla_ragged_paged_attention_ref(f(qn), f(qp), f(want_pages), ctx, tables, qsl, [S], kv_lora_rank=lkv, qk_rope_head_dim=rope, softmax_scale=scale)
+    err = np.abs(tl.from_torch(dp_local_reduce(outs), BF16) - want)
+    assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
