@@ -5,7 +5,8 @@ name (:84, :113), requirements (:117-147), call signature of ``forward_native`` 
 reshape (:256-262, :395-396) and ``AttentionOutput`` result.  Where the reference hands the arrays to
 ``ejkernel.modules.unified_attention`` (:363-388) this module hands device pointers to ``librpa_hip.so``.  The
 operation reads the pools only: the step's K/V are written before by the view's ``concatenate_to_cache``.
-The reference's shard-local path over the ``ATTN_DP`` mesh axis (:290-361) has no one-GPU counterpart.
+One rank's share of the reference's shard-local path over the ``ATTN_DP`` mesh axis (:278-353) is
+``forward_dp_local_shard``; the sum over ranks that follows it there (:355-357) needs more than one GPU.
 """
 
 from __future__ import annotations
@@ -55,6 +56,31 @@ class UnifiedAttn(OperationImpl):
         if is_4d:
             out = out.reshape(shape4)
         return AttentionOutput(attention_weights=None, attention_outputs=out, cache_view=cache_view)
+
+    def forward_dp_local_shard(self, query, local_key_cache, local_value_cache, cache_metadata: RaggedPagesMetadata,
+                               shard_index: int, num_shards: int, softmax_scale: float | None = None,
+                               sliding_window: int | None = None, logits_soft_cap: float | None = None, softmax_aux=None,
+                               **ignore):
+        """What one data-parallel rank computes when the K and V pools are sharded over ranks and every sequence's pages
+        live on the rank of its metadata row (the body of the reference's ``shard_map`` at :296-353, before the sum over
+        ranks): its rows of the lengths, page tables and ``query_start_loc``, page ids rebased by
+        ``shard_index * local_pages``.  The reference also rotates the packed tokens so that the rank's span starts at
+        index 0 (its kernel needs ``query_start_loc[0] == 0``, :319-327) and zeroes the other ranks' tokens afterwards
+        (:345-353); these kernels take the global token indices as they are and write zeros for tokens outside the
+        rank's span, so neither step exists here.  ``query`` is ``[tokens, heads, dim]``; returns the local output."""
+        S = int(cache_metadata.context_lens.shape[0])
+        if num_shards <= 0 or S % num_shards != 0:
+            raise ValueError(f"{S} metadata rows do not divide over {num_shards} shards")
+        if not 0 <= shard_index < num_shards:
+            raise ValueError(f"shard_index {shard_index} outside [0, {num_shards})")
+        rows = S // num_shards
+        r0 = shard_index * rows
+        local_pages = int(local_key_cache.shape[0])
+        tables = cache_metadata.pages_tables.reshape(S, -1)[r0:r0 + rows] - shard_index * local_pages  # ids off the pool are clamped by the kernels
+        return kernels.unified_attention(
+            query.contiguous(), local_key_cache, local_value_cache, cache_metadata.context_lens[r0:r0 + rows].contiguous(),
+            tables.to(cache_metadata.pages_tables.dtype).contiguous(), cache_metadata.query_start_loc[r0:r0 + rows + 1].contiguous(), None,
+            softmax_scale=softmax_scale, sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, softmax_aux=softmax_aux)
 
     def forward_gpu(self, *args, **kwargs) -> AttentionOutput:
         return self.forward_native(*args, **kwargs)

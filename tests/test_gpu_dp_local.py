@@ -122,3 +122,29 @@ def test_mla_dp_local_shards_sum_to_the_global_result(gpu):
     want = orc.mla_ragged_paged_attention_ref(f(qn), f(qp), f(want_pages), ctx, tables, qsl, [S], kv_lora_rank=lkv, qk_rope_head_dim=rope, softmax_scale=scale)
     err = np.abs(tl.from_torch(dp_local_reduce(outs), BF16) - want)
     assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
+
+
+def test_unified_attention_dp_local_shards_sum_to_the_global_result(gpu):
+    """The same scheme over separate K and V pools (easydel/operations/kernels/unified_attention.py:278-357); the
+    operation only reads the pools."""
+    n_shards, local_pages, page_size, Hq, Hkv, D = 2, 300, 64, 32, 8, 128
+    b = _sharded_batch(77, n_shards, 5, local_pages, page_size, Hq, Hkv, D)
+    up = lambda a: torch.from_numpy(a).to(gpu)  # noqa: E731
+    meta = RaggedPagesMetadata(pages_tables=up(b["tables"]), context_lens=up(b["ctx"]), query_start_loc=up(b["qsl"]),
+                               num_seqs=torch.tensor([b["S"]], dtype=torch.int32, device=gpu), page_size=page_size)
+    q = tl.to_torch(b["q"], BF16, gpu)
+    pool = tl.to_torch(b["pages"], BF16, gpu)
+    k_pool, v_pool = pool[:, :, 0::2].contiguous(), pool[:, :, 1::2].contiguous()
+    op = OperationRegistry.create("unified_attention", OperationMetadata())
+    outs = []
+    for sh in range(n_shards):
+        sl = slice(sh * local_pages, (sh + 1) * local_pages)
+        out = op.forward_dp_local_shard(q, k_pool[sl].contiguous(), v_pool[sl].contiguous(), meta, sh, n_shards)
+        torch.cuda.synchronize()
+        m = orc.dp_local_shard_ref(sh, n_shards, b["ctx"], b["tables"], b["qsl"], local_pages, b["T"])
+        assert not np.abs(tl.from_torch(out, BF16)[~m["token_mask"]]).any(), f"shard {sh}: rows of other ranks' tokens must be zero"
+        outs.append(out)
+    want = orc.ragged_paged_attention_ref(orc.bf16_bits_to_f32(b["q"]).astype(np.float64), orc.bf16_bits_to_f32(b["pages"]).astype(np.float64),
+                                          b["ctx"], b["tables"], b["qsl"], [b["S"]])
+    err = np.abs(tl.from_torch(dp_local_reduce(outs), BF16) - want)
+    assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
