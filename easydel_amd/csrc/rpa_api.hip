@@ -540,8 +540,8 @@ static int mla_fill(const char* who, rpa::MlaParams& p, const void* keys_values,
   const int rope_off = (lkv + 127) / 128 * 128;
   if (row_elems < rope_off + rope)
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: row_elems=%d < %d (latent part padded to 128, then the rope key)", who, row_elems, rope_off + rope);
-  if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16)
-    return fail(RPA_ERR_UNSUPPORTED, "%s: kv_dtype %d (want f32 or bf16)", who, kv_dtype);
+  if (kv_dtype != RPA_F32 && kv_dtype != RPA_BF16 && kv_dtype != RPA_F16 && kv_dtype != RPA_FP8_E4M3)
+    return fail(RPA_ERR_UNSUPPORTED, "%s: kv_dtype %d (want f32, bf16, f16 or fp8-e4m3 codes without scales)", who, kv_dtype);
   memset(&p, 0, sizeof(p));
   p.new_kv = keys_values; p.new_pe = keys_pe; p.pages = kv_pages;
   p.context_lens = context_lens; p.block_tables = block_tables; p.qsl = query_start_loc; p.num_seqs = num_seqs;
@@ -560,10 +560,10 @@ int rpa_mla_page_scatter(rpa_stream_t stream, const void* keys_values, const voi
                          const int32_t* num_seqs, int T, int S, int M, int P, int page_size, int kv_lora_rank,
                          int qk_rope_head_dim, int row_elems, int elem_bytes) {
   const char* who = "rpa_mla_page_scatter";
-  if (elem_bytes != 2 && elem_bytes != 4) return fail(RPA_ERR_UNSUPPORTED, "%s: elem_bytes %d (want 2 or 4)", who, elem_bytes);
+  if (elem_bytes != 1 && elem_bytes != 2 && elem_bytes != 4) return fail(RPA_ERR_UNSUPPORTED, "%s: elem_bytes %d (want 1, 2 or 4)", who, elem_bytes);
   rpa::MlaParams p;
   const int rc = mla_fill(who, p, keys_values, keys_pe, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, T, S,
-                          M, P, page_size, kv_lora_rank, qk_rope_head_dim, row_elems, elem_bytes == 4 ? RPA_F32 : RPA_BF16);
+                          M, P, page_size, kv_lora_rank, qk_rope_head_dim, row_elems, elem_bytes == 4 ? RPA_F32 : elem_bytes == 2 ? RPA_BF16 : RPA_FP8_E4M3);
   if (rc) return rc;
   if (T == 0) return RPA_OK;
   if (!keys_values || (!keys_pe && qk_rope_head_dim > 0) || !kv_pages || !context_lens || !block_tables || !query_start_loc || !num_seqs)
@@ -581,7 +581,7 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
                                    const float* softmax_aux) {
   const char* who = "rpa_mla_ragged_paged_attention";
   if (Hq <= 0) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: bad size (Hq=%d)", who, Hq);
-  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16) return fail(RPA_ERR_UNSUPPORTED, "%s: q_dtype %d (want f32 or bf16)", who, q_dtype);
+  if (q_dtype != RPA_F32 && q_dtype != RPA_BF16 && q_dtype != RPA_F16) return fail(RPA_ERR_UNSUPPORTED, "%s: q_dtype %d (want f32, bf16 or f16)", who, q_dtype);
   if (!distribution) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: null distribution", who);
   if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_scale is not finite", who);
   if (softmax_aux && ((uintptr_t)softmax_aux & 3)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_aux must be 4-byte aligned", who);

@@ -148,8 +148,7 @@ __global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
     if (d < lkv) {
       const int64_t o = ((int64_t)t * p.Hq + hq) * lkv + d;
       const float r = acc[k] * inv;
-      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
-      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
+      store_out<QT>(p.out, o, r);
     }
   }
 }
@@ -790,8 +789,7 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(MlaParams p) {
     if (d < lkv) {
       const int64_t o = ((int64_t)t * p.Hq + hq) * lkv + d;
       const float r = acc[k] * inv;
-      if constexpr (QT == RPA_F32) ((float*)p.out)[o] = r;
-      else ((uint16_t*)p.out)[o] = float_to_bf16_bits(r);
+      store_out<QT>(p.out, o, r);
     }
   }
 }
@@ -884,6 +882,8 @@ int launch_generic_q(hipStream_t stream, const MlaParams& p) {
   switch (p.kv_dtype) {
     case RPA_F32: hipLaunchKernelGGL((mla_generic_kernel<QT, RPA_F32>), grid, block, 0, stream, p); break;
     case RPA_BF16: hipLaunchKernelGGL((mla_generic_kernel<QT, RPA_BF16>), grid, block, 0, stream, p); break;
+    case RPA_F16: hipLaunchKernelGGL((mla_generic_kernel<QT, RPA_F16>), grid, block, 0, stream, p); break;
+    case RPA_FP8_E4M3: hipLaunchKernelGGL((mla_generic_kernel<QT, RPA_FP8_E4M3>), grid, block, 0, stream, p); break;  // codes as cast, no scales
     default: return (int)hipErrorInvalidValue;
   }
   return (int)hipGetLastError();
@@ -893,15 +893,18 @@ int launch_generic_q(hipStream_t stream, const MlaParams& p) {
 
 int launch_mla_scatter(hipStream_t stream, const MlaParams& p) {
   const int blocks = (p.T + 3) / 4;
-  if (p.kv_dtype == RPA_F32) hipLaunchKernelGGL((mla_scatter_kernel<uint32_t>), dim3(blocks), dim3(256), 0, stream, p);
-  else if (p.kv_dtype == RPA_BF16) hipLaunchKernelGGL((mla_scatter_kernel<uint16_t>), dim3(blocks), dim3(256), 0, stream, p);
-  else return (int)hipErrorInvalidValue;
+  switch (elem_bytes(p.kv_dtype)) {  // the write copies bits, whatever they encode
+    case 4: hipLaunchKernelGGL((mla_scatter_kernel<uint32_t>), dim3(blocks), dim3(256), 0, stream, p); break;
+    case 2: hipLaunchKernelGGL((mla_scatter_kernel<uint16_t>), dim3(blocks), dim3(256), 0, stream, p); break;
+    default: hipLaunchKernelGGL((mla_scatter_kernel<uint8_t>), dim3(blocks), dim3(256), 0, stream, p); break;
+  }
   return (int)hipGetLastError();
 }
 
 int launch_mla_generic(hipStream_t stream, const MlaParams& p) {
   if (p.lkv > kGenMaxLkv || p.rope > kGenMaxRope) return (int)hipErrorInvalidValue;
-  return p.q_dtype == RPA_F32 ? launch_generic_q<RPA_F32>(stream, p) : launch_generic_q<RPA_BF16>(stream, p);
+  return p.q_dtype == RPA_F32 ? launch_generic_q<RPA_F32>(stream, p)
+         : p.q_dtype == RPA_F16 ? launch_generic_q<RPA_F16>(stream, p) : launch_generic_q<RPA_BF16>(stream, p);
 }
 
 // bf16 queries and pages of the one shape every model with this cache uses (latent 512, rope 64, the rope key right
@@ -946,6 +949,7 @@ int launch_mla_merge(hipStream_t stream, const MlaParams& p) {
   }
   const int blocks = (int)(((int64_t)p.T * p.Hq + 3) / 4);
   if (p.q_dtype == RPA_F32) hipLaunchKernelGGL((mla_merge_kernel<RPA_F32>), dim3(blocks), dim3(256), 0, stream, p);
+  else if (p.q_dtype == RPA_F16) hipLaunchKernelGGL((mla_merge_kernel<RPA_F16>), dim3(blocks), dim3(256), 0, stream, p);
   else hipLaunchKernelGGL((mla_merge_kernel<RPA_BF16>), dim3(blocks), dim3(256), 0, stream, p);
   return (int)hipGetLastError();
 }

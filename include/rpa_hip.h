@@ -256,9 +256,11 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
  *                 value half of the up-projection, _unified.py:1366-1371)
  *   workspace     device scratch of at least rpa_mla_workspace_bytes(...) bytes
  *   softmax_scale as passed by the caller: (qk_nope_head_dim + qk_rope_head_dim) ** -0.5 (_unified.py:1310)
- * q_dtype RPA_F32 or RPA_BF16; kv_dtype RPA_F32 or RPA_BF16; kv_lora_rank <= 512, qk_rope_head_dim <= 256, both
- * multiples of 8.  bf16 with kv_lora_rank 512, rope 64 and page_size % 32 == 0 runs on the matrix cores; every other
- * combination on the fp32 kernel.  Window, soft cap, softmax_aux, padding and error behaviour as for
+ * q_dtype RPA_F32, RPA_BF16 or RPA_F16; kv_dtype RPA_F32, RPA_BF16, RPA_F16 or RPA_FP8_E4M3 (the latent cache holds
+ * no scale arrays, caching/mla_ragged_page/cache.py:197-204, 344: fp8 pages are the plain cast of the rows and are
+ * read back as the codes' own values); kv_lora_rank <= 512, qk_rope_head_dim <= 256, both multiples of 8.  bf16
+ * queries over bf16 pages with kv_lora_rank 512, rope 64 and page_size % 32 == 0 run on the matrix cores; every
+ * other combination on the fp32 kernel.  Window, soft cap, softmax_aux, padding and error behaviour as for
  * rpa_ragged_paged_attention.
  */
 int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope, const void* queries_pe,
@@ -275,7 +277,7 @@ size_t rpa_mla_workspace_bytes(int T, int S, int M, int page_size, int Hq, int k
 
 /*
  * The write half of the MLA operation on its own (same operands and placement as above; num_seqs: device int32 [1]).
- * elem_bytes 2 or 4.
+ * elem_bytes 1, 2 or 4.
  */
 int rpa_mla_page_scatter(rpa_stream_t stream, const void* keys_values, const void* keys_pe, void* kv_pages,
                          const int32_t* context_lens, const int32_t* block_tables, const int32_t* query_start_loc,

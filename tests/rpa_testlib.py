@@ -277,8 +277,8 @@ class MlaBatch:
 
 
 def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64, dtype=BF16, pad_rows=0, pad_tokens=0,
-                   row=None, max_pages=None, distinct_pages=0):
-    """`distinct_pages` > 0: the pool repeats that many random pages (thousands of sequences need thousands of pages,
+                   row=None, max_pages=None, distinct_pages=0, kv_dtype=None):
+    """`kv_dtype`: element format of the latent pages and of the new rows (default: the queries').  `distinct_pages` > 0: the pool repeats that many random pages (thousands of sequences need thousands of pages,
     and drawing every one takes minutes on a slow host)."""
     rng = np.random.default_rng(seed)
     ctx_lens = np.asarray(ctx_lens, np.int32)
@@ -289,6 +289,7 @@ def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64
     b.row = row or lay["kv_dim_padded"]
     b.off = lay["rope_offset"]
     b.Hq, b.lkv, b.rope, b.page_size, b.n, b.q_dtype = Hq, lkv, rope, page_size, n, dtype
+    b.kv_dtype = dtype if kv_dtype is None else kv_dtype
     need = [-(-int(c) // page_size) for c in ctx_lens]
     b.S = n + pad_rows
     b.M = max_pages or max(max(need), 1)
@@ -310,24 +311,31 @@ def make_mla_batch(seed, ctx_lens, q_lens, *, Hq, lkv=512, rope=64, page_size=64
     b.distribution = np.array([0, 0, n], np.int32)
     b.num_seqs = np.array([n], np.int32)
 
-    def enc(x):
-        if dtype == BF16:
-            raw = orc.f32_to_bf16_bits(x.astype(np.float32))
-            return raw, orc.bf16_bits_to_f32(raw).astype(np.float64)
+    def enc(x, tag=dtype):
         x = x.astype(np.float32)
+        if tag == BF16:
+            raw = orc.f32_to_bf16_bits(x)
+            return raw, orc.bf16_bits_to_f32(raw).astype(np.float64)
+        if tag == FP8:  # latent pages hold the plain cast: codes without scales
+            raw = orc.cast_e4m3fn_ref(x)
+            return raw, orc.e4m3fn_bits_to_f32(raw).astype(np.float64)
+        if tag == F16:
+            raw = x.astype(np.float16)
+            return raw, raw.astype(np.float64)
         return x, x.astype(np.float64)
 
+    kvenc = lambda x: enc(x, b.kv_dtype)
     normal = lambda *shape: rng.standard_normal(shape, dtype=np.float32)
     b.qn_raw, b.qn_val = enc(normal(b.T, Hq, lkv))
     b.qp_raw, b.qp_val = enc(normal(b.T, Hq, rope))
-    b.kv_raw, b.kv_val = enc(normal(b.T, lkv))
-    b.pe_raw, b.pe_val = enc(normal(b.T, rope))
+    b.kv_raw, b.kv_val = kvenc(normal(b.T, lkv))
+    b.pe_raw, b.pe_val = kvenc(normal(b.T, rope))
     if distinct_pages and distinct_pages < b.P:
-        raw, val = enc(normal(distinct_pages, page_size, b.row))
+        raw, val = kvenc(normal(distinct_pages, page_size, b.row))
         pick = np.arange(b.P) % distinct_pages
         b.pages_raw, b.pages_val = raw[pick], val[pick]
     else:
-        b.pages_raw, b.pages_val = enc(normal(b.P, page_size, b.row))  # padding holds noise: never read
+        b.pages_raw, b.pages_val = kvenc(normal(b.P, page_size, b.row))  # padding holds noise: never read
     return b
 
 
@@ -346,11 +354,12 @@ def run_gpu_mla(b, *, fused=True, softmax_aux=None, device="cuda:0", **kw):
     from easydel_amd import kernels
 
     t = lambda raw: to_torch(raw, b.q_dtype, device)
+    tk = lambda raw: to_torch(raw, b.kv_dtype, device)
     i32 = lambda a: torch.from_numpy(np.ascontiguousarray(a, np.int32)).to(device)
-    pages = t(b.pages_raw)
+    pages = tk(b.pages_raw)
     aux = None if softmax_aux is None else torch.from_numpy(np.asarray(softmax_aux, np.float32)).to(device)
     out, pages = kernels.mla_ragged_paged_attention(
-        t(b.qn_raw), t(b.qp_raw), t(b.kv_raw) if fused else None, t(b.pe_raw) if fused else None, pages,
+        t(b.qn_raw), t(b.qp_raw), tk(b.kv_raw) if fused else None, tk(b.pe_raw) if fused else None, pages,
         i32(b.context_lens), i32(b.block_tables), i32(b.query_start_loc), i32(b.distribution), softmax_aux=aux, **kw)
     torch.cuda.synchronize()
-    return from_torch(out, b.q_dtype), from_torch(pages, b.q_dtype)
+    return from_torch(out, b.q_dtype), from_torch(pages, b.kv_dtype)

@@ -89,7 +89,7 @@ def test_multi_latent_entry_points_validate_before_any_device_work():
 
     assert call(row=568) == _lib.RPA_ERR_INVALID_ARGUMENT and b"row_elems" in lib.rpa_last_error()
     assert call(rank=1024, row=2048) == _lib.RPA_ERR_UNSUPPORTED and b"kv_lora_rank" in lib.rpa_last_error()
-    assert call(kd=2) == _lib.RPA_ERR_UNSUPPORTED and b"kv_dtype" in lib.rpa_last_error()
+    assert call(kd=3) == _lib.RPA_ERR_UNSUPPORTED and b"kv_dtype" in lib.rpa_last_error()  # int8: the latent cache has no scales
     assert call(dist=None) == _lib.RPA_ERR_INVALID_ARGUMENT and b"distribution" in lib.rpa_last_error()
     assert call(qn=None) == _lib.RPA_ERR_INVALID_ARGUMENT and b"null pointer" in lib.rpa_last_error()
     assert call(kv=a, pe=None) == _lib.RPA_ERR_INVALID_ARGUMENT and b"keys_pe" in lib.rpa_last_error()
@@ -98,5 +98,5 @@ def test_multi_latent_entry_points_validate_before_any_device_work():
     assert call(T=0) == 0  # an empty batch is a no-op
     n = lib.rpa_mla_workspace_bytes(256, 256, 128, 64, 128, 512, 1, 1)
     assert n > 256 * 128 * 514 * 4  # at least one chunk's partial rows when the shapes ask for a split
-    assert lib.rpa_mla_page_scatter(None, a, a, a, a, a, a, a, 4, 2, 8, 16, 64, 512, 64, 640, 1) == _lib.RPA_ERR_UNSUPPORTED
+    assert lib.rpa_mla_page_scatter(None, a, a, a, a, a, a, a, 4, 2, 8, 16, 64, 512, 64, 640, 3) == _lib.RPA_ERR_UNSUPPORTED
     assert lib.rpa_mla_page_scatter(None, None, a, a, a, a, a, a, 4, 2, 8, 16, 64, 512, 64, 640, 2) == _lib.RPA_ERR_INVALID_ARGUMENT

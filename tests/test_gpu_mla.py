@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import rpa_testlib as tl
-from rpa_testlib import BF16, F32, orc
+from rpa_testlib import BF16, F16, F32, FP8, orc
 
 pytestmark = pytest.mark.gpu
 
@@ -35,6 +35,25 @@ def test_small_shapes_run_on_the_fp32_kernel(dtype):
     check(b, "small window+cap", softmax_scale=0.11, sliding_window=20, logits_soft_cap=5.0)
     check(b, "small read-only", fused=False)
     check(b, "small sinks", softmax_aux=np.array([0.5, -1.0, 2.0, 0.0]))
+
+
+@pytest.mark.parametrize("dtype,kv_dtype", [(BF16, FP8), (F32, FP8), (F16, F16), (F16, FP8), (BF16, F16), (F16, BF16)])
+def test_cast_only_fp8_and_float16_latent_pages(dtype, kv_dtype):
+    # the reference's latent cache takes any floating kvdtype and holds no scale arrays
+    # (caching/mla_ragged_page/cache.py:197-204, 344): fp8 pages are plain casts.  These formats run on the fp32 kernel.
+    b = make_mla_batch(11, [17, 64, 130, 255, 1], [1, 1, 8, 33, 1], Hq=4, lkv=64, rope=16, page_size=16, dtype=dtype,
+                       kv_dtype=kv_dtype, pad_rows=2, pad_tokens=3)
+    check(b, "formats small", softmax_scale=0.11)
+    check(b, "formats small window+cap", softmax_scale=0.11, sliding_window=20, logits_soft_cap=5.0)
+    check(b, "formats small read-only", fused=False)
+
+
+@pytest.mark.parametrize("dtype,kv_dtype", [(BF16, FP8), (F16, F16)])
+def test_fp8_and_float16_latent_pages_at_the_model_shape(dtype, kv_dtype):
+    rng = np.random.default_rng(12)
+    ctx = rng.integers(1, 900, size=6).tolist() + [300, 77]
+    b = make_mla_batch(13, ctx, [1] * 6 + [40, 77], Hq=16, dtype=dtype, kv_dtype=kv_dtype, pad_rows=1, pad_tokens=2)
+    check(b, "formats 512+64", softmax_scale=SCALE)
 
 
 def test_fp32_queries_at_the_model_shape():

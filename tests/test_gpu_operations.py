@@ -199,3 +199,59 @@ def test_mla_operation_follows_the_model_flow(gpu, name):
     err = np.abs(got - want)
     # the absorbed queries are rounded to bf16 once more than in the decompressed form; same bars as the kernel tests
     assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
+
+
+def test_mla_operation_casts_new_rows_into_an_fp8_latent_cache(gpu):
+    """An fp8 latent cache (kvdtype float8_e4m3fn; the cache carries no scales, caching/mla_ragged_page/cache.py:197-204):
+    the operation casts the model-dtype rows to the page dtype, the pages then hold the plain cast and attention reads the
+    codes' own values."""
+    from easydel_amd.caching import MLARaggedPagesCacheConfig, MLARaggedPagesCacheView
+
+    rng = np.random.default_rng(6)
+    heads, lkv, rope, page_size = 8, 512, 64, 64
+    scheduled, computed = [1, 1, 33], [200, 64, 31]
+    max_reqs, max_pages = 4, 4
+    n_pages = max_reqs * max_pages + 1
+    table = np.zeros((max_reqs, max_pages), dtype=np.int32)
+    perm = rng.permutation(np.arange(1, n_pages))
+    k = 0
+    for r in range(len(scheduled)):
+        need = -(-(computed[r] + scheduled[r]) // page_size)
+        table[r, :need] = perm[k:k + need]
+        k += need
+    cfg = MLARaggedPagesCacheConfig.create(torch.float8_e4m3fn, num_hidden_layers=1, num_kv_heads=heads, max_model_length=max_pages * page_size,
+                                           kv_lora_rank=lkv, qk_rope_head_dim=rope, page_size=page_size, num_pages=n_pages)
+    view = MLARaggedPagesCacheView.init(cfg, layer_index=0, device=gpu)
+    assert view.kv_pages.dtype == torch.float8_e4m3fn and tuple(view.kv_pages.shape) == (n_pages, page_size // 4, 4, 640)
+    sched_full = np.zeros(max_reqs, np.int32); sched_full[:len(scheduled)] = scheduled
+    comp_full = np.zeros(max_reqs, np.int32); comp_full[:len(computed)] = computed
+    fields = compute_ragged_batch_fields(scheduled_full=sched_full, active_mask_full=sched_full > 0, num_computed_tokens=comp_full,
+                                         page_table=table, version="v3", max_num_reqs=max_reqs, page_size=page_size)
+    meta = RaggedPagesMetadata.from_numpy(fields, version="v3", page_size=page_size, device=gpu)
+    T = int(sum(scheduled))
+    bf = lambda a: orc.bf16_bits_to_f32(orc.f32_to_bf16_bits(a.astype(np.float32))).astype(np.float64)  # noqa: E731
+    f8 = lambda a: orc.e4m3fn_bits_to_f32(orc.cast_e4m3fn_ref(a.astype(np.float32))).astype(np.float64)  # noqa: E731
+    q_abs, q_pe = bf(rng.standard_normal((T, heads, lkv))), bf(rng.standard_normal((T, heads, rope)))
+    latent, k_pe = bf(rng.standard_normal((T, lkv))), bf(rng.standard_normal((T, rope)))
+    pool = np.zeros((n_pages, page_size, 640))
+    pool[..., :lkv] = f8(rng.standard_normal((n_pages, page_size, lkv)))
+    pool[..., 512:576] = f8(rng.standard_normal((n_pages, page_size, rope)))
+    codes = orc.cast_e4m3fn_ref(pool.astype(np.float32))
+    view.kv_pages.view(torch.uint8).copy_(torch.from_numpy(codes).view(view.kv_pages.shape))
+    tt = lambda a: torch.from_numpy(a).to(torch.bfloat16).to(gpu)  # noqa: E731
+    op = OperationRegistry.create("multi_latent_ragged_page_attention_v1", OperationMetadata())
+    scale = (128 + rope) ** -0.5
+    out = op(queries_nope=tt(q_abs)[None], queries_pe=tt(q_pe)[None], keys_values=tt(latent)[None], keys_pe=tt(k_pe)[None],
+             cache_view=view, cache_metadata=meta, softmax_scale=scale, causal=True, mask_info=None)
+    torch.cuda.synchronize()
+    nseq = fields["request_distribution"][2:3]
+    pages = orc.mla_page_scatter_ref(f8(latent), f8(k_pe), pool, fields["context_lens"], table, fields["query_start_loc"], nseq)
+    got_pages = orc.e4m3fn_bits_to_f32(view.kv_pages.view(torch.uint8).view(n_pages, page_size, 640).cpu().numpy())
+    np.testing.assert_array_equal(got_pages, pages)
+    want = orc.mla_ragged_paged_attention_ref(q_abs, q_pe, pages, fields["context_lens"], table, fields["query_start_loc"], nseq,
+                                              kv_lora_rank=lkv, qk_rope_head_dim=rope, softmax_scale=scale)
+    got = out.attention_outputs[0].float().cpu().numpy().astype(np.float64)
+    err = np.abs(got - want)[:T]
+    big = np.abs(want[:T]) >= 4.0  # a bf16 output there is spaced wider than 2e-2: judged by one bf16 step instead
+    bound = np.where(big, 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want[:T]), 1e-30))) - 7), tl.TOL_BF16_MAX)
+    assert (err <= np.maximum(bound, tl.TOL_BF16_MAX)).all() and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
