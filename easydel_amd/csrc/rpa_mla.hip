@@ -373,7 +373,8 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   constexpr float kMaxSlack = 8.f;       // how far a score may exceed the softmax reference before it is raised
   static_assert(NW * RB * 16 == kMlaRows, "merge kernel assumes this row-tile height");
 
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[NSLOT * TILE];
+  constexpr int OFFW = NDMA * 256;       // bytes of a wave's table of load offsets (one dword per lane and instruction)
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[NSLOT * TILE + NW * OFFW];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -421,10 +422,10 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   const char* pages = (const char*)p.pages;
   const int pg = p.page_size;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
-  // (row, global chunk) of DMA instruction j for this lane; recomputed at every issue -- a few integer instructions
-  // against the hundred-odd MFMAs of a tile -- rather than held in eighteen registers
-  // (the lane number passes through an empty assembly statement at every issue, or the compiler would compute the
-  // offsets once before the loop after all and spill them)
+  // (row, global chunk) of DMA instruction j for this lane.  The offsets are the same for every tile whose rows are all
+  // visible: they wait in LDS, one dword per lane and instruction, and an issue reads them back (five reads against
+  // sixty integer instructions; registers to hold them the loop has none, and the lane number passes through an empty
+  // assembly statement at every issue, or the compiler would hoist reads and arithmetic out of the loop and spill them).
   int dma_lane = lane;
   auto dma_row = [&](int j) -> int { return (64 * (wave + NW * j) + dma_lane) / CPR; };
   auto dma_chunk = [&](int j, int r) -> int { return ((64 * (wave + NW * j) + dma_lane) - r * CPR) ^ mla_key(r); };
@@ -435,6 +436,14 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   int cur_slot = 0;
   auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
   int cur_page_raw = load_page(cur_idx);
+  {
+    uint32_t* off_w = (uint32_t*)(lds_all + NSLOT * TILE + wave * OFFW) + lane;
+#pragma unroll
+    for (int j = 0; j < NDMA; ++j) {
+      const int r = dma_row(j);
+      off_w[j * 64] = (uint32_t)r * (uint32_t)p.token_stride + (uint32_t)(dma_chunk(j, r) << 4);
+    }
+  }
   auto issue = [&]() __attribute__((always_inline)) {
     const int cur_page = min(max(cur_page_raw, 0), p.P - 1);
     const char* base = pages + (int64_t)cur_page * p.page_stride + (int64_t)cur_off * p.token_stride;
@@ -444,11 +453,14 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
     dma_lane = lane;
     asm volatile("" : "+v"(dma_lane));
     if (!edge) {
+      const uint32_t* off_r = (const uint32_t*)(lds_all + NSLOT * TILE + wave * OFFW) + dma_lane;
+      uint32_t voff[NDMA];
+#pragma unroll
+      for (int j = 0; j < NDMA; ++j) voff[j] = off_r[j * 64];
 #pragma unroll
       for (int j = 0; j < NDMA; ++j) {
         if (j == NDMA - 1 && !dma_full) break;
-        const int r = dma_row(j);
-        mla_dma16(dst + j * NW * 1024, (uint32_t)r * ts + (uint32_t)(dma_chunk(j, r) << 4), base);
+        mla_dma16(dst + j * NW * 1024, voff[j], base);
       }
     } else {
 #pragma unroll
