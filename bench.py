@@ -54,6 +54,9 @@ def parse_args():
     ap.add_argument("--read-probe", action="store_true",
                     help="instead of a workload: time the library's read-only probe over 8 GiB for 32..256 workgroups and "
                          "16..256 KiB in flight per workgroup, one line per setting")
+    ap.add_argument("--read-probe-paged", action="store_true",
+                    help="instead of a workload: time the paged read probe (the decode kernel's access pattern without its "
+                         "arithmetic: chunk size, split over the waves, load flavour, bytes in flight), one line per setting")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so a counter run shows what a known-size kernel reads")
     return ap.parse_args()
@@ -290,6 +293,41 @@ def read_probe():
                   flush=True)
 
 
+def read_probe_paged():
+    """What the memory system gives the decode kernel's access pattern without its arithmetic: rpa_read_probe_paged over
+    8 GiB (chunks visited in a scattered order, eight waves per chunk), best of four timed launches per setting."""
+    import torch
+
+    from easydel_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    buf = torch.empty(8 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    names = {0: "contiguous eighths, non-temporal loads", 1: "one head per wave, non-temporal loads", 2: "one head per wave, ordinary loads"}
+    for chunk_kib, split in ((16, 0), (64, 0), (64, 1), (64, 2), (256, 0), (256, 1), (256, 2)):
+        for wgs in (192, 256, 512):
+            for kib in (2, 4, 8, 16, 32):
+                if kib % (chunk_kib // 8):
+                    continue
+                best, read = None, 0
+                for rep in range(5):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(stream)
+                    read = lib.rpa_read_probe_paged(stream.cuda_stream, buf.data_ptr(), buf.numel(), wgs, kib, chunk_kib, split, sink.data_ptr())
+                    e1.record(stream)
+                    e1.synchronize()
+                    if read == 0:
+                        raise RuntimeError(lib.rpa_last_error().decode())
+                    ms = e0.elapsed_time(e1)
+                    if rep > 0 and (best is None or ms < best):
+                        best = ms
+                print(json.dumps({"probe": "read-paged", "chunk_kib": chunk_kib, "split": names[split], "workgroups": wgs,
+                                  "kib_in_flight_per_workgroup": 8 * kib, "ms": round(best, 4), "tb_per_s": round(read / best / 1e9, 3),
+                                  "gb_per_s_per_workgroup": round(read / best / 1e6 / wgs, 1)}), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -305,6 +343,8 @@ def main():
     _lib.load()
     if args.read_probe:
         return read_probe()
+    if args.read_probe_paged:
+        return read_probe_paged()
     if args.workload.startswith("mla-"):
         if args.mla_chunks:
             _lib.set_tunable("mla_chunks", args.mla_chunks)

@@ -24,6 +24,7 @@ SIGNATURES = {
     "rpa_set_tunable": (_c_int, [ctypes.c_char_p, _c_int]),
     "rpa_calibration_copy": (_c_int, [_c_vp, _c_vp, _c_vp, _c_sz]),
     "rpa_read_probe": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_vp]),
+    "rpa_read_probe_paged": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_int, _c_int, _c_vp]),
     "rpa_page_scatter_slices": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_i64, _c_int, _c_i64, _c_int]),
     "rpa_page_scatter_ragged": (_c_int, [_c_vp] * 8 + [_c_int] * 10),
     "rpa_attention_workspace_bytes": (_c_sz, [_c_int] * 9),

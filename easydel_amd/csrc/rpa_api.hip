@@ -17,6 +17,7 @@ int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const in
                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int);
 int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
 size_t launch_read_probe(hipStream_t, const void*, size_t, int, int, uint32_t*);
+size_t launch_read_probe_paged(hipStream_t, const void*, size_t, int, int, int, int, uint32_t*);
 int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
                                 const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int, int);
 }  // namespace rpa
@@ -194,6 +195,20 @@ size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int wo
   const size_t read = rpa::launch_read_probe((hipStream_t)stream, src, bytes, workgroups, kib_in_flight_per_wave, (uint32_t*)sink);
   if (read == 0)
     fail(RPA_ERR_INVALID_ARGUMENT, "rpa_read_probe: workgroups > 0, 2 / 4 / 8 / 16 / 32 KiB in flight per wave, and at least one round of loads per wave");
+  return read;
+}
+
+size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
+                            int chunk_kib, int split, void* sink) {
+  if (!src || !sink || ((uintptr_t)src & 15) || ((uintptr_t)sink & 3)) {
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_read_probe_paged: src must be 16-byte aligned and sink a 4-byte device word");
+    return 0;
+  }
+  const size_t read = rpa::launch_read_probe_paged((hipStream_t)stream, src, bytes, workgroups, kib_in_flight_per_wave, chunk_kib,
+                                                   split, (uint32_t*)sink);
+  if (read == 0)
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_read_probe_paged: workgroups > 0, chunk_kib a multiple of 8, 2 / 4 / 8 / 16 / 32 KiB in flight per wave "
+                                   "and a multiple of chunk_kib / 8, split 0..2, and at least one group of chunks per workgroup");
   return read;
 }
 

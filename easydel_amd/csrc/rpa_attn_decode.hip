@@ -140,8 +140,11 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
   auto issue = [&](auto buf, int tb, int page) {  // buf: std::integral_constant, so the register array index is static
     constexpr int B = decltype(buf)::value;
     const char* base = pages + (int64_t)page * p.page_stride + (int64_t)(tb % pg) * p.token_stride + lane_goff;
+    // Non-temporal loads: a decode step reads every cached key and value exactly once, and marked as a stream the pages
+    // come out of HBM a tenth faster than through ordinary loads (the paged read probe shows the same gap without any
+    // arithmetic: 89 % against 78 % of the peak for this very access pattern).
 #pragma unroll
-    for (int u = 0; u < NLD; ++u) stage[B][u] = *(const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride);
+    for (int u = 0; u < NLD; ++u) stage[B][u] = __builtin_nontemporal_load((const u32x4*)(base + (int64_t)(u * TPI) * p.token_stride));
     // a vector load on purpose: a scalar load would be waited for together with the next LDS read
     if constexpr (EB == 1) {
       if (p.kv_scales) sc_stage[B] = *(const u32x2*)(p.kv_scales + (int64_t)page * p.C + 2 * h);

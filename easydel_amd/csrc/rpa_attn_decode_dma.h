@@ -139,14 +139,14 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
     const bool edge = (i_tok + TT > ip.ctx) || (i_tok < ip.vis_lo);
     if (!edge) {
 #pragma unroll
-      for (int u = 0; u < NLH; ++u) dma16(lds + u * 1024, is_v ? voff_v[u] : voff_k[u], base);
+      for (int u = 0; u < NLH; ++u) dma16_nt(lds + u * 1024, is_v ? voff_v[u] : voff_k[u], base);
     } else {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {  // rows nobody may see: a visible row's bytes (same page: pages hold whole 64-token groups)
         const int row = u * RPI + dma_row0;
         const int r = min(max(i_tok + row, ip.vis_lo), ip.ctx - 1) - i_tok;
         const uint32_t off = (uint32_t)r * (uint32_t)p.token_stride + (uint32_t)((dma_c ^ (is_v ? key_v(row) : swz_key<RK>(row))) << 4);
-        dma16(lds + u * 1024, off, base);
+        dma16_nt(lds + u * 1024, off, base);
       }
     }
     ++n_issued;

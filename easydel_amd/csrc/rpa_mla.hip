@@ -337,6 +337,10 @@ __global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_sl
 __device__ __forceinline__ void mla_dma16(uint32_t lds_addr, uint32_t voff, const void* base) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
+// ... with the non-temporal hint: for rows no other workgroup will ask for (see `once` in the kernel)
+__device__ __forceinline__ void mla_dma16_nt(uint32_t lds_addr, uint32_t voff, const void* base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
 template <int N>
 __device__ __forceinline__ void mla_wait_loads_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
@@ -436,6 +440,10 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   int cur_slot = 0;
   auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
   int cur_page_raw = load_page(cur_idx);
+  // A sequence with a single row tile (a decode batch: one token's heads) has its latent rows read by this workgroup
+  // alone: they are streamed with the non-temporal hint, which reads HBM measurably faster.  The row tiles of a prompt
+  // share their rows through the L2 and load them the ordinary way.
+  const bool once = rows_total <= kMlaRows;
   {
     uint32_t* off_w = (uint32_t*)(lds_all + NSLOT * TILE + wave * OFFW) + lane;
 #pragma unroll
@@ -460,7 +468,8 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
 #pragma unroll
       for (int j = 0; j < NDMA; ++j) {
         if (j == NDMA - 1 && !dma_full) break;
-        mla_dma16(dst + j * NW * 1024, voff[j], base);
+        if (once) mla_dma16_nt(dst + j * NW * 1024, voff[j], base);
+        else mla_dma16(dst + j * NW * 1024, voff[j], base);
       }
     } else {
 #pragma unroll
@@ -468,7 +477,8 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
         if (j == NDMA - 1 && !dma_full) break;
         const int r = dma_row(j);
         const int rv = min(max(cur_tb + r, vis_lo), sp.ctx - 1) - cur_tb;
-        mla_dma16(dst + j * NW * 1024, (uint32_t)rv * ts + (uint32_t)(dma_chunk(j, r) << 4), base);
+        if (once) mla_dma16_nt(dst + j * NW * 1024, (uint32_t)rv * ts + (uint32_t)(dma_chunk(j, r) << 4), base);
+        else mla_dma16(dst + j * NW * 1024, (uint32_t)rv * ts + (uint32_t)(dma_chunk(j, r) << 4), base);
       }
     }
     cur_tb += TT;

@@ -30,6 +30,20 @@ size_t rpa_read_probe(rpa_stream_t stream, const void* src, size_t bytes, int wo
                       void* sink);
 
 /*
+ * The same reader over pages (no counterpart in the reference either): `src` is cut into chunks of `chunk_kib` KiB (a
+ * multiple of 8; their number is rounded down to a power of two), every workgroup visits an equal share of them in a
+ * scattered order, `kib_in_flight_per_wave` (2, 4, 8, 16 or 32, a multiple of chunk_kib / 8) KiB per wavefront in flight,
+ * i.e. kib_in_flight_per_wave / (chunk_kib / 8) chunks per workgroup.  `split` says how the eight wavefronts share a chunk:
+ * 0 contiguous eighths; 1 and 2 the way the decode kernels split a page -- the chunk is rows of 4 KiB (a token's keys and
+ * values of eight heads) and wavefront w reads bytes [512 w, 512 w + 512) of every row, two rows per instruction -- with
+ * non-temporal (1) or ordinary (2) loads.  It is the access pattern of the decode kernel over a page pool without its
+ * arithmetic: what separates 1 from 2 is what the non-temporal hint is worth to that kernel.  Returns the bytes the
+ * launch reads, 0 on bad arguments.
+ */
+size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
+                            int chunk_kib, int split, void* sink);
+
+/*
  * Knobs for tests and measurement.  They belong to the calling thread: a value set here is seen only by entry points
  * the same thread calls afterwards (each call reads them once, when it starts), so threads that never call this function
  * always run with the defaults.  Returns the previous value, -1 for an unknown name.

@@ -70,6 +70,10 @@ def test_host_only_entry_points():
     assert lib.rpa_read_probe(None, a, 1 << 30, 256, 3, a) == 0  # 2 / 4 / 8 / 16 / 32 KiB in flight per wave
     assert lib.rpa_read_probe(None, a, 1 << 30, 0, 8, a) == 0
     assert lib.rpa_read_probe(None, a, 4096, 256, 8, a) == 0  # less than one round of loads per wave
+    assert lib.rpa_read_probe_paged(None, None, 1 << 30, 256, 8, 64, 1, None) == 0 and b"rpa_read_probe_paged" in lib.rpa_last_error()
+    assert lib.rpa_read_probe_paged(None, a, 1 << 30, 256, 4, 64, 1, a) == 0  # a wave's eighth of a 64 KiB chunk is 8 KiB
+    assert lib.rpa_read_probe_paged(None, a, 1 << 30, 256, 8, 60, 0, a) == 0  # chunk_kib a multiple of 8
+    assert lib.rpa_read_probe_paged(None, a, 1 << 30, 256, 8, 64, 3, a) == 0  # split 0..2
     prev = _lib.set_tunable("max_splits", 4)
     assert lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1) < n
     _lib.set_tunable("max_splits", prev)
