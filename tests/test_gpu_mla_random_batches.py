@@ -1,6 +1,7 @@
 """GPU parity of the multi-latent attention entry point on seeded random ragged batches: every seed draws its own head
 count, page size and query dtype, a mix of decode, multi-token, chunked-prefill, whole-prompt and empty rows, padding,
-and optionally a sliding window, a soft cap, sinks and the read-only call, and is checked against the float64 oracle
+and optionally a sliding window, a soft cap, sinks, the read-only call and latent pages of another format than the
+queries' (cast-only fp8, float16, bfloat16), and is checked against the float64 oracle
 through the C ABI (fused write bit-exact; output to 1e-5 in fp32, 2e-2 max-abs / 5e-3 mean-abs in bf16, one bf16 step where an
 output passes |4|)."""
 
@@ -10,7 +11,7 @@ import numpy as np
 import pytest
 
 import rpa_testlib as tl
-from rpa_testlib import BF16, F32, make_mla_batch, mla_oracle, run_gpu_mla
+from rpa_testlib import BF16, F16, F32, FP8, make_mla_batch, mla_oracle, run_gpu_mla
 
 pytestmark = pytest.mark.gpu
 
@@ -42,7 +43,13 @@ def test_random_mla_batch(gpu, seed):
         ctx.append(c); q_lens.append(q)
     if sum(q_lens) == 0:
         q_lens[0], ctx[0] = 1, max(ctx[0], 1)
-    b = make_mla_batch(6000 + seed, ctx, q_lens, Hq=Hq, page_size=page_size, dtype=dtype,
+    # a generator of its own, so that a seed keeps the batch it always had: one seed in four holds its latent rows in
+    # another format (these run on the fp32 kernel, like every page format but the bf16 queries' own)
+    fmt = np.random.default_rng(7000 + seed)
+    kv_dtype = None
+    if Hq <= 32 and fmt.random() < 0.25:
+        dtype, kv_dtype = [(BF16, FP8), (F32, FP8), (F16, F16), (F16, FP8), (BF16, F16), (F16, BF16)][int(fmt.integers(0, 6))]
+    b = make_mla_batch(6000 + seed, ctx, q_lens, Hq=Hq, page_size=page_size, dtype=dtype, kv_dtype=kv_dtype,
                        pad_rows=int(rng.integers(0, 4)), pad_tokens=int(rng.integers(0, 6)), max_pages=-(-3000 // page_size))
     kw = {"softmax_scale": (128 + 64) ** -0.5}
     if rng.random() < 0.4:
@@ -53,7 +60,7 @@ def test_random_mla_batch(gpu, seed):
         kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * (128 + 64) ** -0.5
     aux = rng.uniform(-3.0, 7.0, size=Hq).astype(np.float32) if rng.random() < 0.4 else None
     fused = bool(rng.random() < 0.75)
-    what = f"seed {seed}: Hq{Hq} pg{page_size} dtype{dtype} ctx {ctx} q {q_lens} fused={fused} sinks={aux is not None} {sorted(kw)}"
+    what = f"seed {seed}: Hq{Hq} pg{page_size} dtype{dtype} pages{kv_dtype} ctx {ctx} q {q_lens} fused={fused} sinks={aux is not None} {sorted(kw)}"
     print(what, flush=True)
     want, want_pages = mla_oracle(b, fused=fused, softmax_aux=aux, **kw)
     got, got_pages = run_gpu_mla(b, fused=fused, softmax_aux=aux, **kw)
