@@ -50,6 +50,12 @@ def parse_args():
     ap.add_argument("--max-splits", type=int, default=0)
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
+    ap.add_argument("--mla-uniform-context", type=int, default=0,
+                    help="multi-latent decode workloads: every sequence this long (with --mla-chunks 1: one equal unit of "
+                         "work per sequence, which separates the cost of a tile from the cost of a unit and of imbalance)")
+    ap.add_argument("--mla-distinct-pages", type=int, default=0,
+                    help="multi-latent decode workloads: the block tables name only this many different pages, so that the "
+                         "latent rows come out of the L2 instead of HBM (what the kernel costs with memory taken away)")
     ap.add_argument("--sequential-pages", action="store_true", help="experiment: block tables in pool order")
     ap.add_argument("--read-probe", action="store_true",
                     help="instead of a workload: time the library's read-only probe over 8 GiB for 32..256 workgroups and "
@@ -193,6 +199,8 @@ def bench_mla(args):
         Hq, n = (128 if args.workload.endswith("h128") else 16), 256
         q_lens = np.ones(n, np.int32)
         ctx = rng.integers(512, 8193, size=n).astype(np.int32)
+        if args.mla_uniform_context > 0:
+            ctx[:] = args.mla_uniform_context
     need = -(-ctx // pg)
     M = int(need.max())
     P = int(need.sum()) + 64
@@ -202,6 +210,8 @@ def bench_mla(args):
     for i, m in enumerate(need):
         bt[i, :m] = perm[k:k + m]
         k += m
+    if args.mla_distinct_pages > 0 and args.workload != "mla-prefill-h128":
+        bt = (bt % args.mla_distinct_pages).astype(np.int32)
     T = int(q_lens.sum())
     qsl = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
     g = torch.Generator(device=dev).manual_seed(args.seed)
@@ -258,7 +268,8 @@ def bench_mla(args):
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "sequences": n, "query_tokens": T, "q_heads": Hq, "kv_lora_rank": lkv,
                    "qk_rope_head_dim": rope, "page_row_elems": row, "page_size": pg, "pool_pages": P,
-                   "context_tokens_total": int(ctx.sum()), "context_range": [int(ctx.min()), int(ctx.max())], "seed": args.seed},
+                   "context_tokens_total": int(ctx.sum()), "context_range": [int(ctx.min()), int(ctx.max())], "seed": args.seed,
+                   "distinct_pages_in_block_tables": args.mla_distinct_pages or None},
         "roofline": roofline, "cpu_baseline": None,
     }))
 
