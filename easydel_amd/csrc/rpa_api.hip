@@ -38,7 +38,7 @@ struct Tunables {
   int force_generic = 0;
   int prefill_dma = 1;
   int decode_pace = 1;
-  int decode_dma = -1;     // -1: where it measured faster (head size 256); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
+  int decode_dma = -1;     // -1: where it measured faster (head size 256; int8 pages); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
   int mla_chunks = 0;      // 0 = sized from the shapes
   int mla_min_chunk = 0;   // 0 = default
   int stages = 15;         // bit 0: decode plan, 1: decode kernel, 2: prefill / large-row kernel, 3: merge
@@ -349,7 +349,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.decode_sync = tun.decode_sync;
   p.prefill_dma = tun.prefill_dma;
   p.decode_pace = tun.decode_pace;
-  p.decode_dma = tun.decode_dma < 0 ? (p.D == 256 ? 1 : 0) : tun.decode_dma;
+  p.decode_dma = tun.decode_dma < 0 ? ((p.D == 256 || p.kv_dtype == RPA_INT8) ? 1 : 0) : tun.decode_dma;
   p.max_splits = 2;
   p.pre_chunk = 1 << 30;
   p.pre_max_chunks = 1;

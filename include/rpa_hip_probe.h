@@ -55,7 +55,7 @@ size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, 
  *                    tiles in flight pauses once (512 clocks) before issuing its own; 0: never
  *   "decode_dma"     which decode batches (bf16 / float16 pages, fp8 / int8 pages at head size 128; pages of a multiple
  *                    of 64 tokens, four or more KV heads) run on the LDS-direct decode kernel, two tiles in flight per
- *                    wave: -1 (default) 16-bit pages of head size 256, where it measured faster; 0 none; 1 all; 2 all,
+ *                    wave: -1 (default) 16-bit pages of head size 256 and int8 pages, where it measured faster; 0 none; 1 all; 2 all,
  *                    with one tile in flight; 3 all, the K rows of a tile requested together with its V rows (later than
  *                    they could be, but the two halves of each token's bytes then reach the memory side by side)
  *   "prefill_chunks" 0 (default): the key chunks of a prefill row tile are sized on the device from the lengths in the
