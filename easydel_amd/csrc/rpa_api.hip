@@ -136,17 +136,22 @@ int decode_token_bound(int T, int S, int Hq, int Hkv, int dec_rows) {
 // holds few row tiles and evens out sequences of different lengths; every chunk of a row costs a float32 partial
 // row (lkv + 2 floats) written and read back, which with many heads per token is comparable to the keys themselves,
 // hence the longer minimum there.  The partial buffers stay under ~1 GiB.
-void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* min_chunk) {
+void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* rule_chunks, int* min_chunk) {
   // Row tiles a batch of this shape typically holds (a bound it is not: a call may put all its tokens into one row).
   // About 400 units of work, 1.5 per CU, measured best on decode batches of 32 ... 1 024 sequences at 16 and at 128
   // heads: fewer leave CUs idle or the lengths uneven, more pay for their partial rows and their start.
   const long tiles = std::max((long)S, (long)T * Hq / rpa::kMlaRows);
-  long chunks = g_tun.mla_chunks > 0 ? g_tun.mla_chunks : (400 + tiles / 2) / tiles;
-  if (chunks > rpa::kMlaMaxChunks) chunks = rpa::kMlaMaxChunks;
-  if (chunks < 1) chunks = 1;
+  long rule = g_tun.mla_chunks > 0 ? g_tun.mla_chunks : (400 + tiles / 2) / tiles;
+  if (rule > rpa::kMlaMaxChunks) rule = rpa::kMlaMaxChunks;
+  if (rule < 1) rule = 1;
+  // The partial buffers hold more chunks than that where they are cheap (up to 256 MiB in all), for the batches the
+  // plan kernel cuts by length: their rows may be far fewer than the shapes allow.  A set knob is taken literally.
   const size_t per = part_o_bytes(T, Hq, lkv) + part_ml_bytes(T, Hq);
+  long chunks = rule;
+  if (g_tun.mla_chunks <= 0) chunks = std::max(rule, std::min((long)rpa::kMlaMaxChunks, (long)(((size_t)256 << 20) / std::max(per, (size_t)1))));
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   *max_chunks = (int)chunks;
+  *rule_chunks = (int)std::min(rule, chunks);
   *min_chunk = g_tun.mla_min_chunk > 0 ? g_tun.mla_min_chunk : (Hq >= 64 ? 1024 : 512);
 }
 
@@ -541,8 +546,8 @@ int rpa_ragged_paged_attention_v3_quantised(rpa_stream_t stream, const void* q, 
 size_t rpa_mla_workspace_bytes(int T, int S, int M, int page_size, int Hq, int kv_lora_rank, int q_dtype, int kv_dtype) {
   (void)M; (void)page_size; (void)q_dtype; (void)kv_dtype;
   if (T <= 0 || S <= 0 || Hq <= 0 || kv_lora_rank <= 0) return 256;
-  int chunks, min_chunk;
-  mla_split(T, S, Hq, kv_lora_rank, &chunks, &min_chunk);
+  int chunks, rule_chunks, min_chunk;
+  mla_split(T, S, Hq, kv_lora_rank, &chunks, &rule_chunks, &min_chunk);
   return (chunks > 1 ? (size_t)chunks * (part_o_bytes(T, Hq, kv_lora_rank) + part_ml_bytes(T, Hq)) : 0) +
          rpa::mla_plan_bytes(T, S, Hq, chunks) + 512;
 }
@@ -570,6 +575,7 @@ static int mla_fill(const char* who, rpa::MlaParams& p, const void* keys_values,
   p.page_stride = p.token_stride * page_size;
   p.kv_dtype = kv_dtype;
   p.max_chunks = 1;
+  p.rule_chunks = 1;
   p.min_chunk = 512;
   return RPA_OK;
 }
@@ -627,8 +633,8 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
     if (err) return hip_fail(err, "MLA page write launch");
   }
   if (p.mfma) {
-    int chunks, min_chunk;
-    mla_split(T, S, Hq, kv_lora_rank, &chunks, &min_chunk);
+    int chunks, rule_chunks, min_chunk;
+    mla_split(T, S, Hq, kv_lora_rank, &chunks, &rule_chunks, &min_chunk);
     const size_t po = part_o_bytes(T, Hq, kv_lora_rank), pml = part_ml_bytes(T, Hq);
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     // the plan is sized for the chunks the shapes ask for; a small workspace then gets fewer, longer chunks
@@ -639,7 +645,10 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
     if ((size_t)chunks * (po + pml) > usable) chunks = (int)(usable / (po + pml));
     if (chunks < 2) chunks = 1;  // a single chunk writes its rows directly and needs no partial buffers
     p.max_chunks = chunks;
+    p.rule_chunks = std::min(rule_chunks, chunks);
     p.min_chunk = min_chunk;
+    p.auto_chunk = g_tun.mla_chunks <= 0 && g_tun.mla_min_chunk <= 0;  // set knobs are taken literally
+    p.cus = device_cus();
     const size_t slots = (size_t)rpa::mla_plan_slots(T, S, Hq);
     p.plan = (int2*)base;
     p.n_units = (int32_t*)(base + align256(slots * 8));

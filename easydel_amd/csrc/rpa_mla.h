@@ -27,7 +27,9 @@ struct MlaParams {
   int2* plan;      // [row-tile slots] (sequence, key chunks | keys / 64 of a chunk << 8) of the row tile at a slot;
                    // chunks = 0: no such tile
   int32_t* n_units;  // [0] number of (row tile, key chunk) units of the batch = workgroups with work;
-                     // [1] 1 if the list is sorted longest first, 0 if it is in slot order
+                     // [1] 1 if the list is sorted longest first, 0 if it is in slot order;
+                     // [2] chunk length the plan kernel chose for this batch (keys, a multiple of 64), 0: the cut
+                     //     follows rule_chunks / min_chunk
   int2* units;     // [n_units[0]] (slot, chunk)
   int T, S, M, P, page_size, Hq, lkv, rope, rope_off, row_elems;
   int64_t token_stride, page_stride;  // bytes
@@ -36,7 +38,10 @@ struct MlaParams {
   int window;
   float softcap;
   int max_chunks;  // chunks the partial buffers hold; 1 = never split
-  int min_chunk;   // fewest keys per chunk (multiple of 64)
+  int rule_chunks; // chunks a row tile is cut into when the cut follows the shapes (<= max_chunks)
+  int min_chunk;   // fewest keys per chunk then (multiple of 64)
+  int auto_chunk;  // 1: the plan kernel may choose a chunk length from the batch's own lengths (n_units[2])
+  int cus;         // compute units of the device
   int mfma;        // 1: every row served by the MFMA kernel; 0: by the fp32 kernel
 };
 
@@ -56,14 +61,30 @@ __device__ __forceinline__ MlaSeq mla_seq(const MlaParams& p, int i) {
   return s;
 }
 
+// How a row tile's `span` keys are cut: n_chunks chunks of `chunk` keys (a multiple of 64).  With a chunk length L
+// chosen by the plan kernel (small batches): as many even chunks as L asks for and the partial buffers hold; else as
+// even as rule_chunks allows and never shorter than min_chunk.
+__device__ __forceinline__ void mla_cut(const MlaParams& p, int span, int L, int* chunk, int* n_chunks) {
+  *chunk = p.min_chunk;
+  *n_chunks = 0;
+  if (span <= 0) return;
+  if (L > 0) {
+    const int n = min(p.max_chunks, (span + L - 1) / L);
+    *chunk = (((span + n - 1) / n) + 63) & ~63;
+  } else {
+    const int even = (((span + p.rule_chunks - 1) / p.rule_chunks) + 63) & ~63;
+    *chunk = max(p.min_chunk, even);
+  }
+  *n_chunks = (span + *chunk - 1) / *chunk;
+}
+
 // Key range [kv_lo, kv_hi) the row tile [R0, R0 + kMlaRows) of a sequence must visit (kv_lo rounded down to 64), the
-// lowest key any of its rows sees, and how the range is cut: n_chunks chunks of `chunk` keys (a multiple of 64), as
-// even as the bound max_chunks allows and never shorter than min_chunk.  The attention kernel and the merge kernel
-// both derive the cut from this one function.
+// lowest key any of its rows sees, and how the range is cut (mla_cut; L = n_units[2] of the batch's plan).  The plan,
+// the attention kernel and the merge kernel all derive the cut from this one function.
 struct MlaTile {
   int kv_lo, kv_hi, vis_lo, chunk, n_chunks;
 };
-__device__ __forceinline__ MlaTile mla_tile(const MlaParams& p, const MlaSeq& sp, int R0) {
+__device__ __forceinline__ MlaTile mla_tile(const MlaParams& p, const MlaSeq& sp, int R0, int L) {
   MlaTile t;
   const int rows_total = sp.q_len * p.Hq;
   const int last_row = min(R0 + kMlaRows, rows_total) - 1;
@@ -71,14 +92,7 @@ __device__ __forceinline__ MlaTile mla_tile(const MlaParams& p, const MlaSeq& sp
   t.kv_hi = min(sp.ctx, base_pos + last_row / p.Hq + 1);
   t.vis_lo = (p.window > 0) ? max(base_pos + R0 / p.Hq - p.window + 1, 0) : 0;
   t.kv_lo = t.vis_lo & ~63;
-  const int span = t.kv_hi - t.kv_lo;
-  t.chunk = p.min_chunk;
-  t.n_chunks = 0;
-  if (span > 0) {
-    const int even = (((span + p.max_chunks - 1) / p.max_chunks) + 63) & ~63;
-    t.chunk = max(p.min_chunk, even);
-    t.n_chunks = (span + t.chunk - 1) / t.chunk;
-  }
+  mla_cut(p, t.kv_hi - t.kv_lo, L, &t.chunk, &t.n_chunks);
   return t;
 }
 

@@ -153,25 +153,32 @@ __global__ __launch_bounds__(64) void mla_generic_kernel(MlaParams p) {
   }
 }
 
-// What row-tile slot `slot` of the matrix-core kernel's grid holds: (sequence, key chunks | keys / 64 of a chunk << 8),
-// chunks = 0 where there is no tile.
+// The row tile at slot `slot` of the matrix-core kernel's grid: its sequence and the keys it must visit (0: no tile).
 // `qsl` is query_start_loc, or a copy of its first n_live + 1 entries that is quicker to search.
-__device__ __forceinline__ int2 mla_plan_slot(const MlaParams& p, int slot, const int32_t* qsl) {
-  int2 unit = {0, 0};
+__device__ __forceinline__ int mla_slot_span(const MlaParams& p, int slot, const int32_t* qsl, int* seq) {
+  *seq = 0;
   const int n_live = mla_live_rows(p);
-  if (n_live > 0) {
-    int lo_i = 0, hi_i = n_live;  // the last sequence starting at or before `slot`
-    while (hi_i - lo_i > 1) {
-      const int mid = (lo_i + hi_i) >> 1;
-      if ((int)(((int64_t)qsl[mid] * p.Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
-    }
-    const MlaSeq sp = mla_seq(p, lo_i);
-    const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * p.Hq) / kMlaRows) + lo_i);
-    if (sp.live && tile_in_seq >= 0 && tile_in_seq * kMlaRows < sp.q_len * p.Hq) {
-      const MlaTile mt = mla_tile(p, sp, tile_in_seq * kMlaRows);
-      unit.x = lo_i;
-      unit.y = mt.n_chunks | ((min(mt.chunk, mt.kv_hi - mt.kv_lo) >> 6) << 8);  // chunks, and keys / 64 of one chunk
-    }
+  if (n_live <= 0) return 0;
+  int lo_i = 0, hi_i = n_live;  // the last sequence starting at or before `slot`
+  while (hi_i - lo_i > 1) {
+    const int mid = (lo_i + hi_i) >> 1;
+    if ((int)(((int64_t)qsl[mid] * p.Hq) / kMlaRows) + mid <= slot) lo_i = mid; else hi_i = mid;
+  }
+  const MlaSeq sp = mla_seq(p, lo_i);
+  const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * p.Hq) / kMlaRows) + lo_i);
+  if (!sp.live || tile_in_seq < 0 || tile_in_seq * kMlaRows >= sp.q_len * p.Hq) return 0;
+  const MlaTile mt = mla_tile(p, sp, tile_in_seq * kMlaRows, 0);
+  *seq = lo_i;
+  return max(mt.kv_hi - mt.kv_lo, 0);
+}
+// What the plan holds for such a tile: (sequence, key chunks | keys / 64 of a chunk << 8), chunks = 0 where there is none.
+__device__ __forceinline__ int2 mla_plan_entry(const MlaParams& p, int seq, int span, int L) {
+  int2 unit = {0, 0};
+  if (span > 0) {
+    int chunk, n_chunks;
+    mla_cut(p, span, L, &chunk, &n_chunks);
+    unit.x = seq;
+    unit.y = n_chunks | ((min(chunk, span) >> 6) << 8);
   }
   return unit;
 }
@@ -190,7 +197,9 @@ __global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots,
   }
   const int slot = blockIdx.x * 256 + threadIdx.x;
   if (slot >= n_slots) return;
-  p.plan[slot] = mla_plan_slot(p, slot, p.qsl);
+  int seq;
+  const int span = mla_slot_span(p, slot, p.qsl, &seq);
+  p.plan[slot] = mla_plan_entry(p, seq, span, 0);
 }
 
 // Small batches (up to kMlaSortSlots slots): plan and unit list in one launch of one block -- thread t looks up slots
@@ -213,16 +222,52 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   for (int k = tid; k <= min(mla_live_rows(p), kMlaSortSlots); k += 1024) qsl_s[k] = p.qsl[k];
   __syncthreads();
+  // A batch of few row tiles (a quarter of the CUs or fewer: a small decode batch) is cut by length, not by count: every
+  // tile into chunks of about L keys, L such that the whole batch makes at most one unit per CU -- sum(ceil(span / L))
+  // <= W / L + R <= CUs for L = W / (CUs - R), W the keys of all R tiles.  One round of near-equal units then takes
+  // what one chunk takes, where even cuts of every tile leave units as different as the sequences are long.
+  __shared__ long long wave_w[16];
+  __shared__ int wave_r[16];
+  int seq_k[PER], span_k[PER];
+  long long w_keys = 0;
+  int tiles = 0;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int slot = tid * PER + k;
+    seq_k[k] = 0;
+    span_k[k] = slot < n_slots ? mla_slot_span(p, slot, qsl_s, &seq_k[k]) : 0;
+    w_keys += span_k[k];
+    tiles += span_k[k] > 0;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    w_keys += __shfl_xor(w_keys, o);
+    tiles += __shfl_xor(tiles, o);
+  }
+  if (lane == 0) {
+    wave_w[wv] = w_keys;
+    wave_r[wv] = tiles;
+  }
+  __syncthreads();
+  w_keys = 0;
+  tiles = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) {
+    w_keys += wave_w[w];
+    tiles += wave_r[w];
+  }
+  int L = 0;
+  if (p.auto_chunk && p.max_chunks > 1 && tiles > 0 && 4 * tiles <= p.cus) {
+    const long long even = (w_keys + (p.cus - tiles) - 1) / (p.cus - tiles);
+    L = (int)min(max((even + 63) & ~63ll, 128ll), (long long)1 << 30);
+  }
   int y[PER];
   int max_len = 0;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
     const int slot = tid * PER + k;
-    int2 unit = {0, 0};
-    if (slot < n_slots) {
-      unit = mla_plan_slot(p, slot, qsl_s);
-      p.plan[slot] = unit;
-    }
+    const int2 unit = mla_plan_entry(p, seq_k[k], span_k[k], L);
+    if (slot < n_slots) p.plan[slot] = unit;
     y[k] = unit.y;
     if (y[k] & 0xff) max_len = max(max_len, y[k] >> 8);
   }
@@ -287,6 +332,7 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
   if (tid == 0) {
     p.n_units[0] = total;
     p.n_units[1] = 1;
+    p.n_units[2] = L;
   }
 }
 
@@ -328,6 +374,7 @@ __global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_sl
   if (tid == 0) {
     p.n_units[0] = running_s;
     p.n_units[1] = 0;
+    p.n_units[2] = 0;
   }
 }
 
@@ -407,7 +454,7 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   const int rows_total = sp.q_len * Hq;
   const int R0 = tile_in_seq * kMlaRows;
 
-  const MlaTile mt = mla_tile(p, sp, R0);
+  const MlaTile mt = mla_tile(p, sp, R0, p.n_units[2]);
   const int base_pos = sp.ctx - sp.q_len;
   const int vis_lo = mt.vis_lo;
   // the first tile must hold vis_lo, so that rows of it that nobody may see can borrow a visible row's address
@@ -773,7 +820,7 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(MlaParams p) {
     if (!sp.live) zero = true;
     else if (p.mfma && p.max_chunks > 1) {
       const int row = (t - sp.q0) * p.Hq + hq;
-      n_pieces = mla_tile(p, sp, (row / kMlaRows) * kMlaRows).n_chunks;
+      n_pieces = mla_tile(p, sp, (row / kMlaRows) * kMlaRows, p.n_units[2]).n_chunks;
     }
   }
   const bool merge = n_pieces > 1;
@@ -839,7 +886,7 @@ __global__ __launch_bounds__(256, 4) void mla_merge_pair_kernel(MlaParams p) {
 #pragma unroll
       for (int hh = 0; hh < HPW; ++hh) {  // the two heads can lie in different row tiles
         const int row = (t - sp.q0) * p.Hq + hq0 + hh;
-        const int n = mla_tile(p, sp, (row / kMlaRows) * kMlaRows).n_chunks;
+        const int n = mla_tile(p, sp, (row / kMlaRows) * kMlaRows, p.n_units[2]).n_chunks;
         n_p[hh] = n > 1 ? n : 0;  // a row in one piece was written by the kernel that computed it
       }
     }

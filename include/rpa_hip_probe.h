@@ -64,7 +64,8 @@ size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, 
  *   "prefill_dma"    1 (default): prefill tiles are loaded global -> LDS by the load unit where those kernels apply
  *                    (page_size % 32 == 0); 0: every prefill tile is staged through registers (bf16 / 8-bit pages only)
  *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
- *                    the shapes); set it before sizing the workspace
+ *                    the shapes, and batches of few row tiles cut by a chunk length chosen on the device from their
+ *                    own lengths); set it before sizing the workspace
  *   "mla_min_chunk"  fewest keys of such a chunk (rounded up to 64; 0 = default: 1024 at 64 heads and more, else 512)
  *   "force_generic"  non-zero: route every call through the fp32 VALU kernel
  *   "stages"         bit mask of the attention call's launches, for profiling one kernel in isolation:
