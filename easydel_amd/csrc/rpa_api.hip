@@ -145,10 +145,12 @@ void mla_split(int T, int S, int Hq, int lkv, int* max_chunks, int* rule_chunks,
   if (rule > rpa::kMlaMaxChunks) rule = rpa::kMlaMaxChunks;
   if (rule < 1) rule = 1;
   // The partial buffers hold more chunks than that where they are cheap (up to 256 MiB in all), for the batches the
-  // plan kernel cuts by length: their rows may be far fewer than the shapes allow.  A set knob is taken literally.
+  // plan kernel cuts by length: a call of few tokens whose sequence rows are mostly empty (its row tiles number at
+  // least T * Hq / 128, and a quarter of the CUs at most for that cut).  A set knob is taken literally.
   const size_t per = part_o_bytes(T, Hq, lkv) + part_ml_bytes(T, Hq);
   long chunks = rule;
-  if (g_tun.mla_chunks <= 0) chunks = std::max(rule, std::min((long)rpa::kMlaMaxChunks, (long)(((size_t)256 << 20) / std::max(per, (size_t)1))));
+  if (g_tun.mla_chunks <= 0 && (long)T * Hq / rpa::kMlaRows <= std::max(device_cus(), 4) / 4)
+    chunks = std::max(rule, std::min((long)rpa::kMlaMaxChunks, (long)(((size_t)256 << 20) / std::max(per, (size_t)1))));
   while (chunks > 1 && (size_t)chunks * per > ((size_t)1 << 30)) --chunks;
   *max_chunks = (int)chunks;
   *rule_chunks = (int)std::min(rule, chunks);
