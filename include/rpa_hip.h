@@ -272,7 +272,8 @@ int rpa_mla_ragged_paged_attention(rpa_stream_t stream, const void* queries_nope
                                    int kv_dtype, float softmax_scale, int sliding_window, float logits_soft_cap,
                                    const float* softmax_aux);
 
-/* Workspace the call above needs, from the static bounds alone. */
+/* Workspace the call above needs, from the static bounds alone (and the compute-unit count of the current device;
+ * a call handed fewer bytes cuts its rows into fewer, longer key chunks, down to none). */
 size_t rpa_mla_workspace_bytes(int T, int S, int M, int page_size, int Hq, int kv_lora_rank, int q_dtype, int kv_dtype);
 
 /*
