@@ -207,6 +207,7 @@ __global__ __launch_bounds__(256) void mla_plan_kernel(MlaParams p, int n_slots,
 // scan over eight counters instead of one scan per class.  Blocks behind the first write the new rows, as above.
 constexpr int kMlaSortSlots = 4096;
 constexpr int kMlaLenClasses = 8;
+constexpr int kMlaRankSlots = 512;  // lists up to this many slots are sorted exactly
 __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int n_slots) {
   constexpr int PER = kMlaSortSlots / 1024, NC = kMlaLenClasses;
   if (blockIdx.x > 0) {
@@ -277,6 +278,45 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
   __syncthreads();
 #pragma unroll
   for (int w = 0; w < 16; ++w) max_len = max(max_len, wave_max_s[w]);
+  // A list of up to kMlaRankSlots slots (the decode batches: a unit is a large share of a CU's work there, and the order
+  // inside a length class, which is slot order, costs 5 % of such a call) is sorted exactly: every slot's (chunk length,
+  // slot, chunks) goes to LDS as one key, thread t counts the units of all slots that come before slot t -- longer
+  // chunks, or as long and a lower slot -- and writes slot t's units there.
+  if (n_slots <= kMlaRankSlots) {
+    __shared__ uint32_t key_s[kMlaRankSlots];
+    const unsigned len_div = max_len < 32768 ? 1u : (unsigned)(max_len / 32767 + 1);  // chunk lengths / 64 into 15 bits
+#pragma unroll
+    for (int k = 0; k < PER; ++k) {
+      const int slot = tid * PER + k;
+      if (slot < n_slots)
+        key_s[slot] = (y[k] & 0xff) ? ((((unsigned)(y[k] >> 8) / len_div) << 17) | ((unsigned)(kMlaRankSlots - 1 - slot) << 8) | (unsigned)(y[k] & 0xff)) : 0u;
+    }
+    __syncthreads();
+    if (tid < 64) {  // the first wave adds up the units while the others place them
+      int t = 0;
+      for (int s2 = lane; s2 < n_slots; s2 += 64) t += (int)(key_s[s2] & 0xff);
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o);
+      if (lane == 0) {
+        p.n_units[0] = t;
+        p.n_units[1] = 1;
+        p.n_units[2] = L;
+      }
+    }
+    if (tid < n_slots) {
+      const uint32_t mine = key_s[tid];
+      const int v = (int)(mine & 0xff);
+      if (v > 0) {
+        int at = 0;
+        for (int s2 = 0; s2 < n_slots; ++s2) {
+          const uint32_t o = key_s[s2];
+          at += (o > mine) ? (int)(o & 0xff) : 0;  // (length, -slot) differs between slots, so the low bits never decide
+        }
+        for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(tid, ch);
+      }
+    }
+    return;
+  }
   // units of this thread's slots per class, then an inclusive scan over the threads for all classes at once
   int cls[PER], cnt[NC];
 #pragma unroll
