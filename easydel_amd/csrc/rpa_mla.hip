@@ -303,17 +303,32 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
         p.n_units[2] = L;
       }
     }
-    if (tid < n_slots) {
-      const uint32_t mine = key_s[tid];
-      const int v = (int)(mine & 0xff);
-      if (v > 0) {
-        int at = 0;
-        for (int s2 = 0; s2 < n_slots; ++s2) {
+    // The count is shared by as many threads per slot as the block has to spare (2 at 512 slots, 16 at 64 and fewer):
+    // thread t serves slot t % s_pad and the (t / s_pad)-th share of the keys; a wave's lanes walk the same keys.
+    __shared__ int part_s[1024];
+    int s_pad = 64;
+    while (s_pad < n_slots) s_pad <<= 1;
+    const int ways = 1024 / s_pad, share = (n_slots + ways - 1) / ways;
+    const int my_slot = tid & (s_pad - 1), my_part = tid / s_pad;
+    const uint32_t mine = my_slot < n_slots ? key_s[my_slot] : 0u;
+    {
+      int at = 0;
+      const int hi = min(n_slots, (my_part + 1) * share);
+      if (mine & 0xff) {
+#pragma unroll 4
+        for (int s2 = my_part * share; s2 < hi; ++s2) {
           const uint32_t o = key_s[s2];
           at += (o > mine) ? (int)(o & 0xff) : 0;  // (length, -slot) differs between slots, so the low bits never decide
         }
-        for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(tid, ch);
       }
+      part_s[tid] = at;
+    }
+    __syncthreads();
+    if (my_part == 0 && (mine & 0xff)) {
+      int at = 0;
+      for (int w = 0; w < ways; ++w) at += part_s[w * s_pad + my_slot];
+      const int v = (int)(mine & 0xff);
+      for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(my_slot, ch);
     }
     return;
   }
