@@ -79,6 +79,19 @@ def test_more_row_tile_slots_than_the_sorted_unit_list_holds():
     check(b, "3900 sequences", softmax_scale=SCALE)
 
 
+def test_unit_list_in_length_classes():
+    # 700 sequences at 16 heads: 797 row-tile slots -- more than the exact sort of the unit list takes (512), fewer than
+    # the one-block plan holds (4 096): the list is built longest first in eight length classes.  Contexts of 1 ... 2 500
+    # keys, so that the long ones are cut into chunks and the classes are all in use.
+    rng = np.random.default_rng(21)
+    ctx = rng.integers(1, 400, size=700)
+    ctx[::37] = rng.integers(1200, 2500, size=len(ctx[::37]))
+    b = make_mla_batch(22, ctx.tolist(), [1] * len(ctx), Hq=16, page_size=64, pad_rows=5, pad_tokens=3, distinct_pages=211)
+    slots = b.T * b.Hq // 128 + b.S
+    assert 512 < slots <= 4096
+    check(b, "700 sequences", softmax_scale=SCALE)
+
+
 def test_chunked_prefill_and_mixed_rows():
     b = make_mla_batch(4, [200, 97, 400, 31, 1000], [1, 97, 150, 31, 3], Hq=16)
     check(b, "mixed", softmax_scale=SCALE)
