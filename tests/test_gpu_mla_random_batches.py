@@ -21,7 +21,10 @@ GEOMETRIES = [(16, 64, BF16), (128, 64, BF16), (20, 32, BF16), (8, 128, BF16), (
 
 
 # 18 seeds by default; RPA_RANDOM_SEEDS in the environment widens the sweep
-@pytest.mark.parametrize("seed", range(int(os.environ.get("RPA_RANDOM_SEEDS", "18"))))
+_FIRST_SEED = int(os.environ.get("RPA_RANDOM_FIRST_SEED", "0"))  # a sweep over seeds no earlier sweep has seen starts here
+
+
+@pytest.mark.parametrize("seed", range(_FIRST_SEED, _FIRST_SEED + int(os.environ.get("RPA_RANDOM_SEEDS", "18"))))
 def test_random_mla_batch(gpu, seed):
     rng = np.random.default_rng(5000 + seed)
     Hq, page_size, dtype = GEOMETRIES[seed % len(GEOMETRIES)]

@@ -17,7 +17,10 @@ GEOMETRIES = [(128, 64, 32, 8), (128, 16, 8, 8), (64, 32, 64, 8), (64, 16, 8, 2)
 
 
 # 24 seeds by default; RPA_RANDOM_SEEDS=400 in the environment widens the sweep
-@pytest.mark.parametrize("seed", range(int(os.environ.get("RPA_RANDOM_SEEDS", "24"))))
+_FIRST_SEED = int(os.environ.get("RPA_RANDOM_FIRST_SEED", "0"))  # a sweep over seeds no earlier sweep has seen starts here
+
+
+@pytest.mark.parametrize("seed", range(_FIRST_SEED, _FIRST_SEED + int(os.environ.get("RPA_RANDOM_SEEDS", "24"))))
 def test_random_batch(gpu, seed):
     rng = np.random.default_rng(1000 + seed)
     D, page_size, Hq, Hkv = GEOMETRIES[seed % len(GEOMETRIES)]
