@@ -30,7 +30,7 @@ struct MlaParams {
                      // [1] 1 if the list is sorted longest first, 0 if it is in slot order;
                      // [2] chunk length the plan kernel chose for this batch (keys, a multiple of 64), 0: the cut
                      //     follows rule_chunks / min_chunk
-  int2* units;     // [n_units[0]] (slot, chunk)
+  int2* units;     // [n_units[0]] (slot, chunk | sequence << 5): what a workgroup needs to start, in one load
   int T, S, M, P, page_size, Hq, lkv, rope, rope_off, row_elems;
   int64_t token_stride, page_stride;  // bytes
   int q_dtype, kv_dtype;

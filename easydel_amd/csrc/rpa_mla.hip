@@ -284,12 +284,15 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
   // chunks, or as long and a lower slot -- and writes slot t's units there.
   if (n_slots <= kMlaRankSlots) {
     __shared__ uint32_t key_s[kMlaRankSlots];
+    __shared__ int seq_s[kMlaRankSlots];
     const unsigned len_div = max_len < 32768 ? 1u : (unsigned)(max_len / 32767 + 1);  // chunk lengths / 64 into 15 bits
 #pragma unroll
     for (int k = 0; k < PER; ++k) {
       const int slot = tid * PER + k;
-      if (slot < n_slots)
+      if (slot < n_slots) {
         key_s[slot] = (y[k] & 0xff) ? ((((unsigned)(y[k] >> 8) / len_div) << 17) | ((unsigned)(kMlaRankSlots - 1 - slot) << 8) | (unsigned)(y[k] & 0xff)) : 0u;
+        seq_s[slot] = seq_k[k];
+      }
     }
     __syncthreads();
     if (tid < 64) {  // the first wave adds up the units while the others place them
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
       int at = 0;
       for (int w = 0; w < ways; ++w) at += part_s[w * s_pad + my_slot];
       const int v = (int)(mine & 0xff);
-      for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(my_slot, ch);
+      for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(my_slot, ch | (seq_s[my_slot] << 5));
     }
     return;
   }
@@ -382,7 +385,7 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
         at = first[c];
         first[c] += v;
       }
-    for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(tid * PER + k, ch);
+    for (int ch = 0; ch < v; ++ch) p.units[at + ch] = make_int2(tid * PER + k, ch | (seq_k[k] << 5));
   }
   if (tid == 0) {
     p.n_units[0] = total;
@@ -409,7 +412,8 @@ __global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_sl
   __syncthreads();
   for (int base = 0; base < n_slots; base += 1024) {
     const int slot = base + tid;
-    const int v = slot < n_slots ? (p.plan[slot].y & 0xff) : 0;
+    const int2 entry = slot < n_slots ? p.plan[slot] : make_int2(0, 0);
+    const int v = entry.y & 0xff;
     int incl = v;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -421,7 +425,7 @@ __global__ __launch_bounds__(1024) void mla_compact_kernel(MlaParams p, int n_sl
     int before = running_s;
     for (int w = 0; w < wv; ++w) before += wave_tot[w];
     const int first = before + incl - v;
-    for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c);
+    for (int c = 0; c < v; ++c) p.units[first + c] = make_int2(slot, c | (entry.x << 5));
     __syncthreads();
     if (tid == 1023) running_s = before + incl;
     __syncthreads();
@@ -495,15 +499,17 @@ __global__ __launch_bounds__(64 * kMlaWaves, 2) void mla_attn_kernel(MlaParams p
   // Block -> unit of the dense list.  Consecutive blocks go to the eight XCDs in turn.  A list in slot order (large
   // batches) is dealt in contiguous eighths, unit = (block % 8) * n8 + block / 8, so that the row tiles of a long
   // prompt, which read the same keys, share one XCD's L2; a list sorted longest first is dealt block by block.
+  // The unit of a sorted list is asked for together with the list's length (the list has an entry for every block of
+  // the grid, so the load is in bounds whatever it returns), and it names its sequence: two dependent loads fewer
+  // before the first tile can be requested.
+  int2 sc = p.units[blockIdx.x];
   const int total = p.n_units[0];
   const int n8 = (total + kXcds - 1) / kXcds;
   const bool sorted = p.n_units[1] != 0;
   const int u = sorted ? (int)blockIdx.x : (int)((blockIdx.x % kXcds) * n8 + blockIdx.x / kXcds);
   if ((!sorted && (int)(blockIdx.x / kXcds) >= n8) || u >= total) return;
-  const int2 sc = p.units[u];
-  const int slot = sc.x, chunk = sc.y;
-  const int2 unit = p.plan[slot];
-  const int i = unit.x;
+  if (!sorted) sc = p.units[u];
+  const int slot = sc.x, chunk = sc.y & 31, i = sc.y >> 5;
   const MlaSeq sp = mla_seq(p, i);
   const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * Hq) / kMlaRows) + i);
   const int rows_total = sp.q_len * Hq;
@@ -1043,7 +1049,8 @@ int64_t mla_plan_slots(int T, int S, int Hq) { return ((int64_t)T * Hq) / kMlaRo
 static size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
 size_t mla_plan_bytes(int T, int S, int Hq, int max_chunks) {
   const size_t slots = (size_t)mla_plan_slots(T, S, Hq);
-  return up256(slots * 8) + 256 + up256(slots * (size_t)max_chunks * 8);
+  // the unit list has an entry for every block of the attention kernel's grid, which is rounded up to a multiple of 8
+  return up256(slots * 8) + 256 + up256((slots * (size_t)max_chunks + kXcds) * 8);
 }
 
 int launch_mla_mfma(hipStream_t stream, const MlaParams& p) {
