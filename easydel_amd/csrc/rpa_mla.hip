@@ -225,7 +225,7 @@ __global__ __launch_bounds__(1024) void mla_plan_sorted_kernel(MlaParams p, int 
   __syncthreads();
   // A batch of few row tiles (a quarter of the CUs or fewer: a small decode batch) is cut by length, not by count: every
   // tile into chunks of about L keys, L such that the whole batch makes at most one unit per CU -- sum(ceil(span / L))
-  // <= W / L + R <= CUs for L = W / (CUs - R), W the keys of all R tiles.  One round of near-equal units then takes
+  // <= W / L + R <= CUs for L = W / (CUs - R), W the keys of all R tiles.  A single wave of near-equal units over the chip then takes
   // what one chunk takes, where even cuts of every tile leave units as different as the sequences are long.
   __shared__ long long wave_w[16];
   __shared__ int wave_r[16];
