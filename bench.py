@@ -48,6 +48,7 @@ def parse_args():
     ap.add_argument("--decode-sync", type=int, default=-1)
     ap.add_argument("--decode-dma", type=int, default=-1, help="LDS-direct decode kernel: -1 the library's choice, 0 never, 1 wherever built")
     ap.add_argument("--max-splits", type=int, default=0)
+    ap.add_argument("--prefill-x32", type=int, default=-1, help="32x32-tile prefill kernel: -1 the library's choice, 0 never")
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
     ap.add_argument("--mla-uniform-context", type=int, default=0,
@@ -69,7 +70,7 @@ def parse_args():
 
 
 def build_workload(name, seed, sequential=False):
-    from easydel_amd import workloads
+    import bench_workloads as workloads
 
     if name == "c2":
         return workloads.config2_llama_decode(seed, shuffle_pages=not sequential)
@@ -349,7 +350,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
-    from easydel_amd import _lib, kernels, workloads
+    import bench_workloads as workloads
+    from easydel_amd import _lib, kernels
 
     _lib.load()
     if args.read_probe:
@@ -372,6 +374,8 @@ def main():
         _lib.set_tunable("prefill_chunks", args.prefill_chunks)
     if args.max_splits:
         _lib.set_tunable("max_splits", args.max_splits)
+    if args.prefill_x32 >= 0:
+        _lib.set_tunable("prefill_x32", args.prefill_x32)
 
     dev = torch.device("cuda:0")
     w = build_workload(args.workload, args.seed, args.sequential_pages)

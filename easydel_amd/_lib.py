@@ -22,9 +22,6 @@ SIGNATURES = {
     "rpa_version": (ctypes.c_char_p, []),
     "rpa_last_error": (ctypes.c_char_p, []),
     "rpa_set_tunable": (_c_int, [ctypes.c_char_p, _c_int]),
-    "rpa_calibration_copy": (_c_int, [_c_vp, _c_vp, _c_vp, _c_sz]),
-    "rpa_read_probe": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_vp]),
-    "rpa_read_probe_paged": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_int, _c_int, _c_vp]),
     "rpa_page_scatter_slices": (_c_int, [_c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_int, _c_int, _c_i64, _c_int, _c_i64, _c_int]),
     "rpa_page_scatter_ragged": (_c_int, [_c_vp] * 8 + [_c_int] * 10),
     "rpa_attention_workspace_bytes": (_c_sz, [_c_int] * 9),
@@ -55,6 +52,15 @@ SIGNATURES = {
     ),
     "rpa_mla_workspace_bytes": (_c_sz, [_c_int] * 8),
     "rpa_mla_page_scatter": (_c_int, [_c_vp] * 8 + [_c_int] * 9),
+}
+
+
+# the measurement kernels of rpa_hip_probe.h: exported by the test / benchmark build of the library only
+PROBE_SIGNATURES = {
+    "rpa_calibration_copy": (_c_int, [_c_vp, _c_vp, _c_vp, _c_sz]),
+    "rpa_read_probe": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_vp]),
+    "rpa_read_probe_paged": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_int, _c_int, _c_vp]),
+    "rpa_mfma_probe": (ctypes.c_double, [_c_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_vp, _c_vp]),
 }
 
 
@@ -90,6 +96,11 @@ def load() -> ctypes.CDLL:
                 fn = getattr(lib, name)
                 fn.restype = restype
                 fn.argtypes = argtypes
+            for name, (restype, argtypes) in PROBE_SIGNATURES.items():
+                fn = getattr(lib, name, None)  # absent from a product build
+                if fn is not None:
+                    fn.restype = restype
+                    fn.argtypes = argtypes
             _lib = lib
     return _lib
 

@@ -26,9 +26,12 @@ SOURCES = [
     "rpa_attn_prefill.hip",
     "rpa_attn_prefill_dma.hip",
     "rpa_attn_prefill_dma8.hip",
+    "rpa_attn_prefill_x32.hip",
     "rpa_attn_merge.hip",
     "rpa_mla.hip",
 ]
+# measurement kernels and result-changing test knobs: compiled into the test / benchmark build only (-DRPA_PROBES)
+PROBE_SOURCES = ["rpa_probe.hip"]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from scalar float code on this target.
 HIPCC_FLAGS = [
@@ -57,13 +60,15 @@ def _compile(src: str, obj_dir: Path, extra: list[str]) -> Path:
     return obj
 
 
-def build_library(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int = 6) -> Path:
-    """Compile every kernel source and link the shared library.  Always rebuilds."""
-    extra = list(extra_flags or [])
+def build_library(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int = 6, probes: bool = True) -> Path:
+    """Compile every kernel source and link the shared library.  Always rebuilds.  ``probes=False`` is the product
+    build: no measurement kernels, and ``rpa_set_tunable`` does not know the knobs that can make a call skip a stage."""
+    extra = list(extra_flags or []) + (["-DRPA_PROBES"] if probes else [])
+    sources = SOURCES + (PROBE_SOURCES if probes else [])
     obj_dir = OUT_DIR / "obj"
     obj_dir.mkdir(parents=True, exist_ok=True)
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(lambda s: _compile(s, obj_dir, extra), SOURCES))
+        objs = list(pool.map(lambda s: _compile(s, obj_dir, extra), sources))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -96,5 +101,7 @@ def build_ffi(verbose: bool = True) -> Path | None:
 
 
 if __name__ == "__main__":
-    build_library(extra_flags=sys.argv[1:])
+    args = sys.argv[1:]
+    product = "--product" in args
+    build_library(extra_flags=[a for a in args if a != "--product"], probes=not product)
     build_ffi()

@@ -16,9 +16,12 @@ int launch_scatter_slices(hipStream_t, const void*, const int32_t*, const int32_
                           int64_t, int);
 int launch_scatter_ragged(hipStream_t, const void*, const void*, void*, const int32_t*, const int32_t*,
                           const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int);
+#ifdef RPA_PROBES
 int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
 size_t launch_read_probe(hipStream_t, const void*, size_t, int, int, uint32_t*);
 size_t launch_read_probe_paged(hipStream_t, const void*, size_t, int, int, int, int, uint32_t*);
+double launch_mfma_probe(hipStream_t, int, int, int, int, int, unsigned long long*, float*);
+#endif
 int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
                                 const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int, int);
 }  // namespace rpa
@@ -27,7 +30,9 @@ namespace {
 
 thread_local char g_err[512] = "";
 
-// Test and measurement knobs (rpa_set_tunable, declared in rpa_hip_probe.h).  They belong to the thread that sets
+// Test and measurement knobs (rpa_set_tunable, declared in rpa_hip_probe.h).  A build without -DRPA_PROBES knows the
+// tuning knobs only: the two that change what a call computes with ("stages", which can make it skip a launch, and
+// "force_generic") and the measurement kernels exist in the test / benchmark build alone.  They belong to the thread that sets
 // them: a call sees the values of its own thread only, read once when it starts, so a thread that never calls
 // rpa_set_tunable always runs with the defaults below, whatever a profiling or test thread of the same process does.
 struct Tunables {
@@ -37,6 +42,7 @@ struct Tunables {
   int decode_wgs = 0;      // 0 = as many persistent workgroups as are resident at once
   int force_generic = 0;
   int prefill_dma = 1;
+  int prefill_x32 = 1;     // 1: the 32x32-tile prefill kernel serves the shapes it is built for
   int decode_pace = 1;
   int decode_dma = -1;     // -1: where it measured faster (head size 256; int8 pages); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
   int mla_chunks = 0;      // 0 = sized from the shapes
@@ -102,6 +108,7 @@ int device_cus() {
 // than workgroups fit on the chip is not cut at all.  Otherwise this only sizes the partial buffers: the plan kernel
 // picks the chunk length from the lengths of the batch it finds on the device.
 void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int* chunk_keys, int* max_chunks) {
+  // (the row-tile bound below is taken with the smaller of the two row-tile heights: it only sizes buffers)
   const long span = (long)M * page_size;
   int chunks = g_tun.prefill_chunks > 0 ? g_tun.prefill_chunks : rpa::kMaxPrefillChunks;
   if (chunks > rpa::kMaxPrefillChunks) chunks = rpa::kMaxPrefillChunks;
@@ -180,16 +187,20 @@ int rpa_set_tunable(const char* name, int value) {
     return swap(g_tun.decode_sync, pow2);
   }
   if (!strcmp(name, "decode_wgs")) return swap(g_tun.decode_wgs, value < 0 ? 0 : value);
+#ifdef RPA_PROBES
   if (!strcmp(name, "force_generic")) return swap(g_tun.force_generic, value != 0);
+  if (!strcmp(name, "stages")) return swap(g_tun.stages, value & 15);
+#endif
   if (!strcmp(name, "prefill_dma")) return swap(g_tun.prefill_dma, value != 0);
+  if (!strcmp(name, "prefill_x32")) return swap(g_tun.prefill_x32, value != 0);
   if (!strcmp(name, "decode_pace")) return swap(g_tun.decode_pace, value != 0);
   if (!strcmp(name, "decode_dma")) return swap(g_tun.decode_dma, value < 0 ? -1 : value > 3 ? 3 : value);
   if (!strcmp(name, "mla_min_chunk")) return swap(g_tun.mla_min_chunk, value <= 0 ? 0 : ((value + 63) & ~63));
   if (!strcmp(name, "mla_chunks")) return swap(g_tun.mla_chunks, value < 0 ? 0 : (value > rpa::kMlaMaxChunks ? rpa::kMlaMaxChunks : value));
-  if (!strcmp(name, "stages")) return swap(g_tun.stages, value & 15);
   return -1;
 }
 
+#ifdef RPA_PROBES
 int rpa_calibration_copy(rpa_stream_t stream, void* dst, const void* src, size_t bytes) {
   if (!dst || !src || (bytes & 15) || ((uintptr_t)dst & 15) || ((uintptr_t)src & 15))
     return fail(RPA_ERR_INVALID_ARGUMENT, "rpa_calibration_copy: pointers and size must be 16-byte aligned");
@@ -222,6 +233,20 @@ size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, 
                                    "and a multiple of chunk_kib / 8, split 0..2, and at least one group of chunks per workgroup");
   return read;
 }
+
+double rpa_mfma_probe(rpa_stream_t stream, int shape, int source, int mfmas_per_operand, int waves_per_simd, int iters,
+                      void* clocks, void* sink) {
+  if (!clocks || !sink || ((uintptr_t)clocks & 7) || ((uintptr_t)sink & 3)) {
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_mfma_probe: clocks must be two 8-byte device words, sink a 4-byte device word");
+    return 0.0;
+  }
+  const double flops = rpa::launch_mfma_probe((hipStream_t)stream, shape, source, mfmas_per_operand, waves_per_simd, iters,
+                                              (unsigned long long*)clocks, (float*)sink);
+  if (flops == 0.0)
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_mfma_probe: shape 0 / 1, source 0..2, 1 / 2 / 4 MFMAs per operand, 1 or 2 waves per SIMD, iters > 0");
+  return flops;
+}
+#endif  // RPA_PROBES
 
 int rpa_page_scatter_slices(rpa_stream_t stream, const void* new_kv, const int32_t* slice_indices,
                             const int32_t* num_slices, void* kv_pages, int T, int N, int64_t num_positions,
@@ -326,6 +351,15 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: kv_scales with pages that are not 8-bit (kv_dtype %d)", who, kv_dtype);
   if (kv_scales && ((uintptr_t)kv_scales & 7))
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: kv_scales must be 8-byte aligned", who);
+  // Pages of bare codes exist for fp8 only (the reference's cast-only cache, ragged_page_attention.py:570-580); int8
+  // codes mean nothing without their scales.
+  if (!kv_scales && kv_dtype == RPA_INT8)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "%s: int8 KV pages need kv_scales (only fp8 pages may be unscaled)", who);
+  // The decode plan counts the keys of a batch in 32-bit integers (spans of the flattened key stream); pages shared
+  // between sequences let that sum exceed the pool, so the bound is on what the block tables can address.
+  if ((int64_t)S * M * page_size >= ((int64_t)1 << 31))
+    return fail(RPA_ERR_UNSUPPORTED, "%s: S * M * page_size = %lld tokens addressable by the block tables, the limit is 2^31 - 1 per call",
+                who, (long long)((int64_t)S * M * page_size));
   if (!std::isfinite(softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_scale is not finite", who);
   if (softmax_aux && ((uintptr_t)softmax_aux & 3))
     return fail(RPA_ERR_INVALID_ARGUMENT, "%s: softmax_aux must be 4-byte aligned", who);
@@ -355,6 +389,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.decode_wgs = tun.decode_wgs;
   p.decode_sync = tun.decode_sync;
   p.prefill_dma = tun.prefill_dma;
+  p.pre_rows = rpa::kPrefillRows;
   p.decode_pace = tun.decode_pace;
   p.decode_dma = tun.decode_dma < 0 ? ((p.D == 256 || p.kv_dtype == RPA_INT8) ? 1 : 0) : tun.decode_dma;
   p.max_splits = 2;
@@ -405,6 +440,10 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     p.pre_max_chunks = pre_chunks;
     p.pre_auto = tun.prefill_chunks <= 0 ? 1 : 0;
     p.pre_slots = device_cus() * (Dc <= 128 ? 2 : 1);  // resident workgroups of the large-row kernels
+    if (tun.prefill_dma && tun.prefill_x32 && rpa::prefill_x32_supported(p)) {  // 256-row workgroups, one per CU
+      p.pre_rows = 256;
+      p.pre_slots = device_cus();
+    }
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
     p.plan = (int32_t*)base;
     p.part_o = (float*)(base + pb);

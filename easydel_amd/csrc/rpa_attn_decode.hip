@@ -533,8 +533,8 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     sum += span_of(i, sp, toks);
     tsum += toks;
     if (sp.live && !sp.small_rows && sp.q_len > 0) {
-      const int tile_reach = p.window > 0 ? min(sp.ctx, p.window + kPrefillRows / p.group + 64) : sp.ctx;
-      const int tiles = (sp.q_len * p.group + kPrefillRows - 1) / kPrefillRows;
+      const int tile_reach = p.window > 0 ? min(sp.ctx, p.window + p.pre_rows / p.group + 64) : sp.ctx;
+      const int tiles = (sp.q_len * p.group + p.pre_rows - 1) / p.pre_rows;
       const int span = max(min(tile_reach, sp.ctx - sp.q_len / 2), 1);  // causal: half the new keys on average
       work += (unsigned long long)tiles * (unsigned)span;
       reach = max(reach, tile_reach);
@@ -730,10 +730,10 @@ int decode_row_limit(int T, int S, int D, int kv_dtype) {
 
 bool decode_supported(const AttnParams& p) {
   // bf16 queries over bf16 / fp8 / int8 pages, or float16 queries over float16 pages (the MFMA operands of a kernel
-  // are of one 16-bit type); float16 pages also need the LDS-direct prefill kernel's page sizes, the only large-row
-  // kernel built for them
+  // are of one 16-bit type); float16 pages also need the LDS-direct prefill kernel (its page sizes and offset range,
+  // and a call that has not switched it off): it is the only large-row kernel built for them
   if (p.kv_dtype == RPA_F32) return false;
-  if (p.kv_dtype == RPA_F16 ? (p.q_dtype != RPA_F16 || p.page_size % 32 != 0) : p.q_dtype != RPA_BF16) return false;
+  if (p.kv_dtype == RPA_F16 ? (p.q_dtype != RPA_F16 || !p.prefill_dma || !prefill_dma_supported(p)) : p.q_dtype != RPA_BF16) return false;
   if (p.D != 64 && p.D != 128 && p.D != 256) return false;
   if (p.Dq > p.D || p.Dq % 8 != 0) return false;  // a q row is read in 16-byte chunks, whole chunks inside or outside Dq
   if (p.page_size % 16 != 0) return false;

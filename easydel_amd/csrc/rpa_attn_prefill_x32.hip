@@ -1,0 +1,673 @@
+// MFMA prefill / chunked-prefill attention for bf16 (or float16) pages on 32x32x16 tiles: one wave per SIMD, 64 query
+// rows per wave, and a steady-state step whose instruction order and register files are written down, not left to the
+// scheduler and the allocator.
+//
+// Why this shape.  A bf16 MFMA stream whose A operands come out of LDS sustains, on this chip, 65-78 % of the matrix
+// peak with 16x16x32 tiles and two row blocks per operand (what attn_prefill_dma_kernel does), but 86 % with 32x32x16
+// tiles and two 32-row blocks per operand, already with one wave per SIMD: a 32x32x16 MFMA occupies the pipe for 32
+// cycles, takes the same 1 KiB operand, and leaves the issue port free for six vector instructions.  So a wave here
+// owns 64 rows (row = (token, GQA head)) of one (sequence, KV head): Q as B operands (S^T = K Q^T) and the O^T
+// accumulators stay in registers for the whole key range, every K and V operand read from LDS feeds two MFMAs, and a
+// workgroup of four waves (256 rows) has a CU to itself.  With a single wave per SIMD nothing but the wave's own
+// instruction order overlaps the matrix pipe with the softmax, so the step -- one block of 32 keys -- is
+// software-pipelined over three blocks and its order is pinned (a sched_barrier after every MFMA slot):
+//
+//   step b :  MFMA slots 0..15   S(b+2) = K(b+2) Q^T       | vector: softmax of block b+1, half a pair of probabilities per slot
+//             MFMA slots 16..31  O     += V(b)^T P(b)^T     | vector: the softmax goes on; row maxima of S(b+2)
+//
+// Operands are read four ahead of their MFMAs, across the phase and step boundaries.  The wave has 512 registers; which
+// of them sit in the accumulation file is stated through the operand constraints of the MFMAs (issued as single
+// assembly statements): O^T and Q live there (192 registers the vector ALU never touches), the scores are produced in
+// ordinary registers because the vector ALU reads them next.  The compiler does not see into those statements, so the
+// waits this chip wants between an MFMA and a vector instruction that reads its result are stated here as well: in the
+// pinned step the first reader of a result comes at least sixteen MFMA slots behind its writer, everywhere else an
+// explicit pause (mfma_settle) precedes the reader.
+//
+// Tiles of 64 keys travel global -> LDS through the load unit (global_load_lds_dwordx4), K four tiles and V three
+// tiles ahead, in rings of four slots each (128 KiB at head size 128); one barrier per tile, i.e. per two steps.
+//
+// Softmax as in attn_prefill_dma_kernel: probabilities are taken against a per-row reference that is only raised when a
+// score exceeds it by more than kMaxSlack (log2 units); here the reference is kept at whole numbers, so that raising it
+// scales what has been accumulated -- and the probabilities of the block still waiting for its PV product -- by a power
+// of two, exactly.  Row sums are taken from the packed 16-bit probabilities (v_dot2), i.e. of exactly the weights the
+// PV product uses.
+//
+// Tiles that need masking (the window's lower edge, the causal diagonal) and the first and the last two tiles of a key
+// range run through the same two steps written plainly (phases one after the other, flags at run time); the pinned
+// steps serve the unmasked middle.
+#include <type_traits>
+
+#include "rpa_mfma.h"
+
+namespace rpa {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+
+// The pause between an MFMA issued through an assembly statement and an instruction that reads its result (the
+// compiler cannot place it): 32 wait states, more than the eight passes of a 32x32x16 MFMA plus the margin this chip asks for.
+// The registers whose readers it protects are operands of the statement: that is what orders it behind the MFMAs that
+// write them and ahead of the instructions that read them.
+__device__ __forceinline__ void mfma_settle(f32x16& a, f32x16& b) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a), "+v"(b)); }
+template <int N>
+__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[N]) {
+  static_assert(N == 8, "written out for eight accumulator tiles");
+  asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]));
+}
+
+template <int HT>
+struct Wide16;
+template <>
+struct Wide16<RPA_BF16> {
+  // S^T accumulation: result in ordinary registers, K operand in ordinary registers, Q operand in the accumulation file
+  static __device__ __forceinline__ void mfma_s0(f32x16& acc, const u32x4& a, const u32x4& q) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(q));
+  }
+  static __device__ __forceinline__ void mfma_s(f32x16& acc, const u32x4& a, const u32x4& q) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(q));
+  }
+  // O^T accumulation: accumulator in the accumulation file, V and P operands in ordinary registers
+  static __device__ __forceinline__ void mfma_o(f32x16& acc, const u32x4& a, const u32x4& b) {
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  // sum += lo(w) + hi(w), the two bf16 halves of w
+  static __device__ __forceinline__ float add_pair(uint32_t w, float sum) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3F803F80u), sum, false);
+  }
+  static __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float a) {  // both halves times a
+    return pack_bf16(__uint_as_float(w << 16) * a, __uint_as_float(w & 0xffff0000u) * a);
+  }
+};
+template <>
+struct Wide16<RPA_F16> {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ void mfma_s0(f32x16& acc, const u32x4& a, const u32x4& q) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(acc) : "v"(a), "a"(q));
+  }
+  static __device__ __forceinline__ void mfma_s(f32x16& acc, const u32x4& a, const u32x4& q) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(q));
+  }
+  static __device__ __forceinline__ void mfma_o(f32x16& acc, const u32x4& a, const u32x4& b) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ float add_pair(uint32_t w, float sum) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), __builtin_bit_cast(f16x2, 0x3C003C00u), sum, false);
+  }
+  static __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float a) {
+    const f16x2 v = __builtin_bit_cast(f16x2, w);
+    return Half16<RPA_F16>::pack((float)v[0] * a, (float)v[1] * a);
+  }
+};
+
+// Swizzle of the V half of a tile for the transposing reads of 32x32x16 operands: one ds_read_b64_tr_b16 fetches, for
+// each half of the wave, 64 contiguous bytes of four consecutive key rows; XOR-ing the 16-byte chunk index with four
+// times the row number (mod 4) puts those four rows on distinct quarters of the banks.
+template <int ROW_BYTES>
+__device__ __forceinline__ int swz_key_v32(int tok) {
+  constexpr int NCH = ROW_BYTES / 16;
+  if constexpr (NCH >= 16) return (tok & 3) << 2;
+  else if constexpr (NCH == 8) return (tok & 1) << 2;
+  else return 0;
+}
+
+constexpr int kWideRows = 256;  // query rows one workgroup of this kernel owns
+
+template <int D, int NW, int RB, int HT>
+__global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p) {
+  using H = Half16<HT>;
+  using W = Wide16<HT>;
+  constexpr int TT = 64;                 // keys per tile (what a barrier and a set of loads cover)
+  constexpr int BK = 32;                 // keys per block (what a step computes)
+  constexpr int RKL = D * 2;             // bytes of one K (or V) row
+  constexpr int CPR = RKL / 16;          // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;          // rows one DMA instruction covers
+  constexpr int NLH = TT / (RPI * NW);   // DMA instructions per wave per tile, for K and again for V
+  static_assert(TT % (RPI * NW) == 0 && NLH >= 1, "the waves' DMA instructions tile the rows exactly");
+  static_assert(NLH == 1 || (RPI * NW) % 16 == 0, "a lane's swizzle key must not depend on the instruction");
+  constexpr int NKK = D / 16;            // k-steps of the score MFMA = K operands per block
+  constexpr int DB = D / 32;             // 32-dim blocks of O^T
+  constexpr int NVO = DB * 2;            // V operands per block: (dim block, 16-key half)
+  constexpr int ROWS = NW * RB * 32;
+  static_assert(ROWS == kWideRows, "the plan and merge kernels are told this row-tile height");
+  constexpr float kMaxSlack = 8.f;
+  constexpr int HALF = TT * RKL;         // bytes of the K (or V) rows of one tile
+  constexpr int KN = 4, VN = 4;          // ring slots
+  static_assert(KN * HALF <= 65536, "K operand reads address their ring slot through the instruction's 16-bit offset");
+  constexpr int NQ = NKK * RB;           // MFMA slots of the score phase
+  constexpr int NP = NVO * RB;           // MFMA slots of the PV phase
+  constexpr int PD = 4;                  // operands read ahead
+  constexpr int NPAIR = RB * 8;          // pairs of probabilities per lane and block
+  static_assert(NQ + NP == 2 * NPAIR && NP == NPAIR, "half a pair of the softmax per MFMA slot, one three-way maximum per PV slot");
+  static_assert(NKK >= PD && NVO >= PD, "the operand ring is shorter than either phase");
+  static_assert(RB == 2, "mfma_settle names the score tiles of two row blocks");
+
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[(KN + VN) * HALF];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int j32 = lane & 31, hh = lane >> 5;  // row inside a 32-row block, half of the wave
+  const int n = lane & 15;
+  const int G = p.group;
+
+  // ---- block -> (sequence, row tile, KV head, key chunk) ---------------------------------------------
+  const int h = blockIdx.x % p.Hkv;
+  const int n_slots = gridDim.x / (p.Hkv * p.pre_max_chunks);
+  const int slot = (blockIdx.x / p.Hkv) % n_slots;
+  const int chunk = blockIdx.x / (p.Hkv * n_slots);
+  if (p.plan[2] == 0) return;
+  const int n_live = live_rows(p);
+  if (n_live <= 0) return;
+  int lo_i = 0, hi_i = n_live;
+  while (hi_i - lo_i > 1) {
+    const int mid = (lo_i + hi_i) >> 1;
+    if ((int)(((int64_t)p.qsl[mid] * G) / ROWS) + mid <= slot) lo_i = mid; else hi_i = mid;
+  }
+  const int i = lo_i;
+  const SeqPlan sp = seq_plan(p, i);
+  if (!sp.live || sp.small_rows) return;
+  const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * G) / ROWS) + i);
+  const int rows_total = sp.q_len * G;
+  const int R0 = tile_in_seq * ROWS;
+  if (tile_in_seq < 0 || R0 >= rows_total) return;
+
+  const PrefillTile pt = prefill_tile(p, sp, R0);
+  if (pt.n_chunks == 0 && chunk == 0) {  // every row of the tile lies before position 0 and sees no key: zeros
+    for (int e = tid; e < ROWS * (p.Dq / 4); e += 64 * NW) {
+      const int row = R0 + e / (p.Dq / 4), d4 = e % (p.Dq / 4);
+      if (row < rows_total)
+        *(u32x2*)((uint16_t*)p.out + ((int64_t)(sp.q0 + row / G) * p.Hq + h * G + row % G) * p.Dq + 4 * d4) = (u32x2){0u, 0u};
+    }
+    return;
+  }
+  if (chunk >= pt.n_chunks) return;
+  const int base_pos = sp.ctx - sp.q_len;
+  const int vis_lo = pt.vis_lo;
+  const int kv_lo = max(pt.kv_lo + chunk * pt.chunk_len, vis_lo & ~(TT - 1));
+  const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : pt.kv_lo + (chunk + 1) * pt.chunk_len;
+  const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
+  const bool single = pt.n_chunks == 1;
+
+  // ---- per row-block lane state --------------------------------------------------------------------
+  int row_lo[RB], row_hi[RB];
+  bool row_ok[RB];
+  int out_tok[RB], out_head[RB];
+  u32x4 qf[RB][NKK];
+  int wave_lo, wave_hi;          // keys every row of the wave sees: [max row_lo, min row_hi)
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int row = R0 + (wave * RB + rb) * 32 + j32;
+    row_ok[rb] = row < rows_total;
+    const int r_tok = row_ok[rb] ? row / G : (rows_total - 1) / G;  // padded rows shadow the last row
+    const int r_head = row_ok[rb] ? row - r_tok * G : 0;
+    const int pos = base_pos + r_tok;
+    row_hi[rb] = min(pos + 1, sp.ctx);
+    row_lo[rb] = (p.window > 0) ? max(pos - p.window + 1, 0) : 0;
+    out_tok[rb] = sp.q0 + r_tok;
+    out_head[rb] = h * G + r_head;
+    const char* qrow = (const char*)p.q + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * p.Dq * 2;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {  // B operand of k-step kk: dims 16 kk + 8 hh .. + 7 of the lane's row
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row_ok[rb] && kk * 16 + 8 * hh < p.Dq) v = *(const u32x4*)(qrow + (kk * 16 + 8 * hh) * 2);
+      qf[rb][kk] = v;
+    }
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {  // waited for here, not inside the loop; kept in the accumulation file from here on
+      u32x4 v = qf[rb][kk];
+      asm volatile("" : "+a"(v));
+      qf[rb][kk] = v;
+    }
+  {
+    int lo_max = 0, hi_min = 0x7fffffff;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      lo_max = max(lo_max, row_lo[rb]);
+      hi_min = min(hi_min, row_hi[rb]);
+    }
+#pragma unroll
+    for (int o = 1; o < 32; o <<= 1) {
+      lo_max = max(lo_max, __shfl_xor(lo_max, o));
+      hi_min = min(hi_min, __shfl_xor(hi_min, o));
+    }
+    wave_lo = __builtin_amdgcn_readfirstlane(lo_max);
+    wave_hi = __builtin_amdgcn_readfirstlane(hi_min);
+  }
+
+  // ---- tile loads ------------------------------------------------------------------------------------
+  typedef const __attribute__((address_space(4))) int32_t* ConstI32;
+  ConstI32 bt = (ConstI32)(uintptr_t)(p.block_tables + (int64_t)i * p.M);
+  const char* k_pages = (const char*)p.k_pages;
+  const char* v_pages = (const char*)p.v_pages;
+  const int pg = p.page_size;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
+  const int dma_row = wave * RPI + lane / CPR;
+  const int dma_chunk = (lane % CPR) ^ swz_key<RKL>(dma_row);
+  const int dma_chunk_v = (lane % CPR) ^ swz_key_v32<RKL>(dma_row);
+  const uint32_t dma_wave_lds = (uint32_t)wave * 1024u;
+  uint32_t voff_k[NLH], voff_v[NLH];
+#pragma unroll
+  for (int u = 0; u < NLH; ++u) {
+    const uint32_t roff = (uint32_t)(dma_row + u * NW * RPI) * (uint32_t)p.token_stride;
+    voff_k[u] = roff + (uint32_t)(dma_chunk << 4);
+    voff_v[u] = roff + (uint32_t)(dma_chunk_v << 4);
+  }
+  auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
+  // Two cursors walk the tiles of the key range, the K cursor ahead of the V cursor.
+  struct Cursor { int idx, off, tb, slot, page_raw; };
+  Cursor kc, vc;
+  kc.idx = kv_lo / pg; kc.off = kv_lo - kc.idx * pg; kc.tb = kv_lo; kc.slot = 0; kc.page_raw = load_page(kc.idx);
+  vc = kc;
+  auto issue = [&](Cursor& c, bool is_v) __attribute__((always_inline)) {
+    const int page = min(max(c.page_raw, 0), p.P - 1);
+    const int64_t tile_off = (int64_t)page * p.page_stride + (int64_t)c.off * p.token_stride + (int64_t)h * p.head_stride;
+    const char* base = (is_v ? v_pages : k_pages) + tile_off;
+    const bool edge = (c.tb + TT > sp.ctx) || (c.tb < vis_lo);
+    const uint32_t lds = lds_base + (uint32_t)((is_v ? KN : 0) + c.slot) * HALF + dma_wave_lds;
+    if (!edge) {
+#pragma unroll
+      for (int u = 0; u < NLH; ++u) dma16(lds + u * NW * 1024, is_v ? voff_v[u] : voff_k[u], base);
+    } else {
+#pragma unroll
+      for (int u = 0; u < NLH; ++u) {  // keys nobody may see: any visible row's bytes
+        const int r = min(max(c.tb + dma_row + u * NW * RPI, vis_lo), sp.ctx - 1) - c.tb;
+        const uint32_t roff = (uint32_t)r * (uint32_t)p.token_stride;
+        dma16(lds + u * NW * 1024, roff + (uint32_t)((is_v ? dma_chunk_v : dma_chunk) << 4), base);
+      }
+    }
+    c.tb += TT;
+    c.off += TT;
+    if (c.off >= pg) {
+      c.off -= pg;
+      ++c.idx;
+    }
+    c.slot = (c.slot + 1) & 3;
+    c.page_raw = load_page(c.idx);
+  };
+  int k_issued = 0, v_issued = 0;  // tiles whose K / V rows have been requested
+  auto issue_k = [&]() __attribute__((always_inline)) { if (k_issued < n_tiles) { issue(kc, false); ++k_issued; } };
+  auto issue_v = [&]() __attribute__((always_inline)) { if (v_issued < n_tiles) { issue(vc, true); ++v_issued; } };
+
+  // ---- registers of the pipeline -------------------------------------------------------------------------
+  // Block b of the key range = (tile b / 2, half b % 2).  Scores and probabilities of block b live in buffer b % 2.
+  f32x16 sa[2][RB];            // raw scores S^T: lane = row j32, register r = key 8 (r / 4) + 4 hh + r % 4 of the block
+  u32x4 pb[2][RB][2];          // packed probabilities, as the two B operands (16 keys each) of the PV product
+  f32x16 o_acc[RB][DB];        // O^T: lane = row j32, register r = dim 8 (r / 4) + 4 hh + r % 4 of the 32-dim block
+  float m_ref[RB], m_neg[RB], l_run[RB], lmx[RB];
+  u32x4 ops[PD];               // operands read ahead of their MFMAs
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    m_ref[rb] = -INFINITY;
+    m_neg[rb] = 0.f;
+    l_run[rb] = 0.f;
+    lmx[rb] = -INFINITY;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      asm volatile("" : "+a"(z));
+      o_acc[rb][db] = z;
+    }
+  }
+  const float sc_mul = p.scale_log2;
+
+  // Lane addresses of the operand reads, relative to a ring slot.  K operand kk of a block: key j32 of the block, chunk 2 kk + hh.
+  uint32_t kaddr[NKK];
+#pragma unroll
+  for (int kk = 0; kk < NKK; ++kk) kaddr[kk] = lds_base + (uint32_t)(j32 * RKL + (((2 * kk + hh) ^ swz_key<RKL>(j32)) << 4));
+  // V operand (db, s) of a block: two transposing reads; the lane addresses key 16 s + 4 hh (+ 8) + n / 4 of the block,
+  // dims 32 db + 16 (lane / 16 % 2) + 4 (n % 4).
+  uint32_t vaddr[DB];
+  {
+    const int key = 4 * hh + (n >> 2);
+    const int byte0 = 32 * ((lane >> 4) & 1) + 8 * (n & 3);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int off = 64 * db + byte0;
+      vaddr[db] = lds_base + (uint32_t)(KN * HALF + key * RKL + ((((off >> 4) ^ swz_key_v32<RKL>(key))) << 4) + (off & 15));
+    }
+  }
+  // operand kk of the block in half `half` of K slot `kslot` (offsets that are constants fold into the instruction)
+  auto read_k = [&](int kslot, int half, int kk) __attribute__((always_inline)) -> u32x4 {
+    return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)(kaddr[kk] + (uint32_t)(kslot * HALF + half * BK * RKL));
+  };
+  auto read_v = [&](int vslot, int half, int o) __attribute__((always_inline)) -> u32x4 {  // operand o = (db, s)
+    const int db = o / 2, s = o % 2;
+    const uint32_t a = vaddr[db] + (uint32_t)(vslot * HALF + (half * BK + 16 * s) * RKL);
+    const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)a));
+    const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)(a + 8 * RKL)));
+    return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+  };
+
+  // Raises the references of the rows whose new scores (maxima in lmx, raw) exceed them by more than the slack; what
+  // has been accumulated, and the pending probabilities pend (relative to the old reference), are scaled to match.
+  auto check = [&](u32x4 (&pend)[RB][2], bool has_pending) __attribute__((always_inline)) {
+    bool grow = false;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) grow |= lmx[rb] * sc_mul > m_ref[rb] + kMaxSlack;
+    if (__any(grow)) {
+      mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc);  // the accumulators may still be on their way
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        const float mx = xor32_max(lmx[rb]) * sc_mul;
+        const float m_new = fmaxf(m_ref[rb], ceilf(mx));
+        float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref[rb] - m_new);  // a power of two, or 0
+        m_ref[rb] = m_new;
+        m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
+        asm volatile("s_nop 1" : "+v"(alpha));
+        l_run[rb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          f32x16 o = o_acc[rb][db];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[r] *= alpha;
+          o_acc[rb][db] = o;
+        }
+        if (has_pending) {
+#pragma unroll
+          for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) pend[rb][s][w] = W::scale_pair(pend[rb][s][w], alpha);
+        }
+      }
+    }
+  };
+
+  // ---- the pinned step ---------------------------------------------------------------------------------------
+  // PAR = (b + 1) % 2: the buffer of block b+1 (the other receives block b+2 and held block b).  ka: lane addresses of
+  // the K operands of block b+2; kn: of the first PD operands of block b+3 (read at the end); va: lane addresses of the V
+  // operands of block b.
+  auto fast_step = [&](auto par_tag, const uint32_t (&ka)[NKK], const uint32_t (&kn)[PD], const uint32_t (&va)[DB]) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_tag)::value;
+    f32x16 (&s_cur)[RB] = sa[PAR];              // S(b+1), consumed by the softmax
+    f32x16 (&s_nxt)[RB] = sa[PAR ^ 1];          // S(b+2), produced
+    u32x4 (&p_cur)[RB][2] = pb[PAR ^ 1];        // P(b), consumed by the PV product
+    u32x4 (&p_nxt)[RB][2] = pb[PAR];            // P(b+1), produced
+    auto rk = [&](uint32_t a) __attribute__((always_inline)) -> u32x4 { return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)a; };
+    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 {
+      const int db = o / 2, s = o % 2;
+      const uint32_t a = va[db] + (uint32_t)(16 * s * RKL);
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)a));
+      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)(a + 8 * RKL)));
+      return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    };
+    float xa = 0.f, xb = 0.f, ea = 0.f, eb = 0.f;  // softmax values in flight between slots
+    float mx_part[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) mx_part[rb] = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < NQ + NP; ++k) {
+      // -- the MFMA of the slot and, behind an operand's last MFMA, the read of the operand PD further on
+      const int g = k / RB, rb = k % RB;  // operand of the step (K operands, then V operands), row block
+      if (k < NQ) {
+        if (g == 0) W::mfma_s0(s_nxt[rb], ops[g % PD], qf[rb][g]);
+        else W::mfma_s(s_nxt[rb], ops[g % PD], qf[rb][g]);
+      } else {
+        const int v = g - NKK, db = v / 2, s = v % 2;
+        W::mfma_o(o_acc[rb][db], ops[g % PD], p_cur[rb][s]);
+      }
+      if (rb == RB - 1) {
+        const int nx = g + PD;
+        if (nx < NKK) ops[g % PD] = rk(ka[nx]);
+        else if (nx < NKK + NVO) ops[g % PD] = rv(nx - NKK);
+        else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
+      }
+      // -- the softmax of block b+1: pair i = k / 2 = (row block, register pair); first half on even slots (the scaled
+      //    differences of pair i, and pair i-1 packed and summed), second half on odd slots (the exponentials)
+      {
+        const int ip = k / 2;
+        if ((k & 1) == 0) {
+          if (ip > 0) {
+            const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;
+            const uint32_t pk = H::pack(ea, eb);
+            p_nxt[prb][pr2 / 4][pr2 % 4] = pk;
+            l_run[prb] = W::add_pair(pk, l_run[prb]);
+          }
+          const int srb = ip / 8, sr2 = ip % 8;
+          xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
+          xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc_mul, m_neg[srb]);
+        } else {
+          ea = __builtin_amdgcn_exp2f(xa);
+          eb = __builtin_amdgcn_exp2f(xb);
+        }
+      }
+      // -- row maxima of S(b+2), whose MFMAs lie at least sixteen slots back: one three-way maximum per PV slot
+      if (k >= NQ) {
+        const int e = k - NQ, mrb = e / 8, mr2 = e % 8;
+        mx_part[mrb] = __builtin_fmaxf(__builtin_fmaxf(mx_part[mrb], s_nxt[mrb][2 * mr2]), s_nxt[mrb][2 * mr2 + 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    {  // the last pair
+      constexpr int jp = NPAIR - 1, prb = jp / 8, pr2 = jp % 8;
+      const uint32_t pk = H::pack(ea, eb);
+      p_nxt[prb][pr2 / 4][pr2 % 4] = pk;
+      l_run[prb] = W::add_pair(pk, l_run[prb]);
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) lmx[rb] = mx_part[rb];
+  };
+
+  // ---- the same step written plainly, with run-time flags ---------------------------------------------------------
+  // do_qk: block b+2 exists; do_sm: block b+1 exists; do_pv: block b >= 0; next_k: block b+3 exists (its first operands
+  // are read at the end); first: the first operands of block b+2 have not been read ahead.  kb2: first key of block b+2.
+  // koff / nkoff / voff: byte offsets (slot and half) of blocks b+2 / b+3 in the K ring and of block b in the V ring.
+  auto slow_step = [&](auto par_tag, uint32_t koff, uint32_t nkoff, uint32_t voff, bool do_qk, bool do_sm, bool do_pv, bool next_k, bool first, int kb2) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_tag)::value;
+    f32x16 (&s_cur)[RB] = sa[PAR];
+    f32x16 (&s_nxt)[RB] = sa[PAR ^ 1];
+    u32x4 (&p_cur)[RB][2] = pb[PAR ^ 1];
+    u32x4 (&p_nxt)[RB][2] = pb[PAR];
+    auto rk = [&](uint32_t off, int kk) __attribute__((always_inline)) -> u32x4 {
+      return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)(kaddr[kk] + off);
+    };
+    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 {
+      const int db = o / 2, s = o % 2;
+      const uint32_t a = vaddr[db] + voff + (uint32_t)(16 * s * RKL);
+      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)a));
+      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)(a + 8 * RKL)));
+      return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    };
+    if (do_qk) {
+      if (first) {
+#pragma unroll
+        for (int o = 0; o < PD; ++o) ops[o] = rk(koff, o);
+      }
+#pragma unroll
+      for (int g = 0; g < NKK; ++g) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          if (g == 0) W::mfma_s0(s_nxt[rb], ops[g % PD], qf[rb][g]);
+          else W::mfma_s(s_nxt[rb], ops[g % PD], qf[rb][g]);
+        }
+        if (g + PD < NKK) ops[g % PD] = rk(koff, g + PD);
+      }
+    }
+    if (do_sm) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r2 = 0; r2 < 8; ++r2) {
+          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[rb][2 * r2], sc_mul, m_neg[rb]));
+          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[rb][2 * r2 + 1], sc_mul, m_neg[rb]));
+          const uint32_t pk = H::pack(e0, e1);
+          p_nxt[rb][r2 / 4][r2 % 4] = pk;
+          l_run[rb] = W::add_pair(pk, l_run[rb]);
+        }
+    }
+    if (do_pv) {
+      u32x4 vo[PD];
+#pragma unroll
+      for (int o = 0; o < PD; ++o) vo[o] = rv(o);
+#pragma unroll
+      for (int g = 0; g < NVO; ++g) {
+        const int db = g / 2, s = g % 2;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          W::mfma_o(o_acc[rb][db], vo[g % PD], p_cur[rb][s]);
+        }
+        if (g + PD < NVO) vo[g % PD] = rv(g + PD);
+      }
+    }
+    if (do_qk) {  // mask S(b+2) in place and take the row maxima
+      mfma_settle(s_nxt[0], s_nxt[RB - 1]);
+      const bool plain = kb2 >= wave_lo && kb2 + BK <= wave_hi;  // no row of the wave masks a key of this block
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        float mx = -INFINITY;
+        const int lo_rel = row_lo[rb] - kb2 - 4 * hh;
+        const uint32_t span = (uint32_t)(row_hi[rb] - row_lo[rb]);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float sv = s_nxt[rb][r];
+          if (!plain) {
+            const int c = 8 * (r / 4) + (r % 4);
+            sv = ((uint32_t)(c - lo_rel) < span) ? sv : -INFINITY;
+            s_nxt[rb][r] = sv;
+          }
+          mx = fmaxf(mx, sv);
+        }
+        lmx[rb] = mx;
+      }
+    }
+    if (next_k) {
+#pragma unroll
+      for (int o = 0; o < PD; ++o) ops[o] = rk(nkoff, o);
+    }
+  };
+
+  // ---- the walk over the key range -------------------------------------------------------------------------
+  // Trip tt (tt = -1 .. n_tiles - 1) is the two steps b = 2 tt, 2 tt + 1: scores of tile tt+1, PV products of tile tt.
+  // It starts at a barrier behind which K(tt+2) and V(tt) are visible and the slots of K(tt) and V(tt-1) are free:
+  // V(tt+3) and K(tt+4) are requested into them.  Requests so far, in order: K0 V0 K1 V1 K2 | V2 K3 | V3 K4 | ...
+  issue_k();
+  issue_v();
+  issue_k();
+  issue_v();
+  issue_k();
+  // trips the pinned code may serve: tt >= 0, tile tt+2 exists, tile tt+1 unmasked for the whole wave
+  const int tt_fast_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT - 1);
+  const int tt_fast_hi = max(tt_fast_lo, min(n_tiles - 2, (wave_hi - kv_lo) / TT - 1));  // first trip behind them
+  const int n_blocks = 2 * n_tiles;
+  auto trip_head = [&](int tt) __attribute__((always_inline)) {
+    // in flight may stay what the previous trip requested: V(tt+2) and K(tt+3)
+    const int vin = (tt + 2 < n_tiles && tt + 2 >= 2) ? 1 : 0, kin = (tt + 3 < n_tiles && tt + 3 >= 3) ? 1 : 0;
+    if (vin + kin == 2) wait_loads_and_barrier<2 * NLH>();
+    else if (vin + kin == 1) wait_loads_and_barrier<NLH>();
+    else wait_loads_and_barrier<0>();
+    issue_v();
+    issue_k();
+  };
+  auto slow_trip = [&](int tt) __attribute__((always_inline)) {
+    trip_head(tt);
+#pragma unroll
+    for (int hb = 0; hb < 2; ++hb) {  // step b = 2 tt + hb: block b+2 = (tile tt+1, half hb), block b+3, block b = (tile tt, half hb)
+      const int b = 2 * tt + hb;
+      const bool do_qk = b + 2 < n_blocks, do_sm = b + 1 >= 0 && b + 1 < n_blocks, do_pv = b >= 0;
+      const bool next_k = b + 3 < n_blocks, first = b == -2;
+      const uint32_t koff = (uint32_t)(((tt + 1) & 3) * HALF + hb * BK * RKL);
+      const uint32_t nkoff = hb == 0 ? koff + BK * RKL : (uint32_t)(((tt + 2) & 3) * HALF);
+      const uint32_t voff = (uint32_t)((tt & 3) * HALF + hb * BK * RKL);
+      const int kb2 = kv_lo + (b + 2) * BK;
+      // buffers: block b+1 in (b + 1) % 2 = 1 - hb
+      if (hb == 0) {
+        if (do_sm) check(pb[0], do_pv);
+        slow_step(std::integral_constant<int, 1>{}, koff, nkoff, voff, do_qk, do_sm, do_pv, next_k, first, kb2);
+      } else {
+        if (do_sm) check(pb[1], do_pv);
+        slow_step(std::integral_constant<int, 0>{}, koff, nkoff, voff, do_qk, do_sm, do_pv, next_k, first, kb2);
+      }
+    }
+  };
+  int tt = -1;
+  for (; tt < tt_fast_lo; ++tt) slow_trip(tt);
+  for (; tt < tt_fast_hi; ++tt) {
+    trip_head(tt);
+    // lane addresses of this trip's operands: K of tile tt+1, the first K operands of tile tt+2, V of tile tt
+    const uint32_t k_off = (uint32_t)(((tt + 1) & 3) * HALF), kn_off = (uint32_t)(((tt + 2) & 3) * HALF), v_off = (uint32_t)((tt & 3) * HALF);
+    uint32_t ka0[NKK], ka1[NKK], kn0[PD], kn1[PD], va0[DB], va1[DB];
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      ka0[kk] = kaddr[kk] + k_off;
+      ka1[kk] = ka0[kk] + BK * RKL;  // a constant apart: folds into the instruction's offset
+    }
+#pragma unroll
+    for (int o = 0; o < PD; ++o) {
+      kn0[o] = ka1[o];
+      kn1[o] = kaddr[o] + kn_off;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      va0[db] = vaddr[db] + v_off;
+      va1[db] = va0[db] + BK * RKL;
+    }
+    check(pb[0], true);
+    fast_step(std::integral_constant<int, 1>{}, ka0, kn0, va0);
+    check(pb[1], true);
+    fast_step(std::integral_constant<int, 0>{}, ka1, kn1, va1);
+  }
+  for (; tt < n_tiles; ++tt) slow_trip(tt);
+
+  // ---- epilogue -----------------------------------------------------------------------------------------
+  mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc);
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 32);
+    if (row_ok[rb]) {
+      if (single) {
+        const float l_fin = with_sink(p, out_head[rb], m_ref[rb], l_tot);
+        const float inv = l_fin > 0.f ? 1.f / l_fin : 0.f;
+        uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * p.Dq + 4 * hh;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const f32x16 o = o_acc[rb][db];
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {  // registers 4 q4 .. 4 q4 + 3 are dims 32 db + 8 q4 + 4 hh + 0..3
+            const u32x2 w = {H::pack(o[4 * q4] * inv, o[4 * q4 + 1] * inv), H::pack(o[4 * q4 + 2] * inv, o[4 * q4 + 3] * inv)};
+            if (32 * db + 8 * q4 + 4 * hh < p.Dq) *(u32x2*)(orow + 32 * db + 8 * q4) = w;
+          }
+        }
+      } else {
+        const int64_t pslot = ((int64_t)chunk * p.T + out_tok[rb]) * p.Hq + out_head[rb];
+        float* prow = p.pre_o + pslot * D + 4 * hh;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const f32x16 o = o_acc[rb][db];
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4)
+            *(f32x4*)(prow + 32 * db + 8 * q4) = (f32x4){o[4 * q4], o[4 * q4 + 1], o[4 * q4 + 2], o[4 * q4 + 3]};
+        }
+        if (hh == 0) {
+          p.pre_ml[pslot * 2 + 0] = m_ref[rb];
+          p.pre_ml[pslot * 2 + 1] = l_tot;
+        }
+      }
+    }
+  }
+}
+
+template <int D, int NW, int RB, int HT>
+static int launch_x32(hipStream_t stream, const AttnParams& p) {
+  const int64_t slots = ((int64_t)p.T * p.group) / kWideRows + p.S;  // upper bound on row tiles of the batch
+  const int64_t blocks = slots * p.Hkv * p.pre_max_chunks;
+  if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL((attn_prefill_x32_kernel<D, NW, RB, HT>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  return (int)hipGetLastError();
+}
+
+// bf16 (or float16) pages of a multiple of 64 tokens, head size 128, no soft cap
+bool prefill_x32_supported(const AttnParams& p) {
+  return (p.kv_dtype == RPA_BF16 || p.kv_dtype == RPA_F16) && p.page_size % 64 == 0 && p.D == 128 && !(p.softcap > 0.f) &&
+         (int64_t)64 * p.token_stride < ((int64_t)1 << 31);
+}
+
+int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p) {
+  if (p.kv_dtype == RPA_F16) return launch_x32<128, 4, 2, RPA_F16>(stream, p);
+  return launch_x32<128, 4, 2, RPA_BF16>(stream, p);
+}
+
+}  // namespace rpa

@@ -12,7 +12,7 @@ constexpr int kRowBlock = 16;      // MFMA M/N extent: rows (token, group-head p
 constexpr int kMaxSplitsCap = 256;   // hard upper bound on split-K partials per sequence
 constexpr int kPlanHeader = 16;      // ints before the prefix array in the decode plan
 constexpr int kMaxDecodeWgs = 4096;  // persistent decode workgroups per KV-head group
-constexpr int kPrefillRows = 128;    // query rows (token x group head) one prefill workgroup owns
+constexpr int kPrefillRows = 128;    // query rows (token x group head) one prefill workgroup owns (the 32x32-tile kernel: 256; AttnParams::pre_rows)
 constexpr int kMaxPrefillChunks = 8; // key chunks one prefill row tile may be split into
 constexpr int kMinPrefillChunk = 2048; // fewest keys of such a chunk
 constexpr int kMaxDevices = 64;      // devices of one process the per-device caches hold
@@ -62,6 +62,7 @@ struct AttnParams {
   int pre_max_chunks;  // chunks the prefill partial buffers hold; 1 = never split
   int pre_auto;        // 1: the plan kernel sets the chunk length from the batch's lengths; 0: pre_chunk as given
   int pre_slots;       // workgroups of the prefill kernel the chip holds at once
+  int pre_rows;        // query rows (token x group head) one workgroup of the call's prefill kernel owns: 128 or 256
   int decode_sync;   // decode workgroups re-align their waves with a barrier every this many tiles (power of two), 0 = never
   int decode_pace;   // 0: the decode kernel never pauses a wave (see PACE there); default 1
   int decode_dma;    // 1: bf16 decode tiles go global -> LDS directly where that kernel applies; 0: always through registers
@@ -111,7 +112,7 @@ __device__ __forceinline__ float with_sink(const AttnParams& p, int hq, float m_
   return l + __builtin_amdgcn_exp2f(__builtin_fmaf(p.sinks[hq], 1.4426950408889634f, -m_log2));
 }
 
-// Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + kPrefillRows) of a sequence) must visit, kv_lo
+// Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + pre_rows) of a sequence) must visit, kv_lo
 // rounded down to 64, and the split-K chunks the prefill kernel cuts it into: the range over the chunk length the
 // plan kernel chose (plan[4]), rounded to the nearest count the partial buffers hold, all chunks of one length (a
 // multiple of 64; the last one holds what is left), so that the workgroups of a sequence finish together.
@@ -121,7 +122,7 @@ struct PrefillTile {
 __device__ __forceinline__ PrefillTile prefill_tile(const AttnParams& p, const SeqPlan& sp, int R0) {
   PrefillTile t;
   const int rows_total = sp.q_len * p.group;
-  const int last_row = min(R0 + kPrefillRows, rows_total) - 1;
+  const int last_row = min(R0 + p.pre_rows, rows_total) - 1;
   const int base_pos = sp.ctx - sp.q_len;
   t.kv_hi = min(sp.ctx, base_pos + last_row / p.group + 1);
   t.vis_lo = (p.window > 0) ? max(base_pos + R0 / p.group - p.window + 1, 0) : 0;
@@ -276,6 +277,8 @@ int decode_row_limit(int T, int S, int D, int kv_dtype);
 bool prefill_supported(const AttnParams& p);
 bool prefill_dma_supported(const AttnParams& p);
 int launch_attn_prefill_dma8(hipStream_t stream, const AttnParams& p);  // 8-bit pages: codes loaded straight into LDS, widened there
+int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p);   // bf16 pages, 32x32x16 tiles, 256-row workgroups
+bool prefill_x32_supported(const AttnParams& p);
 bool prefill_dma8_supported(const AttnParams& p);
 
 }  // namespace rpa

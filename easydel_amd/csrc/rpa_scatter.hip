@@ -216,127 +216,6 @@ int launch_scatter_ragged_quant(hipStream_t stream, const void* key, const void*
   return (int)hipGetLastError();
 }
 
-// Plain grid-stride copy of 16-byte vectors: the known-size kernel that calibrates HBM traffic counters.
-__global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n16) {
-  const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x; k < n16; k += stride) dst[k] = src[k];
-}
-
-int launch_calibration_copy(hipStream_t stream, void* dst, const void* src, size_t bytes) {
-  hipLaunchKernelGGL(calibration_copy_kernel, dim3(4096), dim3(256), 0, stream, (const uint4*)src, (uint4*)dst, bytes >> 4);
-  return (int)hipGetLastError();
-}
-
-// Read-only probe of the memory system: `workgroups` workgroups of eight waves (96 KiB of LDS each, so one per CU), every
-// wave streaming its own contiguous share of the buffer with 16-byte loads, DEPTH instructions (KiB) in flight.
-typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
-template <int DEPTH>
-__global__ __launch_bounds__(512) void read_probe_kernel(const probe_u32x4* __restrict__ src, size_t kib_per_wave, uint32_t* __restrict__ sink) {
-  __shared__ char occupy[98304];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const probe_u32x4* p = src + ((size_t)blockIdx.x * 8 + wave) * kib_per_wave * 64 + lane;
-  probe_u32x4 acc = {0u, 0u, 0u, 0u};
-  for (size_t c = 0; c + DEPTH <= kib_per_wave; c += DEPTH) {
-    probe_u32x4 v[DEPTH];
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) v[d] = __builtin_nontemporal_load(p + (c + d) * 64);
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) acc ^= v[d];
-  }
-  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) sink[0] = occupy[lane];  // keeps the loads and the LDS alive
-}
-
-// Returns the bytes the launch reads (0: bad arguments): bytes / (8 workgroups) rounded down to whole rounds of loads.
-size_t launch_read_probe(hipStream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
-                         uint32_t* sink) {
-  if (workgroups <= 0) return 0;
-  size_t per = bytes / ((size_t)workgroups * 8) / 1024;
-  per -= per % (size_t)(kib_in_flight_per_wave > 0 ? kib_in_flight_per_wave : 1);
-  if (per == 0) return 0;
-#define RPA_PROBE(D) hipLaunchKernelGGL(read_probe_kernel<D>, dim3(workgroups), dim3(512), 0, stream, (const probe_u32x4*)src, per, sink)
-  switch (kib_in_flight_per_wave) {
-    case 2: RPA_PROBE(2); break;
-    case 4: RPA_PROBE(4); break;
-    case 8: RPA_PROBE(8); break;
-    case 16: RPA_PROBE(16); break;
-    case 32: RPA_PROBE(32); break;
-    default: return 0;
-  }
-#undef RPA_PROBE
-  return hipGetLastError() == hipSuccess ? per * 1024 * 8 * (size_t)workgroups : 0;
-}
-
-// The same reader over pages: the buffer is cut into chunks of `chunk_kib` KiB, a workgroup visits its chunks in a
-// scattered order (a multiplicative permutation of the chunk numbers, as a block table of a long-lived pool would hand
-// them out), DEPTH KiB per wave in flight, i.e. DEPTH / (chunk_kib / 8) chunks per workgroup.  SPLIT says how the eight
-// waves share a chunk: 0 contiguous eighths; 1 and 2 the decode kernel's own split -- the chunk is rows of 4 KiB (a
-// token's keys and values of eight heads) and wave w reads bytes [512 w, 512 w + 512) of every row, two rows per
-// instruction -- with non-temporal (1) or ordinary (2) loads.
-template <int DEPTH, int SPLIT>
-__global__ __launch_bounds__(512) void read_probe_paged_kernel(const probe_u32x4* __restrict__ src, uint32_t chunk_mask, uint32_t chunks_per_wg,
-                                                               uint32_t kib_per_wave_chunk, uint32_t* __restrict__ sink) {
-  __shared__ char occupy[98304];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const uint32_t per = kib_per_wave_chunk;          // KiB of a chunk one wave reads (DEPTH is a multiple of it)
-  const uint32_t group = DEPTH / per;               // chunks in flight per workgroup
-  probe_u32x4 acc = {0u, 0u, 0u, 0u};
-  for (uint32_t c = 0; c + group <= chunks_per_wg; c += group) {
-    probe_u32x4 v[DEPTH];
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const uint32_t step = c + (uint32_t)d / per;                                               // which of the workgroup's chunks
-      const uint32_t chunk = ((blockIdx.x * chunks_per_wg + step) * 0x9E3779B1u) & chunk_mask;  // where it lies
-      if constexpr (SPLIT == 0) {
-        const probe_u32x4* p = src + ((size_t)chunk * 8 + wave) * per * 64 + lane;
-        v[d] = __builtin_nontemporal_load(p + ((uint32_t)d % per) * 64);
-      } else {
-        const uint32_t row = 2 * ((uint32_t)d % per) + (lane >> 5);  // of the chunk's 2 per rows
-        const probe_u32x4* p = src + (size_t)chunk * 8 * per * 64 + (size_t)row * 256 + wave * 32 + (lane & 31);
-        if constexpr (SPLIT == 1) v[d] = __builtin_nontemporal_load(p);
-        else v[d] = *p;
-      }
-    }
-#pragma unroll
-    for (int d = 0; d < DEPTH; ++d) acc ^= v[d];
-  }
-  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) sink[0] = occupy[lane];  // keeps the loads and the LDS alive
-}
-
-// Returns the bytes the launch reads (0: bad arguments).  The number of chunks in the buffer is rounded down to a power of
-// two (the permutation needs one), each workgroup takes an equal share of them in whole groups.
-size_t launch_read_probe_paged(hipStream_t stream, const void* src, size_t bytes, int workgroups, int kib_in_flight_per_wave,
-                               int chunk_kib, int split, uint32_t* sink) {
-  if (workgroups <= 0 || chunk_kib < 8 || (chunk_kib & 7) || kib_in_flight_per_wave <= 0 || split < 0 || split > 2) return 0;
-  const uint32_t per = (uint32_t)chunk_kib / 8;
-  if ((uint32_t)kib_in_flight_per_wave % per) return 0;
-  size_t n_chunks = bytes / ((size_t)chunk_kib * 1024);
-  if (n_chunks == 0) return 0;
-  size_t pow2 = 1;
-  while (pow2 * 2 <= n_chunks && pow2 < ((size_t)1 << 31)) pow2 *= 2;
-  const uint32_t group = (uint32_t)kib_in_flight_per_wave / per;
-  uint32_t per_wg = (uint32_t)(pow2 / (size_t)workgroups);
-  per_wg -= per_wg % group;
-  if (per_wg == 0) return 0;
-#define RPA_PROBE_S(D, S)                                                                                                \
-  hipLaunchKernelGGL((read_probe_paged_kernel<D, S>), dim3(workgroups), dim3(512), 0, stream, (const probe_u32x4*)src, \
-                     (uint32_t)(pow2 - 1), per_wg, per, sink)
-#define RPA_PROBE(D)                \
-  if (split == 0) RPA_PROBE_S(D, 0); \
-  else if (split == 1) RPA_PROBE_S(D, 1); \
-  else RPA_PROBE_S(D, 2)
-  switch (kib_in_flight_per_wave) {
-    case 2: RPA_PROBE(2); break;
-    case 4: RPA_PROBE(4); break;
-    case 8: RPA_PROBE(8); break;
-    case 16: RPA_PROBE(16); break;
-    case 32: RPA_PROBE(32); break;
-    default: return 0;
-  }
-#undef RPA_PROBE
-#undef RPA_PROBE_S
-  return hipGetLastError() == hipSuccess ? (size_t)per_wg * (size_t)chunk_kib * 1024 * (size_t)workgroups : 0;
-}
-
 int launch_scatter_slices(hipStream_t stream, const void* new_kv, const int32_t* si, const int32_t* num_slices,
                           void* pages, int T, int N, int64_t num_positions, int page_size, int64_t row_bytes,
                           int shard) {

@@ -10,9 +10,12 @@ package imports it.  It is what a maintainer of the reference imports from the g
 ``unified_attention.py:363-388``, ``multi_latent_ragged_page_attention.py:495-511``,
 ``easydel/caching/ragged_page/utils.py:302-387``).
 
-Every wrapper sizes the scratch buffer from the static shapes (``rpa_attention_workspace_bytes``: plain host
-arithmetic, no device call) and declares it as an extra result, so XLA owns it; buffers updated in place are donated
-through ``input_output_aliases``.
+Every wrapper sizes the scratch buffer from the static shapes (``rpa_attention_workspace_bytes``) and declares it as
+an extra result, so XLA owns it; buffers updated in place are donated through ``input_output_aliases``.  The sizing
+functions launch nothing, but they ask HIP for the current device's CU count and read the calling thread's test
+knobs, so a size taken on the tracing thread may differ from what the executing thread and device would ask for.  That
+is safe -- a call lays its workspace out from the bytes it is handed and splits less when they are fewer -- but a
+different layout means a different split-K rounding, so results are only bit-identical for equal workspace sizes.
 """
 
 from __future__ import annotations

@@ -119,7 +119,7 @@ class _RaggedPageAttn(OperationImpl):
     def forward_v3_dp_local_shard(self, query, key, value, local_kv_pages, cache_metadata: RaggedPagesMetadata,
                                   shard_index: int, num_shards: int, softmax_scale: float | None = None,
                                   logits_soft_cap: float | None = None, sliding_window: int | None = None,
-                                  softmax_aux=None, **ignore):
+                                  softmax_aux=None, local_kv_scales=None, num_kv_heads: int | None = None, **ignore):
         """What one data-parallel rank computes when the page pool is sharded over ranks and every sequence's pages
         live on the rank that owns its metadata row (the body of the reference's ``shard_map`` at :645-717, before the
         sum over ranks): the rank takes its ``S / num_shards`` rows of ``context_lens``, ``pages_tables`` and
@@ -128,8 +128,21 @@ class _RaggedPageAttn(OperationImpl):
         pool, runs the fused write + attention on its pages, and returns output rows that are zero for the tokens of
         other ranks' sequences.  Returns ``(local_output, local_kv_pages)``; the ranks' outputs are then summed in
         float32 (:699-717) -- ``dp_local_reduce`` does that for outputs gathered on one device.  Nothing here reads
-        device values on the host."""
+        device values on the host.
+
+        A rank's share of a scaled 8-bit pool comes with its rows of the scales, ``local_kv_scales [local_pages, C]``:
+        the write then quantises and the call returns ``(local_output, local_kv_pages, local_kv_scales)``.  int8 pages
+        without scales are refused (only fp8 pages may hold bare codes, the reference's cast-only cache)."""
         context_lens, tables, query_start_loc, distribution = dp_local_metadata(cache_metadata, shard_index, num_shards, int(local_kv_pages.shape[0]))
+        if local_kv_scales is not None:
+            if key.dtype not in (torch.float32, torch.bfloat16):
+                key, value = key.to(torch.float32), value.to(torch.float32)
+            return kernels.ragged_paged_attention_v3_quantised(
+                query, key.contiguous(), value.to(key.dtype).contiguous(), local_kv_pages, local_kv_scales, context_lens, tables,
+                query_start_loc, distribution, softmax_scale=softmax_scale, sliding_window=sliding_window,
+                logits_soft_cap=logits_soft_cap, num_kv_heads=num_kv_heads, softmax_aux=softmax_aux)
+        if local_kv_pages.dtype == torch.int8:
+            raise ValueError("int8 KV pages are always scaled: pass this rank's rows of the scales as local_kv_scales")
         if key.dtype != local_kv_pages.dtype or value.dtype != local_kv_pages.dtype:
             key, value = key.to(local_kv_pages.dtype), value.to(local_kv_pages.dtype)
         # tokens outside [query_start_loc[0], query_start_loc[total]) belong to other ranks: the kernels write zeros

@@ -138,8 +138,9 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
  *
  *   q             device, [T][Hq][D]          q_dtype in {RPA_F32, RPA_BF16, RPA_F16}
  *   kv_pages      device, [P][page_size][C][Dp] kv_dtype
- *   kv_scales     device, float [P][C] or NULL; 8-bit pages only.  NULL with 8-bit pages: the codes are the values
- *                 (scale 1), which is how the reference stores an fp8 cache (a bare cast, ragged_page_attention.py:570-580)
+ *   kv_scales     device, float [P][C] or NULL; 8-bit pages only.  NULL with fp8 pages: the codes are the values
+ *                 (scale 1), which is how the reference stores an fp8 cache (a bare cast, ragged_page_attention.py:570-580).
+ *                 int8 pages always need their scales (RPA_ERR_INVALID_ARGUMENT without).
  *   context_lens  device, int32 [S]           tokens in the cache per sequence, new ones included
  *   block_tables  device, int32 [S][M]
  *   query_start_loc device, int32 [S+1]
@@ -156,6 +157,11 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
  *                 less than one: out = sum_j exp(s_j) v_j / (sum_j exp(s_j) + exp(softmax_aux[hq])).  This is the
  *                 GPT-OSS definition the reference's model file feeds (modules/gpt_oss/modeling_gpt_oss.py:436-442).
  * Query row r of sequence i sits at position ctx_i - q_len_i + r and attends causally.
+ * Limits: S * M * page_size < 2^31 (what the block tables of one call can address; RPA_ERR_UNSUPPORTED beyond).
+ * Padded head storage (Dp > D): the Dp - D padding elements of every stored row must be zero, or at least finite --
+ * the matrix-core kernels multiply them by zero query elements, and 0 x NaN / Inf would reach the scores.  Pages written
+ * through this library have zero padding (a pool must start zeroed, as the reference's does); a pool filled by another
+ * writer must keep that promise.
  */
 int rpa_ragged_paged_attention(rpa_stream_t stream, const void* q, const void* kv_pages,
                                const float* kv_scales, const int32_t* context_lens,
@@ -211,6 +217,9 @@ int rpa_ragged_paged_attention_v3(rpa_stream_t stream, const void* q, const void
  * workspace would allow.
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race --
  * serialise them.  Nothing in the array has to survive or be cleared between calls (each call writes what it reads).
+ * The first call on a device looks up the array's address and the device's CU count, and the first call that reaches a
+ * kernel variant its occupancy; these are not stream operations and may be refused while a stream is being captured.
+ * Before capturing this entry point, make one ordinary call with the same shapes and dtypes on that device.
  */
 #define RPA_STATIC_WORKSPACE_BYTES (64u << 20)
 int rpa_ragged_paged_attention_v3_static(rpa_stream_t stream, const void* q, const void* key, const void* value,

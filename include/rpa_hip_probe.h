@@ -1,6 +1,9 @@
 /*
  * rpa_hip_probe.h -- test and measurement aids of librpa_hip.so, kept apart from the operator entry points of
- * rpa_hip.h.  Nothing here has a counterpart in the reference and a serving runtime needs none of it.
+ * rpa_hip.h.  Nothing here has a counterpart in the reference and a serving runtime needs none of it.  The measurement
+ * kernels, and the two knobs of rpa_set_tunable that change what a call computes with ("stages", "force_generic"), exist
+ * only in a library built with -DRPA_PROBES (easydel_amd/build.py builds that one for tests and benchmarks; its
+ * --product switch leaves them out: rpa_set_tunable then answers -1 for those names and the probes are not exported).
  */
 #ifndef RPA_HIP_PROBE_H_
 #define RPA_HIP_PROBE_H_
@@ -44,6 +47,22 @@ size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, 
                             int chunk_kib, int split, void* sink);
 
 /*
+ * Measurement aid with no counterpart in the reference: what a stream of bf16 MFMAs sustains on this chip when its A
+ * operands come out of LDS, i.e. the ceiling of the prefill kernels' inner loops.  One workgroup of four wavefronts per
+ * CU (waves_per_simd = 1) or two (= 2) issue, per wavefront, 32 * mfmas_per_operand * iters MFMAs of `shape` (0:
+ * 16x16x32, 1: 32x32x16); `source` says where the A operands come from: 0 registers, 1 ds_read_b128 in the pattern the
+ * prefill kernels read K tiles with, 2 pairs of ds_read_b64_tr_b16 in their V pattern; every operand feeds
+ * mfmas_per_operand (1, 2 or 4) MFMAs with distinct B operands and accumulators, as a wavefront that owns so many row
+ * blocks would; operands are read four ahead.  Returns the floating-point operations of the launch (0 on bad
+ * arguments); time the launch with events on `stream`.  `clocks` is two 8-byte device words the caller zeroes: the
+ * launch adds shader-clock cycles to the first and ticks of the 100 MHz wall clock to the second, summed over the
+ * workgroups, so 100 * clocks[0] / clocks[1] is the clock in MHz the kernel ran at.  `sink` is one device word, never
+ * written in practice.
+ */
+double rpa_mfma_probe(rpa_stream_t stream, int shape, int source, int mfmas_per_operand, int waves_per_simd, int iters,
+                      void* clocks, void* sink);
+
+/*
  * Knobs for tests and measurement.  They belong to the calling thread: a value set here is seen only by entry points
  * the same thread calls afterwards (each call reads them once, when it starts), so threads that never call this function
  * always run with the defaults.  Returns the previous value, -1 for an unknown name.
@@ -63,6 +82,8 @@ size_t rpa_read_probe_paged(rpa_stream_t stream, const void* src, size_t bytes, 
  *                    fixed from the block-table bound (1 = never split); set it before sizing the workspace
  *   "prefill_dma"    1 (default): prefill tiles are loaded global -> LDS by the load unit where those kernels apply
  *                    (page_size % 32 == 0); 0: every prefill tile is staged through registers (bf16 / 8-bit pages only)
+ *   "prefill_x32"    1 (default): bf16 / float16 pages of a multiple of 64 tokens at head size 128, without soft cap, take the
+ *                    prefill kernel built on 32x32x16 tiles (256-row workgroups); 0: never
  *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
  *                    the shapes, and batches of few row tiles cut by a chunk length chosen on the device from their
  *                    own lengths); set it before sizing the workspace

@@ -27,8 +27,8 @@ def test_header_symbols_are_exported_and_bound():
     lib = ctypes.CDLL(str(_lib.LIB_PATH))
     for n in names:
         assert hasattr(lib, n), f"{n} declared in rpa_hip.h but not exported by librpa_hip.so"
-        assert n in _lib.SIGNATURES, f"{n} has no ctypes prototype in easydel_amd/_lib.py"
-    assert sorted(_lib.SIGNATURES) == names
+        assert n in _lib.SIGNATURES or n in _lib.PROBE_SIGNATURES, f"{n} has no ctypes prototype in easydel_amd/_lib.py"
+    assert sorted(list(_lib.SIGNATURES) + list(_lib.PROBE_SIGNATURES)) == names
 
 
 def test_host_only_entry_points():
@@ -50,6 +50,20 @@ def test_host_only_entry_points():
     assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"Dp" in lib.rpa_last_error()  # stored rows narrower than the head
     with pytest.raises(_lib.RpaError):
         _lib.check(rc)
+    # the block tables of one call may address at most 2^31 - 1 tokens (S * M * page_size): refused before any device work
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 4096, 8192, 1 << 20, 64, 8, 2, 64, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_UNSUPPORTED and b"2^31" in lib.rpa_last_error()
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 4096, 8191, 1 << 20, 64, 8, 2, 64, 64, 4, 1, 1, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"null pointer" in lib.rpa_last_error()  # one page less per row: the sizes pass
+    # int8 pages are always scaled; fp8 pages may hold bare codes (the reference's cast-only cache)
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 1, 3, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"int8 KV pages need kv_scales" in lib.rpa_last_error()
+    rc = lib.rpa_ragged_paged_attention(None, None, None, None, None, None, None, None, None, None, 0,
+                                        4, 1, 1, 1, 16, 8, 2, 64, 64, 4, 1, 2, 1.0, 0, 0.0, None)
+    assert rc == _lib.RPA_ERR_INVALID_ARGUMENT and b"null pointer" in lib.rpa_last_error()
     # pointers are checked for null and alignment before anything is launched (the values below are never dereferenced)
     a = 0x7000_0000_0000
     rc = lib.rpa_ragged_paged_attention(None, a + 8, a, None, a, a, a, a, a, a, 1 << 20,
@@ -78,6 +92,28 @@ def test_host_only_entry_points():
     assert lib.rpa_attention_workspace_bytes(256, 256, 128, 64, 32, 8, 128, 1, 1) < n
     _lib.set_tunable("max_splits", prev)
     assert _lib.set_tunable("no_such_knob", 1) == -1
+    assert lib.rpa_mfma_probe(None, 1, 1, 2, 1, 100, None, None) == 0.0 and b"rpa_mfma_probe" in lib.rpa_last_error()
+    assert lib.rpa_mfma_probe(None, 1, 1, 3, 1, 100, a, a) == 0.0  # 1, 2 or 4 MFMAs per operand
+
+
+def test_product_build_has_no_probes_and_no_stage_knob(tmp_path):
+    """The API source compiled without -DRPA_PROBES (what `python -m easydel_amd.build --product` links) neither defines
+    the measurement entry points nor knows the knobs that change what a call computes with."""
+    import subprocess
+
+    from easydel_amd import build
+
+    obj = tmp_path / "rpa_api_product.o"
+    cmd = [build._hipcc(), *build.HIPCC_FLAGS, "-c", str(build.CSRC / "rpa_api.hip"), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    syms = subprocess.run(["nm", "--defined-only", str(obj)], capture_output=True, text=True).stdout
+    for name in _lib.PROBE_SIGNATURES:
+        assert name not in syms, f"{name} is defined in a product build"
+    assert "rpa_ragged_paged_attention_v3" in syms and "rpa_set_tunable" in syms
+    strings = subprocess.run(["strings", str(obj)], capture_output=True, text=True).stdout
+    assert "force_generic" not in strings and "\nstages\n" not in "\n" + strings + "\n"
+    assert "decode_sync" in strings  # the tuning knobs stay
 
 
 def test_multi_latent_entry_points_validate_before_any_device_work():

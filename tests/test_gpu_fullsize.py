@@ -6,7 +6,8 @@ import pytest
 import torch
 
 import rpa_testlib as tl
-from easydel_amd import kernels, workloads
+import bench_workloads as workloads
+from easydel_amd import kernels
 from rpa_testlib import orc
 
 pytestmark = pytest.mark.gpu
