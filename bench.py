@@ -42,6 +42,11 @@ def parse_args():
                          "unified: separate K and V pools [P, page, Hkv, D], two slice scatters then the attention call")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-configs", action="store_true",
+                    help="default workload only: do not measure the other benchmark configurations afterwards")
+    ap.add_argument("--mfma-probe", action="store_true",
+                    help="instead of a workload: the library's matrix-core feed probe (bf16 MFMA streams with operands from "
+                         "registers or LDS, both tile shapes, 1 / 2 / 4 MFMAs per operand, one and two waves per SIMD), one line per setting")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
     ap.add_argument("--decode-wgs", type=int, default=0)
     ap.add_argument("--prefill-chunks", type=int, default=0)
@@ -340,45 +345,59 @@ def read_probe_paged():
                                   "gb_per_s_per_workgroup": round(read / best / 1e6 / wgs, 1)}), flush=True)
 
 
-def main():
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
+def mfma_probe():
+    """What a stream of bf16 MFMAs sustains with its A operands in registers or read from LDS the way the prefill kernels
+    read K and V tiles: rpa_mfma_probe, best of three timed launches per setting, with the clock the kernel ran at."""
     import torch
 
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
+    from easydel_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    shapes = {0: "16x16x32", 1: "32x32x16"}
+    sources = {0: "registers", 1: "LDS, ds_read_b128 (K pattern)", 2: "LDS, 2 x ds_read_b64_tr_b16 (V pattern)"}
+    for source in (0, 1, 2):
+        for shape in (0, 1):
+            for reuse in (1, 2, 4):
+                for waves in (1, 2):
+                    iters = 8000 // reuse
+                    best, flops, mhz = None, 0.0, 0.0
+                    for rep in range(4):
+                        clocks.zero_()
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record(stream)
+                        flops = lib.rpa_mfma_probe(stream.cuda_stream, shape, source, reuse, waves, iters, clocks.data_ptr(), sink.data_ptr())
+                        e1.record(stream)
+                        e1.synchronize()
+                        if flops == 0.0:
+                            raise RuntimeError(lib.rpa_last_error().decode())
+                        ms = e0.elapsed_time(e1)
+                        if rep > 0 and (best is None or ms < best):
+                            best = ms
+                            c = clocks.cpu().numpy()
+                            mhz = 100.0 * float(c[0]) / float(c[1])
+                    tf = flops / best / 1e9
+                    print(json.dumps({"probe": "mfma", "shape": shapes[shape], "a_operands": sources[source], "mfmas_per_operand": reuse,
+                                      "waves_per_simd": waves, "ms": round(best, 4), "tflop_per_s": round(tf, 1),
+                                      "frac_of_2500": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "clock_mhz": round(mhz)}), flush=True)
+
+
+_KEEP = []
+
+
+def measure(args, workload, with_cpu):
+    """One workload: the whole step timed on the host clock around synchronised launches, its kernels timed alone with
+    events on the launch stream, and (with_cpu) the C restatement timed on the host cores.  Returns the result record."""
+    import torch
+
     import bench_workloads as workloads
     from easydel_amd import _lib, kernels
 
-    _lib.load()
-    if args.read_probe:
-        return read_probe()
-    if args.read_probe_paged:
-        return read_probe_paged()
-    if args.workload.startswith("mla-"):
-        if args.mla_chunks:
-            _lib.set_tunable("mla_chunks", args.mla_chunks)
-        if args.mla_min_chunk:
-            _lib.set_tunable("mla_min_chunk", args.mla_min_chunk)
-        return bench_mla(args)
-    if args.decode_wgs:
-        _lib.set_tunable("decode_wgs", args.decode_wgs)
-    if args.decode_sync >= 0:
-        _lib.set_tunable("decode_sync", args.decode_sync)
-    if args.decode_dma >= 0:
-        _lib.set_tunable("decode_dma", args.decode_dma)
-    if args.prefill_chunks:
-        _lib.set_tunable("prefill_chunks", args.prefill_chunks)
-    if args.max_splits:
-        _lib.set_tunable("max_splits", args.max_splits)
-    if args.prefill_x32 >= 0:
-        _lib.set_tunable("prefill_x32", args.prefill_x32)
-
     dev = torch.device("cuda:0")
-    w = build_workload(args.workload, args.seed, args.sequential_pages)
+    w = build_workload(workload, args.seed, args.sequential_pages)
     tens = workloads.device_tensors(w, dev, seed=args.seed)
     quant = w.kv_dtype in ("fp8", "int8")
     out = torch.empty_like(tens["query"])
@@ -477,7 +496,7 @@ def main():
             "frac": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "traffic_source": None,
             "algorithmic_bytes_per_launch": nbytes, "kernel_ms": ms}
         if not unified:
-            kern["attn_decode_kernel"]["traffic"], kern["attn_decode_kernel"]["traffic_source"] = measured_traffic(args.workload)
+            kern["attn_decode_kernel"]["traffic"], kern["attn_decode_kernel"]["traffic_source"] = measured_traffic(workload)
     if (~small & (w.q_lens > 0)).any():
         ms = time_stage(4, args.steps)
         flops = w.attention_flops(~small)
@@ -488,7 +507,7 @@ def main():
             "kernel_ms": ms}
         if not unified:
             kern["attn_prefill_kernel"]["traffic"], kern["attn_prefill_kernel"]["traffic_source"] = \
-                measured_traffic(args.workload, "attn_prefill_kernel")
+                measured_traffic(workload, "attn_prefill_kernel")
     _lib.set_tunable("stages", prev)
     dominant = max(kern, key=lambda k: kern[k]["kernel_ms"])
     roofline = dict(kern[dominant], kernel=dominant)
@@ -532,7 +551,7 @@ def main():
         result["attn_hbm_tb_s"] = kern["attn_decode_kernel"]["achieved"] / 1e3
         result["attn_hbm_pct_of_8tb_s"] = 100.0 * kern["attn_decode_kernel"]["frac"]
 
-    if not args.no_cpu_baseline:
+    if with_cpu and not args.no_cpu_baseline:
         # the whole batch fits the host here; it is re-run for about 10 s
         sample = args.cpu_sample_seqs or w.S
         base, cpu_out, rows = cpu_baseline(w, tens, sample)
@@ -544,6 +563,67 @@ def main():
     else:
         result["cpu_baseline"] = None
 
+    _KEEP.append((tens, out))  # pools stay allocated: handing blocks of this size back to the driver slows later kernels by a few percent
+    return result
+
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    import bench_workloads as workloads
+    from easydel_amd import _lib, kernels
+
+    _lib.load()
+    if args.read_probe:
+        return read_probe()
+    if args.read_probe_paged:
+        return read_probe_paged()
+    if args.mfma_probe:
+        return mfma_probe()
+    if args.workload.startswith("mla-"):
+        if args.mla_chunks:
+            _lib.set_tunable("mla_chunks", args.mla_chunks)
+        if args.mla_min_chunk:
+            _lib.set_tunable("mla_min_chunk", args.mla_min_chunk)
+        return bench_mla(args)
+    if args.decode_wgs:
+        _lib.set_tunable("decode_wgs", args.decode_wgs)
+    if args.decode_sync >= 0:
+        _lib.set_tunable("decode_sync", args.decode_sync)
+    if args.decode_dma >= 0:
+        _lib.set_tunable("decode_dma", args.decode_dma)
+    if args.prefill_chunks:
+        _lib.set_tunable("prefill_chunks", args.prefill_chunks)
+    if args.max_splits:
+        _lib.set_tunable("max_splits", args.max_splits)
+    if args.prefill_x32 >= 0:
+        _lib.set_tunable("prefill_x32", args.prefill_x32)
+
+    result = measure(args, args.workload, True)
+    if args.workload == "c2" and args.layout == "interleaved" and not args.no_extra_configs:
+        # the other benchmark configurations, each with its step time and its dominant kernel against its roofline
+        # (no host leg for them); the headline fields above stay those of the decode configuration
+        extra = {}
+        for name in ("c3", "c4-fp8", "c4-int8", "c5-global", "c5-window"):
+            r = measure(args, name, False)
+            roof = r["roofline"]
+            rec = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"], "dtype": r["dtype"],
+                   "kernel": roof["kernel"], "kernel_ms": roof["kernel_ms"],
+                   "roofline": {k: roof[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+                   "traffic_source": roof.get("traffic_source"), "kernels_ms": {k: v["kernel_ms"] for k, v in r["kernels"].items()}}
+            for key in ("algorithmic_bytes_per_launch", "algorithmic_flops_per_launch"):
+                if key in roof:
+                    rec[key.replace("_per_launch", "")] = roof[key]
+            extra[name] = rec
+        result["configs"] = extra
     print(json.dumps(result))
 
 

@@ -13,7 +13,8 @@
 // software-pipelined over three blocks and its order is pinned (a sched_barrier after every MFMA slot):
 //
 //   step b :  MFMA slots 0..15   S(b+2) = K(b+2) Q^T       | vector: softmax of block b+1, half a pair of probabilities per slot
-//             MFMA slots 16..31  O     += V(b)^T P(b)^T     | vector: the softmax goes on; row maxima of S(b+2)
+//             MFMA slots 16..19  row sums of P(b)            |
+//             MFMA slots 20..35  O     += V(b)^T P(b)^T     | vector: the softmax goes on; row maxima of S(b+2)
 //
 // Operands are read four ahead of their MFMAs, across the phase and step boundaries.  The wave has 512 registers; which
 // of them sit in the accumulation file is stated through the operand constraints of the MFMAs (issued as single
@@ -29,8 +30,11 @@
 // Softmax as in attn_prefill_dma_kernel: probabilities are taken against a per-row reference that is only raised when a
 // score exceeds it by more than kMaxSlack (log2 units); here the reference is kept at whole numbers, so that raising it
 // scales what has been accumulated -- and the probabilities of the block still waiting for its PV product -- by a power
-// of two, exactly.  Row sums are taken from the packed 16-bit probabilities (v_dot2), i.e. of exactly the weights the
-// PV product uses.
+// of two, exactly.  Row sums come from the matrix cores (a tile of ones against P^T: four more MFMAs per step), so that
+// they are the sums of the probabilities as rounded to 16 bits, the very weights of the PV product -- a row that one
+// key dominates then comes out exact.  The vector ALU, the busier unit here, could not do it cheaper: the dot-product
+// instruction that adds a packed pair (v_dot2) runs in the matrix pipe and waits for the MFMA in flight (measured: 52
+// instead of 36 cycles per MFMA slot), and unpacking costs four instructions per pair.
 //
 // Tiles that need masking (the window's lower edge, the causal diagonal) and the first and the last two tiles of a key
 // range run through the same two steps written plainly (phases one after the other, flags at run time); the pinned
@@ -50,9 +54,9 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 // write them and ahead of the instructions that read them.
 __device__ __forceinline__ void mfma_settle(f32x16& a, f32x16& b) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a), "+v"(b)); }
 template <int N>
-__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[N]) {
-  static_assert(N == 8, "written out for eight accumulator tiles");
-  asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]));
+__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[N], f32x16 (&l)[2]) {
+  static_assert(N == 8, "written out for eight accumulator tiles and two row-sum tiles");
+  asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]), "+a"(l[0]), "+a"(l[1]));
 }
 
 template <int HT>
@@ -70,10 +74,6 @@ struct Wide16<RPA_BF16> {
   static __device__ __forceinline__ void mfma_o(f32x16& acc, const u32x4& a, const u32x4& b) {
     asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
   }
-  // sum += lo(w) + hi(w), the two bf16 halves of w
-  static __device__ __forceinline__ float add_pair(uint32_t w, float sum) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, w), __builtin_bit_cast(bf16x2_t, 0x3F803F80u), sum, false);
-  }
   static __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float a) {  // both halves times a
     return pack_bf16(__uint_as_float(w << 16) * a, __uint_as_float(w & 0xffff0000u) * a);
   }
@@ -89,9 +89,6 @@ struct Wide16<RPA_F16> {
   }
   static __device__ __forceinline__ void mfma_o(f32x16& acc, const u32x4& a, const u32x4& b) {
     asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ float add_pair(uint32_t w, float sum) {
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, w), __builtin_bit_cast(f16x2, 0x3C003C00u), sum, false);
   }
   static __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float a) {
     const f16x2 v = __builtin_bit_cast(f16x2, w);
@@ -134,10 +131,11 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   constexpr int KN = 4, VN = 4;          // ring slots
   static_assert(KN * HALF <= 65536, "K operand reads address their ring slot through the instruction's 16-bit offset");
   constexpr int NQ = NKK * RB;           // MFMA slots of the score phase
+  constexpr int NSUM = 2 * RB;           // MFMA slots of the row sums (ones x P^T, per row block and 16-key half)
   constexpr int NP = NVO * RB;           // MFMA slots of the PV phase
   constexpr int PD = 4;                  // operands read ahead
   constexpr int NPAIR = RB * 8;          // pairs of probabilities per lane and block
-  static_assert(NQ + NP == 2 * NPAIR && NP == NPAIR, "half a pair of the softmax per MFMA slot, one three-way maximum per PV slot");
+  static_assert(NQ + NP == 2 * NPAIR && NP == NPAIR, "half a pair of the softmax per MFMA slot of the two products, one three-way maximum per PV slot");
   static_assert(NKK >= PD && NVO >= PD, "the operand ring is shorter than either phase");
   static_assert(RB == 2, "mfma_settle names the score tiles of two row blocks");
 
@@ -238,71 +236,89 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   }
 
   // ---- tile loads ------------------------------------------------------------------------------------
-  typedef const __attribute__((address_space(4))) int32_t* ConstI32;
-  ConstI32 bt = (ConstI32)(uintptr_t)(p.block_tables + (int64_t)i * p.M);
-  const char* k_pages = (const char*)p.k_pages;
-  const char* v_pages = (const char*)p.v_pages;
+  // Wave w moves rows [RW w, RW (w + 1)) of a tile's K rows, and again of its V rows, with NLH instructions of RPI rows
+  // each into consecutive 1 KiB blocks of LDS: one m0 per half tile, the instruction offsets u KiB select the block.
+  // (An instruction offset moves the global address as well: it is taken out of the lane offsets beforehand.)
+  constexpr int RW = TT / NW;
+  static_assert(RW == NLH * RPI && RW * RKL == NLH * 1024, "a wave's rows are whole DMA instructions");
+  const char* k_base = (const char*)p.k_pages + (int64_t)h * p.head_stride;
+  const char* v_base = (const char*)p.v_pages + (int64_t)h * p.head_stride;
+  const uint32_t tok_stride = (uint32_t)p.token_stride;  // 64 rows of it fit 31 bits (the host checks)
   const int pg = p.page_size;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds_all;
-  const int dma_row = wave * RPI + lane / CPR;
-  const int dma_chunk = (lane % CPR) ^ swz_key<RKL>(dma_row);
-  const int dma_chunk_v = (lane % CPR) ^ swz_key_v32<RKL>(dma_row);
-  const uint32_t dma_wave_lds = (uint32_t)wave * 1024u;
+  const uint32_t dma_wave_lds = (uint32_t)wave * (uint32_t)(RW * RKL);
+  auto dma_row = [&](int u) -> int { return wave * RW + u * RPI + lane / CPR; };  // row of the tile instruction u of this lane's wave moves
+  auto dma_chunk = [&](int u, bool is_v) -> int { return (lane % CPR) ^ (is_v ? swz_key_v32<RKL>(dma_row(u)) : swz_key<RKL>(dma_row(u))); };
   uint32_t voff_k[NLH], voff_v[NLH];
 #pragma unroll
   for (int u = 0; u < NLH; ++u) {
-    const uint32_t roff = (uint32_t)(dma_row + u * NW * RPI) * (uint32_t)p.token_stride;
-    voff_k[u] = roff + (uint32_t)(dma_chunk << 4);
-    voff_v[u] = roff + (uint32_t)(dma_chunk_v << 4);
+    const uint32_t roff = (uint32_t)dma_row(u) * tok_stride - (uint32_t)(u * 1024);
+    voff_k[u] = roff + (uint32_t)(dma_chunk(u, false) << 4);
+    voff_v[u] = roff + (uint32_t)(dma_chunk(u, true) << 4);
   }
-  auto load_page = [&](int idx) -> int { return __builtin_amdgcn_readfirstlane(bt[min(idx, p.M - 1)]); };
-  // Two cursors walk the tiles of the key range, the K cursor ahead of the V cursor.
-  struct Cursor { int idx, off, tb, slot, page_raw; };
-  Cursor kc, vc;
-  kc.idx = kv_lo / pg; kc.off = kv_lo - kc.idx * pg; kc.tb = kv_lo; kc.slot = 0; kc.page_raw = load_page(kc.idx);
-  vc = kc;
-  auto issue = [&](Cursor& c, bool is_v) __attribute__((always_inline)) {
-    const int page = min(max(c.page_raw, 0), p.P - 1);
-    const int64_t tile_off = (int64_t)page * p.page_stride + (int64_t)c.off * p.token_stride + (int64_t)h * p.head_stride;
-    const char* base = (is_v ? v_pages : k_pages) + tile_off;
-    const bool edge = (c.tb + TT > sp.ctx) || (c.tb < vis_lo);
-    const uint32_t lds = lds_base + (uint32_t)((is_v ? KN : 0) + c.slot) * HALF + dma_wave_lds;
-    if (!edge) {
-#pragma unroll
-      for (int u = 0; u < NLH; ++u) dma16(lds + u * NW * 1024, is_v ? voff_v[u] : voff_k[u], base);
+  // Block-table entries are held 64 columns at a time, one per lane, and picked with v_readlane: the loop then holds no
+  // scalar memory load, whose out-of-order return would turn every wait for an LDS operand into a wait for all of them.
+  const int32_t* bt_row = p.block_tables + (int64_t)i * p.M;
+  int col_base = kv_lo / pg;
+  int pages_vec = bt_row[min(col_base + lane, p.M - 1)];
+  int cur_col = col_base, cur_off = kv_lo - col_base * pg, cur_tb = kv_lo;
+  // Descriptor of the tile the cursor was last at: K of a tile is requested a trip before its V, which reuses it.
+  int64_t tile_off = 0;
+  bool tile_edge = false;
+  int tile_tb = 0;
+  auto next_tile = [&]() __attribute__((always_inline)) {
+    if (cur_col - col_base >= 64) {
+      col_base = cur_col;
+      pages_vec = bt_row[min(col_base + lane, p.M - 1)];
+      asm volatile("" : "+v"(pages_vec));  // waited for here, once in 64 columns, not at the look-up every tile shares
+    }
+    const int page = min(max(__builtin_amdgcn_readlane(pages_vec, cur_col - col_base), 0), p.P - 1);
+    tile_off = (int64_t)page * p.page_stride + (int64_t)((uint32_t)cur_off * tok_stride);
+    tile_edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
+    tile_tb = cur_tb;
+    cur_tb += TT;
+    cur_off += TT;
+    if (cur_off >= pg) {
+      cur_off -= pg;
+      ++cur_col;
+    }
+  };
+  auto issue_half = [&](bool is_v, int slot) __attribute__((always_inline)) {  // K or V rows of the described tile into ring slot `slot`
+    const char* base = (is_v ? v_base : k_base) + tile_off;
+    const uint32_t lds = lds_base + (uint32_t)((is_v ? KN : 0) + slot) * HALF + dma_wave_lds;
+    if (!tile_edge) {
+      dma16_group<NLH>(lds, is_v ? voff_v : voff_k, base);
     } else {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {  // keys nobody may see: any visible row's bytes
-        const int r = min(max(c.tb + dma_row + u * NW * RPI, vis_lo), sp.ctx - 1) - c.tb;
-        const uint32_t roff = (uint32_t)r * (uint32_t)p.token_stride;
-        dma16(lds + u * NW * 1024, roff + (uint32_t)((is_v ? dma_chunk_v : dma_chunk) << 4), base);
+        const int r = min(max(tile_tb + dma_row(u), vis_lo), sp.ctx - 1) - tile_tb;
+        dma16(lds + u * 1024, (uint32_t)r * tok_stride + (uint32_t)(dma_chunk(u, is_v) << 4), base);
       }
     }
-    c.tb += TT;
-    c.off += TT;
-    if (c.off >= pg) {
-      c.off -= pg;
-      ++c.idx;
-    }
-    c.slot = (c.slot + 1) & 3;
-    c.page_raw = load_page(c.idx);
   };
-  int k_issued = 0, v_issued = 0;  // tiles whose K / V rows have been requested
-  auto issue_k = [&]() __attribute__((always_inline)) { if (k_issued < n_tiles) { issue(kc, false); ++k_issued; } };
-  auto issue_v = [&]() __attribute__((always_inline)) { if (v_issued < n_tiles) { issue(vc, true); ++v_issued; } };
+  // K(i) goes to K slot i % 4, V(i) to V slot i % 4
+  auto issue_k = [&](int tile) __attribute__((always_inline)) { if (tile < n_tiles) { next_tile(); issue_half(false, tile & 3); } };
+  auto issue_v = [&](int tile) __attribute__((always_inline)) { if (tile < n_tiles) issue_half(true, tile & 3); };
 
   // ---- registers of the pipeline -------------------------------------------------------------------------
   // Block b of the key range = (tile b / 2, half b % 2).  Scores and probabilities of block b live in buffer b % 2.
   f32x16 sa[2][RB];            // raw scores S^T: lane = row j32, register r = key 8 (r / 4) + 4 hh + r % 4 of the block
   u32x4 pb[2][RB][2];          // packed probabilities, as the two B operands (16 keys each) of the PV product
   f32x16 o_acc[RB][DB];        // O^T: lane = row j32, register r = dim 8 (r / 4) + 4 hh + r % 4 of the 32-dim block
-  float m_ref[RB], m_neg[RB], l_run[RB], lmx[RB];
+  f32x16 l_acc[RB];            // row sums, from the matrix cores: every register of lane j32 holds the sum of row j32
+  float m_ref[RB], m_neg[RB], lmx[RB];
   u32x4 ops[PD];               // operands read ahead of their MFMAs
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     m_ref[rb] = -INFINITY;
     m_neg[rb] = 0.f;
-    l_run[rb] = 0.f;
+    {
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      asm volatile("" : "+a"(z));
+      l_acc[rb] = z;
+    }
     lmx[rb] = -INFINITY;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
@@ -314,6 +330,11 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     }
   }
   const float sc_mul = p.scale_log2;
+  // The A operand of the row sums: ones, written to registers once, here.  (Left to the compiler it is rebuilt from
+  // scalar registers right in front of the MFMA that reads it, and an MFMA issued through an assembly statement gets
+  // no pause behind a vector instruction that writes one of its operands: it read the old register contents.)
+  u32x4 ones = {H::kOnes, H::kOnes, H::kOnes, H::kOnes};
+  asm volatile("" : "+v"(ones));
 
   // Lane addresses of the operand reads, relative to a ring slot.  K operand kk of a block: key j32 of the block, chunk 2 kk + hh.
   uint32_t kaddr[NKK];
@@ -350,7 +371,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) grow |= lmx[rb] * sc_mul > m_ref[rb] + kMaxSlack;
     if (__any(grow)) {
-      mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc);  // the accumulators may still be on their way
+      mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);  // the accumulators may still be on their way
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const float mx = xor32_max(lmx[rb]) * sc_mul;
@@ -359,7 +380,11 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         m_ref[rb] = m_new;
         m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
         asm volatile("s_nop 1" : "+v"(alpha));
-        l_run[rb] *= alpha;
+        {
+          f32x16 l = l_acc[rb];
+          l[0] *= alpha;  // the register the epilogue reads; the others hold the same sum and are never read
+          l_acc[rb] = l;
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           f32x16 o = o_acc[rb][db];
@@ -400,32 +425,40 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) mx_part[rb] = -INFINITY;
 #pragma unroll
-    for (int k = 0; k < NQ + NP; ++k) {
-      // -- the MFMA of the slot and, behind an operand's last MFMA, the read of the operand PD further on
-      const int g = k / RB, rb = k % RB;  // operand of the step (K operands, then V operands), row block
+    for (int k = 0; k < NQ + NSUM + NP; ++k) {
+      // -- the MFMA of the slot: scores, then the row sums of block b (a V^T tile of ones against P^T leaves, in every
+      //    accumulator register of lane j32, the sum of row j32's probabilities as rounded to 16 bits: exactly the weights
+      //    the PV product uses), then the PV product; behind an operand's last MFMA, the read of the operand PD further on
       if (k < NQ) {
+        const int g = k / RB, rb = k % RB;
         if (g == 0) W::mfma_s0(s_nxt[rb], ops[g % PD], qf[rb][g]);
         else W::mfma_s(s_nxt[rb], ops[g % PD], qf[rb][g]);
+        if (rb == RB - 1) {
+          const int nx = g + PD;
+          if (nx < NKK) ops[g % PD] = rk(ka[nx]);
+          else ops[g % PD] = rv(nx - NKK);
+        }
+      } else if (k < NQ + NSUM) {
+        const int e = k - NQ, rb = e % RB, sh = e / RB;
+        W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
       } else {
-        const int v = g - NKK, db = v / 2, s = v % 2;
-        W::mfma_o(o_acc[rb][db], ops[g % PD], p_cur[rb][s]);
+        const int kk2 = k - NQ - NSUM, v = kk2 / RB, rb = kk2 % RB, db = v / 2, sh = v % 2, g = NKK + v;
+        W::mfma_o(o_acc[rb][db], ops[g % PD], p_cur[rb][sh]);
+        if (rb == RB - 1) {
+          const int nx = g + PD;
+          if (nx < NKK + NVO) ops[g % PD] = rv(nx - NKK);
+          else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
+        }
       }
-      if (rb == RB - 1) {
-        const int nx = g + PD;
-        if (nx < NKK) ops[g % PD] = rk(ka[nx]);
-        else if (nx < NKK + NVO) ops[g % PD] = rv(nx - NKK);
-        else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
-      }
-      // -- the softmax of block b+1: pair i = k / 2 = (row block, register pair); first half on even slots (the scaled
-      //    differences of pair i, and pair i-1 packed and summed), second half on odd slots (the exponentials)
-      {
-        const int ip = k / 2;
-        if ((k & 1) == 0) {
+      // -- the softmax of block b+1, on the slots of the two products: pair i = (row block, register pair); first half
+      //    on even slots (the scaled differences of pair i, and pair i-1 packed), second half on odd slots (exponentials)
+      if (k < NQ || k >= NQ + NSUM) {
+        const int ks = k < NQ ? k : k - NSUM;
+        const int ip = ks / 2;
+        if ((ks & 1) == 0) {
           if (ip > 0) {
             const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;
-            const uint32_t pk = H::pack(ea, eb);
-            p_nxt[prb][pr2 / 4][pr2 % 4] = pk;
-            l_run[prb] = W::add_pair(pk, l_run[prb]);
+            p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
           }
           const int srb = ip / 8, sr2 = ip % 8;
           xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
@@ -435,18 +468,16 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           eb = __builtin_amdgcn_exp2f(xb);
         }
       }
-      // -- row maxima of S(b+2), whose MFMAs lie at least sixteen slots back: one three-way maximum per PV slot
-      if (k >= NQ) {
-        const int e = k - NQ, mrb = e / 8, mr2 = e % 8;
+      // -- row maxima of S(b+2), whose MFMAs lie at least five slots back: one three-way maximum per PV slot
+      if (k >= NQ + NSUM) {
+        const int e = k - NQ - NSUM, mrb = e / 8, mr2 = e % 8;
         mx_part[mrb] = __builtin_fmaxf(__builtin_fmaxf(mx_part[mrb], s_nxt[mrb][2 * mr2]), s_nxt[mrb][2 * mr2 + 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     {  // the last pair
       constexpr int jp = NPAIR - 1, prb = jp / 8, pr2 = jp % 8;
-      const uint32_t pk = H::pack(ea, eb);
-      p_nxt[prb][pr2 / 4][pr2 % 4] = pk;
-      l_run[prb] = W::add_pair(pk, l_run[prb]);
+      p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
     }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) lmx[rb] = mx_part[rb];
@@ -494,15 +525,17 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         for (int r2 = 0; r2 < 8; ++r2) {
           const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[rb][2 * r2], sc_mul, m_neg[rb]));
           const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[rb][2 * r2 + 1], sc_mul, m_neg[rb]));
-          const uint32_t pk = H::pack(e0, e1);
-          p_nxt[rb][r2 / 4][r2 % 4] = pk;
-          l_run[rb] = W::add_pair(pk, l_run[rb]);
+          p_nxt[rb][r2 / 4][r2 % 4] = H::pack(e0, e1);
         }
     }
     if (do_pv) {
-      u32x4 vo[PD];
+      u32x4 (&vo)[PD] = ops;  // the K operands read ahead for the next step are read at the end of this one
 #pragma unroll
       for (int o = 0; o < PD; ++o) vo[o] = rv(o);
+#pragma unroll
+      for (int sh = 0; sh < 2; ++sh)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);  // row sums of block b
 #pragma unroll
       for (int g = 0; g < NVO; ++g) {
         const int db = g / 2, s = g % 2;
@@ -544,11 +577,11 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // Trip tt (tt = -1 .. n_tiles - 1) is the two steps b = 2 tt, 2 tt + 1: scores of tile tt+1, PV products of tile tt.
   // It starts at a barrier behind which K(tt+2) and V(tt) are visible and the slots of K(tt) and V(tt-1) are free:
   // V(tt+3) and K(tt+4) are requested into them.  Requests so far, in order: K0 V0 K1 V1 K2 | V2 K3 | V3 K4 | ...
-  issue_k();
-  issue_v();
-  issue_k();
-  issue_v();
-  issue_k();
+  issue_k(0);
+  issue_v(0);
+  issue_k(1);
+  issue_v(1);
+  issue_k(2);
   // trips the pinned code may serve: tt >= 0, tile tt+2 exists, tile tt+1 unmasked for the whole wave
   const int tt_fast_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT - 1);
   const int tt_fast_hi = max(tt_fast_lo, min(n_tiles - 2, (wave_hi - kv_lo) / TT - 1));  // first trip behind them
@@ -559,8 +592,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     if (vin + kin == 2) wait_loads_and_barrier<2 * NLH>();
     else if (vin + kin == 1) wait_loads_and_barrier<NLH>();
     else wait_loads_and_barrier<0>();
-    issue_v();
-    issue_k();
+    issue_v(tt + 3);
+    issue_k(tt + 4);
   };
   auto slow_trip = [&](int tt) __attribute__((always_inline)) {
     trip_head(tt);
@@ -585,6 +618,16 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   };
   int tt = -1;
   for (; tt < tt_fast_lo; ++tt) slow_trip(tt);
+  // What the pinned loop reads but never writes is touched once here: should the compiler have parked any of it in
+  // memory across the code above, its wait for the reload lands here and not inside the loop, where a wait on the
+  // vector-memory counter would also wait for the tiles in flight.
+#pragma unroll
+  for (int kk = 0; kk < NKK; ++kk) asm volatile("" : "+v"(kaddr[kk]));
+#pragma unroll
+  for (int db = 0; db < DB; ++db) asm volatile("" : "+v"(vaddr[db]));
+#pragma unroll
+  for (int u = 0; u < NLH; ++u) asm volatile("" : "+v"(voff_k[u]), "+v"(voff_v[u]));
+  asm volatile("" : "+v"(pages_vec));
   for (; tt < tt_fast_hi; ++tt) {
     trip_head(tt);
     // lane addresses of this trip's operands: K of tile tt+1, the first K operands of tile tt+2, V of tile tt
@@ -613,10 +656,10 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   for (; tt < n_tiles; ++tt) slow_trip(tt);
 
   // ---- epilogue -----------------------------------------------------------------------------------------
-  mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc);
+  mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const float l_tot = l_run[rb] + __shfl_xor(l_run[rb], 32);
+    const float l_tot = l_acc[rb][0];
     if (row_ok[rb]) {
       if (single) {
         const float l_fin = with_sink(p, out_head[rb], m_ref[rb], l_tot);

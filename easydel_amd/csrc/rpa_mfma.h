@@ -132,6 +132,23 @@ __device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const vo
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
+// N such DMAs of one wave into consecutive 1 KiB blocks of LDS starting at lds_addr: m0 is set once and the instruction
+// offsets u * 1024 select the block.  The offset is added to the global address as well, so the caller's lane offset
+// voff[u] must already have u * 1024 taken out of it.
+template <int N>
+__device__ __forceinline__ void dma16_group(uint32_t lds_addr, const uint32_t (&voff)[N], const void* base) {
+  static_assert(N == 1 || N == 2 || N == 4, "one, two or four instructions per group");
+  if constexpr (N == 4)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %5\n\tglobal_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\tglobal_load_lds_dwordx4 %4, %5 offset:3072"
+                 ::"s"(lds_addr), "v"(voff[0]), "v"(voff[1]), "v"(voff[2]), "v"(voff[3]), "s"(base) : "memory");
+  else if constexpr (N == 2)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %3\n\tglobal_load_lds_dwordx4 %2, %3 offset:1024"
+                 ::"s"(lds_addr), "v"(voff[0]), "v"(voff[1]), "s"(base) : "memory");
+  else
+    dma16(lds_addr, voff[0], base);
+}
+
 // ... with the non-temporal hint, for data no wave will ask for again (the pages a decode kernel streams): kept out
 // of the caches' longer-lived lines, such a stream reads HBM measurably faster.
 __device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const void* base) {
