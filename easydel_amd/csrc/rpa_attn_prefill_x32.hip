@@ -138,6 +138,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   static_assert(NQ + NP == 2 * NPAIR && NP == NPAIR, "half a pair of the softmax per MFMA slot of the two products, one three-way maximum per PV slot");
   static_assert(NKK >= PD && NVO >= PD, "the operand ring is shorter than either phase");
   static_assert(RB == 2, "mfma_settle names the score tiles of two row blocks");
+  static_assert(NLH <= NSUM, "a step requests its half tile from the slots of the row sums");
 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_all[(KN + VN) * HALF];
 
@@ -307,10 +308,12 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   f32x16 o_acc[RB][DB];        // O^T: lane = row j32, register r = dim 8 (r / 4) + 4 hh + r % 4 of the 32-dim block
   f32x16 l_acc[RB];            // row sums, from the matrix cores: every register of lane j32 holds the sum of row j32
   float m_ref[RB], m_neg[RB], lmx[RB];
+  float thr[RB];               // (m_ref + slack) in units of the raw scores: what a block's maximum is compared with
   u32x4 ops[PD];               // operands read ahead of their MFMAs
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     m_ref[rb] = -INFINITY;
+    thr[rb] = -INFINITY;
     m_neg[rb] = 0.f;
     {
       f32x16 z;
@@ -330,6 +333,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     }
   }
   const float sc_mul = p.scale_log2;
+  const float inv_sc = 1.f / sc_mul;
   // The A operand of the row sums: ones, written to registers once, here.  (Left to the compiler it is rebuilt from
   // scalar registers right in front of the MFMA that reads it, and an MFMA issued through an assembly statement gets
   // no pause behind a vector instruction that writes one of its operands: it read the old register contents.)
@@ -369,7 +373,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   auto check = [&](u32x4 (&pend)[RB][2], bool has_pending) __attribute__((always_inline)) {
     bool grow = false;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) grow |= lmx[rb] * sc_mul > m_ref[rb] + kMaxSlack;
+    for (int rb = 0; rb < RB; ++rb) grow |= lmx[rb] > thr[rb];
     if (__any(grow)) {
       mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);  // the accumulators may still be on their way
 #pragma unroll
@@ -378,6 +382,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         const float m_new = fmaxf(m_ref[rb], ceilf(mx));
         float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref[rb] - m_new);  // a power of two, or 0
         m_ref[rb] = m_new;
+        thr[rb] = (m_new + kMaxSlack) * inv_sc;
         m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
         asm volatile("s_nop 1" : "+v"(alpha));
         {
@@ -406,7 +411,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // PAR = (b + 1) % 2: the buffer of block b+1 (the other receives block b+2 and held block b).  ka: lane addresses of
   // the K operands of block b+2; kn: of the first PD operands of block b+3 (read at the end); va: lane addresses of the V
   // operands of block b.
-  auto fast_step = [&](auto par_tag, const uint32_t (&ka)[NKK], const uint32_t (&kn)[PD], const uint32_t (&va)[DB]) __attribute__((always_inline)) {
+  auto fast_step = [&](auto par_tag, const uint32_t (&ka)[NKK], const uint32_t (&kn)[PD], const uint32_t (&va)[DB], uint32_t dma_lds,
+                       const uint32_t (&dma_voff)[NLH], const char* dma_base) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;
     f32x16 (&s_cur)[RB] = sa[PAR];              // S(b+1), consumed by the softmax
     f32x16 (&s_nxt)[RB] = sa[PAR ^ 1];          // S(b+2), produced
@@ -431,6 +437,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       //    the PV product uses), then the PV product; behind an operand's last MFMA, the read of the operand PD further on
       if (k < NQ) {
         const int g = k / RB, rb = k % RB;
+        if (rb == 0 && g % 2 == 0) asm volatile("" ::"v"(ops[g % PD]), "v"(ops[(g + 1) % PD]));  // one wait for two operands
         if (g == 0) W::mfma_s0(s_nxt[rb], ops[g % PD], qf[rb][g]);
         else W::mfma_s(s_nxt[rb], ops[g % PD], qf[rb][g]);
         if (rb == RB - 1) {
@@ -441,8 +448,12 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       } else if (k < NQ + NSUM) {
         const int e = k - NQ, rb = e % RB, sh = e / RB;
         W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
+        // These slots carry no softmax and no operand read: the step's share of the tile loads is requested here (half
+        // a tile: NLH instructions), where the time the load unit takes to accept 1 KiB of addresses hides behind an MFMA.
+        if (e < NLH) dma16_at(dma_lds, e, dma_voff[e], dma_base);
       } else {
         const int kk2 = k - NQ - NSUM, v = kk2 / RB, rb = kk2 % RB, db = v / 2, sh = v % 2, g = NKK + v;
+        if (rb == 0 && g % 2 == 0) asm volatile("" ::"v"(ops[g % PD]), "v"(ops[(g + 1) % PD]));
         W::mfma_o(o_acc[rb][db], ops[g % PD], p_cur[rb][sh]);
         if (rb == RB - 1) {
           const int nx = g + PD;
@@ -456,13 +467,13 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         const int ks = k < NQ ? k : k - NSUM;
         const int ip = ks / 2;
         if ((ks & 1) == 0) {
-          if (ip > 0) {
-            const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;
-            p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
-          }
           const int srb = ip / 8, sr2 = ip % 8;
           xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
           xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc_mul, m_neg[srb]);
+          if (ip > 0) {  // behind the two multiply-adds: they are the distance an exponential wants from its reader
+            const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;
+            p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
+          }
         } else {
           ea = __builtin_amdgcn_exp2f(xa);
           eb = __builtin_amdgcn_exp2f(xb);
@@ -584,7 +595,10 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   issue_k(2);
   // trips the pinned code may serve: tt >= 0, tile tt+2 exists, tile tt+1 unmasked for the whole wave
   const int tt_fast_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT - 1);
-  const int tt_fast_hi = max(tt_fast_lo, min(n_tiles - 2, (wave_hi - kv_lo) / TT - 1));  // first trip behind them
+  // ... and tile tt+4 exists and lies wholly inside the context: the pinned steps request V(tt+3) and K(tt+4) themselves,
+  // with plain lane offsets
+  const int n_whole = min(n_tiles, (sp.ctx - kv_lo) / TT);  // tiles without a row past the context
+  const int tt_fast_hi = max(tt_fast_lo, min(n_whole - 4, (wave_hi - kv_lo) / TT - 1));  // first trip behind them
   const int n_blocks = 2 * n_tiles;
   auto trip_head = [&](int tt) __attribute__((always_inline)) {
     // in flight may stay what the previous trip requested: V(tt+2) and K(tt+3)
@@ -629,7 +643,14 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   for (int u = 0; u < NLH; ++u) asm volatile("" : "+v"(voff_k[u]), "+v"(voff_v[u]));
   asm volatile("" : "+v"(pages_vec));
   for (; tt < tt_fast_hi; ++tt) {
-    trip_head(tt);
+    // tiles up to K(tt+2) and V(tt) have landed; in flight stay the requests of the trip before, V(tt+2) and K(tt+3)
+    wait_loads_and_barrier<2 * NLH>();
+    // this trip requests V(tt+3), from inside its first step, and K(tt+4), from inside its second
+    const char* v_ptr = v_base + tile_off;  // tile tt+3: described when its K rows were requested
+    next_tile();
+    const char* k_ptr = k_base + tile_off;  // tile tt+4
+    const uint32_t v_lds = lds_base + (uint32_t)(KN + ((tt + 3) & 3)) * HALF + dma_wave_lds;
+    const uint32_t k_lds = lds_base + (uint32_t)((tt + 4) & 3) * HALF + dma_wave_lds;
     // lane addresses of this trip's operands: K of tile tt+1, the first K operands of tile tt+2, V of tile tt
     const uint32_t k_off = (uint32_t)(((tt + 1) & 3) * HALF), kn_off = (uint32_t)(((tt + 2) & 3) * HALF), v_off = (uint32_t)((tt & 3) * HALF);
     uint32_t ka0[NKK], ka1[NKK], kn0[PD], kn1[PD], va0[DB], va1[DB];
@@ -649,9 +670,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       va1[db] = va0[db] + BK * RKL;
     }
     check(pb[0], true);
-    fast_step(std::integral_constant<int, 1>{}, ka0, kn0, va0);
+    fast_step(std::integral_constant<int, 1>{}, ka0, kn0, va0, v_lds, voff_v, v_ptr);
     check(pb[1], true);
-    fast_step(std::integral_constant<int, 0>{}, ka1, kn1, va1);
+    fast_step(std::integral_constant<int, 0>{}, ka1, kn1, va1, k_lds, voff_k, k_ptr);
   }
   for (; tt < n_tiles; ++tt) slow_trip(tt);
 

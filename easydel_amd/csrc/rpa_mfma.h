@@ -149,6 +149,14 @@ __device__ __forceinline__ void dma16_group(uint32_t lds_addr, const uint32_t (&
     dma16(lds_addr, voff[0], base);
 }
 
+// Instruction u of such a group on its own (u < 4): m0 is set again, the instruction offset u * 1024 selects the block.
+__device__ __forceinline__ void dma16_at(uint32_t lds_addr, int u, uint32_t voff, const void* base) {
+  if (u == 0) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+  else if (u == 1) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+  else if (u == 2) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:2048" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+  else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:3072" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
 // ... with the non-temporal hint, for data no wave will ask for again (the pages a decode kernel streams): kept out
 // of the caches' longer-lived lines, such a stream reads HBM measurably faster.
 __device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const void* base) {
