@@ -390,6 +390,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
   p.decode_sync = tun.decode_sync;
   p.prefill_dma = tun.prefill_dma;
   p.pre_rows = rpa::kPrefillRows;
+  p.pre_x32 = 0;
   p.decode_pace = tun.decode_pace;
   p.decode_dma = tun.decode_dma < 0 ? ((p.D == 256 || p.kv_dtype == RPA_INT8) ? 1 : 0) : tun.decode_dma;
   p.max_splits = 2;
@@ -440,8 +441,9 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     p.pre_max_chunks = pre_chunks;
     p.pre_auto = tun.prefill_chunks <= 0 ? 1 : 0;
     p.pre_slots = device_cus() * (Dc <= 128 ? 2 : 1);  // resident workgroups of the large-row kernels
-    if (tun.prefill_dma && tun.prefill_x32 && rpa::prefill_x32_supported(p)) {  // 256-row workgroups, one per CU
-      p.pre_rows = 256;
+    if (tun.prefill_dma && tun.prefill_x32 && rpa::prefill_x32_rows(p) > 0) {  // one workgroup per CU
+      p.pre_x32 = 1;
+      p.pre_rows = rpa::prefill_x32_rows(p);
       p.pre_slots = device_cus();
     }
     char* base = (char*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);

@@ -361,7 +361,7 @@ static int launch_kvt(hipStream_t stream, const AttnParams& p) {
 bool prefill_supported(const AttnParams& p) { return decode_supported(p); }
 
 int launch_attn_prefill(hipStream_t stream, const AttnParams& p) {
-  if (p.pre_rows == 256) return launch_attn_prefill_x32(stream, p);  // chosen by the caller together with the row-tile height
+  if (p.pre_x32) return launch_attn_prefill_x32(stream, p);  // chosen by the caller together with the row-tile height
   if (p.prefill_dma && prefill_dma_supported(p)) return launch_attn_prefill_dma(stream, p);
   if (p.prefill_dma && prefill_dma8_supported(p)) return launch_attn_prefill_dma8(stream, p);
   switch (p.kv_dtype) {

@@ -24,8 +24,11 @@
 // pinned step the first reader of a result comes at least sixteen MFMA slots behind its writer, everywhere else an
 // explicit pause (mfma_settle) precedes the reader.
 //
-// Tiles of 64 keys travel global -> LDS through the load unit (global_load_lds_dwordx4), K four tiles and V three
-// tiles ahead, in rings of four slots each (128 KiB at head size 128); one barrier per tile, i.e. per two steps.
+// Tiles travel global -> LDS through the load unit (global_load_lds_dwordx4) into one ring for K and one for V.  At head
+// size 128 a tile is 64 keys (two steps), the rings hold four tiles each (128 KiB), K is requested four tiles and V three
+// tiles ahead, and there is one barrier per tile.  At head size 256 a wave owns 32 rows (the O^T tile of 64 rows would
+// not fit its registers), a tile is one block of 32 keys, the rings hold five tiles each (160 KiB: all of the CU's LDS),
+// K is requested six and V four tiles ahead, and there is one barrier per step.
 //
 // Softmax as in attn_prefill_dma_kernel: probabilities are taken against a per-row reference that is only raised when a
 // score exceeds it by more than kMaxSlack (log2 units); here the reference is kept at whole numbers, so that raising it
@@ -52,11 +55,13 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 // compiler cannot place it): 32 wait states, more than the eight passes of a 32x32x16 MFMA plus the margin this chip asks for.
 // The registers whose readers it protects are operands of the statement: that is what orders it behind the MFMAs that
 // write them and ahead of the instructions that read them.
-__device__ __forceinline__ void mfma_settle(f32x16& a, f32x16& b) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(a), "+v"(b)); }
-template <int N>
-__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[N], f32x16 (&l)[2]) {
-  static_assert(N == 8, "written out for eight accumulator tiles and two row-sum tiles");
+__device__ __forceinline__ void mfma_settle(f32x16 (&s)[2]) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s[0]), "+v"(s[1])); }
+__device__ __forceinline__ void mfma_settle(f32x16 (&s)[1]) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(s[0])); }
+__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[8], f32x16 (&l)[2]) {
   asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]), "+a"(l[0]), "+a"(l[1]));
+}
+__device__ __forceinline__ void mfma_settle_acc(f32x16 (&o)[8], f32x16 (&l)[1]) {
+  asm volatile("s_nop 15\n\ts_nop 15" : "+a"(o[0]), "+a"(o[1]), "+a"(o[2]), "+a"(o[3]), "+a"(o[4]), "+a"(o[5]), "+a"(o[6]), "+a"(o[7]), "+a"(l[0]));
 }
 
 template <int HT>
@@ -107,40 +112,50 @@ __device__ __forceinline__ int swz_key_v32(int tok) {
   else return 0;
 }
 
-constexpr int kWideRows = 256;  // query rows one workgroup of this kernel owns
-
-template <int D, int NW, int RB, int HT>
+template <int D, int NW, int RB, int HT, bool CAP>
 __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p) {
   using H = Half16<HT>;
   using W = Wide16<HT>;
-  constexpr int TT = 64;                 // keys per tile (what a barrier and a set of loads cover)
   constexpr int BK = 32;                 // keys per block (what a step computes)
+  constexpr int SPT = D <= 128 ? 2 : 1;  // steps per tile
+  constexpr int TT = BK * SPT;           // keys per tile (what a barrier and a set of loads cover)
   constexpr int RKL = D * 2;             // bytes of one K (or V) row
   constexpr int CPR = RKL / 16;          // 16-byte chunks per row
   constexpr int RPI = 64 / CPR;          // rows one DMA instruction covers
   constexpr int NLH = TT / (RPI * NW);   // DMA instructions per wave per tile, for K and again for V
   static_assert(TT % (RPI * NW) == 0 && NLH >= 1, "the waves' DMA instructions tile the rows exactly");
-  static_assert(NLH == 1 || (RPI * NW) % 16 == 0, "a lane's swizzle key must not depend on the instruction");
   constexpr int NKK = D / 16;            // k-steps of the score MFMA = K operands per block
   constexpr int DB = D / 32;             // 32-dim blocks of O^T
   constexpr int NVO = DB * 2;            // V operands per block: (dim block, 16-key half)
   constexpr int ROWS = NW * RB * 32;
-  static_assert(ROWS == kWideRows, "the plan and merge kernels are told this row-tile height");
   constexpr float kMaxSlack = 8.f;
   constexpr int HALF = TT * RKL;         // bytes of the K (or V) rows of one tile
-  constexpr int KN = 4, VN = 4;          // ring slots
-  static_assert(KN * HALF <= 65536, "K operand reads address their ring slot through the instruction's 16-bit offset");
+  constexpr int KN = SPT == 2 ? 4 : 5;   // ring slots (tiles), of K and again of V
+  // The barrier with index u stands in front of step SPT u.  Behind it K tiles up to u + KNO are visible (the steps up to
+  // the next barrier read as far as the first operands of block SPT u + SPT + 2) and V tiles up to u; K tiles below
+  // u + 2 / SPT and V tiles below u will not be read again.  It requests the tiles that take the newest free slots:
+  constexpr int KNO = (SPT + 2) / SPT;
+  constexpr int KAH = 2 / SPT - 1 + KN;  // K of tile u + KAH ...
+  constexpr int VAH = KN - 1;            // ... behind V of tile u + VAH
+  constexpr int DQ = KAH - VAH;          // a tile's V rows are requested this many tiles behind its K rows
+  constexpr int FLYB = KAH - KNO - 1;    // all requests of this many barriers may still be in flight at a barrier
+  constexpr int U0 = -2 / SPT;           // the first barrier (step -2)
+  static_assert(2 * KN * HALF <= 160 * 1024 && FLYB >= 1 && DQ >= 1 && 2 * FLYB * NLH <= 48, "ring sizes");
   constexpr int NQ = NKK * RB;           // MFMA slots of the score phase
   constexpr int NSUM = 2 * RB;           // MFMA slots of the row sums (ones x P^T, per row block and 16-key half)
   constexpr int NP = NVO * RB;           // MFMA slots of the PV phase
   constexpr int PD = 4;                  // operands read ahead
   constexpr int NPAIR = RB * 8;          // pairs of probabilities per lane and block
-  static_assert(NQ + NP == 2 * NPAIR && NP == NPAIR, "half a pair of the softmax per MFMA slot of the two products, one three-way maximum per PV slot");
+  constexpr int SPP = (NQ + NP) / NPAIR; // MFMA slots of the two products per pair of the softmax
+  constexpr int MSP = NP / NPAIR;        // PV slots per three-way maximum
+  static_assert(SPP * NPAIR == NQ + NP && MSP * NPAIR == NP && (SPP == 2 || SPP == 4), "the softmax is dealt out over the MFMA slots of the two products");
+  static_assert(!CAP || SPP == 4, "the soft cap's stages take four slots per pair");
   static_assert(NKK >= PD && NVO >= PD, "the operand ring is shorter than either phase");
-  static_assert(RB == 2, "mfma_settle names the score tiles of two row blocks");
-  static_assert(NLH <= NSUM, "a step requests its half tile from the slots of the row sums");
+  constexpr int NG = SPT == 2 ? 1 : 2;   // half tiles a step requests: at two steps per tile V in the first, K in the second
+  constexpr int NDI = NG * NLH;          // DMA instructions of a step: in the slots of the row sums, then every other PV slot
+  static_assert(NDI <= NSUM + NP / 2, "slots for the step's DMA instructions");
 
-  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[(KN + VN) * HALF];
+  __shared__ __attribute__((aligned(1024))) unsigned char lds_all[2 * KN * HALF];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -182,7 +197,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   if (chunk >= pt.n_chunks) return;
   const int base_pos = sp.ctx - sp.q_len;
   const int vis_lo = pt.vis_lo;
-  const int kv_lo = max(pt.kv_lo + chunk * pt.chunk_len, vis_lo & ~(TT - 1));
+  const int kv_lo = max(pt.kv_lo + chunk * pt.chunk_len, vis_lo & ~63);
   const int kv_hi = (chunk == pt.n_chunks - 1) ? pt.kv_hi : pt.kv_lo + (chunk + 1) * pt.chunk_len;
   const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
   const bool single = pt.n_chunks == 1;
@@ -263,20 +278,31 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   int col_base = kv_lo / pg;
   int pages_vec = bt_row[min(col_base + lane, p.M - 1)];
   int cur_col = col_base, cur_off = kv_lo - col_base * pg, cur_tb = kv_lo;
-  // Descriptor of the tile the cursor was last at: K of a tile is requested a trip before its V, which reuses it.
-  int64_t tile_off = 0;
-  bool tile_edge = false;
-  int tile_tb = 0;
-  auto next_tile = [&]() __attribute__((always_inline)) {
-    if (cur_col - col_base >= 64) {
+  // Descriptors of the tiles the cursor was last at, newest first: a tile's V rows are requested DQ tiles behind its K rows.
+  struct TileDesc {
+    int64_t off;
+    bool edge;
+    int tb;
+  };
+  TileDesc td[DQ];
+#pragma unroll
+  for (int j = 0; j < DQ; ++j) td[j] = TileDesc{0, false, 0};
+  // The next 64 columns are fetched when the cursor is within `margin` columns of the end of the held ones.
+  auto refill_pages = [&](int margin) __attribute__((always_inline)) {
+    if (cur_col - col_base >= 64 - margin) {
       col_base = cur_col;
       pages_vec = bt_row[min(col_base + lane, p.M - 1)];
       asm volatile("" : "+v"(pages_vec));  // waited for here, once in 64 columns, not at the look-up every tile shares
     }
+  };
+  auto next_tile = [&](bool refill = true) __attribute__((always_inline)) {  // (also for tiles past the range: the cursor then only counts)
+    if (refill) refill_pages(0);
     const int page = min(max(__builtin_amdgcn_readlane(pages_vec, cur_col - col_base), 0), p.P - 1);
-    tile_off = (int64_t)page * p.page_stride + (int64_t)((uint32_t)cur_off * tok_stride);
-    tile_edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
-    tile_tb = cur_tb;
+#pragma unroll
+    for (int j = DQ - 1; j > 0; --j) td[j] = td[j - 1];
+    td[0].off = (int64_t)page * p.page_stride + (int64_t)((uint32_t)cur_off * tok_stride);
+    td[0].edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
+    td[0].tb = cur_tb;
     cur_tb += TT;
     cur_off += TT;
     if (cur_off >= pg) {
@@ -284,30 +310,28 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       ++cur_col;
     }
   };
-  auto issue_half = [&](bool is_v, int slot) __attribute__((always_inline)) {  // K or V rows of the described tile into ring slot `slot`
-    const char* base = (is_v ? v_base : k_base) + tile_off;
+  auto issue_half = [&](bool is_v, int slot, const TileDesc& t) __attribute__((always_inline)) {  // K or V rows of tile t into ring slot `slot`
+    const char* base = (is_v ? v_base : k_base) + t.off;
     const uint32_t lds = lds_base + (uint32_t)((is_v ? KN : 0) + slot) * HALF + dma_wave_lds;
-    if (!tile_edge) {
+    if (!t.edge) {
       dma16_group<NLH>(lds, is_v ? voff_v : voff_k, base);
     } else {
 #pragma unroll
       for (int u = 0; u < NLH; ++u) {  // keys nobody may see: any visible row's bytes
-        const int r = min(max(tile_tb + dma_row(u), vis_lo), sp.ctx - 1) - tile_tb;
+        const int r = min(max(t.tb + dma_row(u), vis_lo), sp.ctx - 1) - t.tb;
         dma16(lds + u * 1024, (uint32_t)r * tok_stride + (uint32_t)(dma_chunk(u, is_v) << 4), base);
       }
     }
   };
-  // K(i) goes to K slot i % 4, V(i) to V slot i % 4
-  auto issue_k = [&](int tile) __attribute__((always_inline)) { if (tile < n_tiles) { next_tile(); issue_half(false, tile & 3); } };
-  auto issue_v = [&](int tile) __attribute__((always_inline)) { if (tile < n_tiles) issue_half(true, tile & 3); };
 
   // ---- registers of the pipeline -------------------------------------------------------------------------
-  // Block b of the key range = (tile b / 2, half b % 2).  Scores and probabilities of block b live in buffer b % 2.
+  // Block b of the key range = (tile b / SPT, part b % SPT).  Scores and probabilities of block b live in buffer b % 2.
   f32x16 sa[2][RB];            // raw scores S^T: lane = row j32, register r = key 8 (r / 4) + 4 hh + r % 4 of the block
   u32x4 pb[2][RB][2];          // packed probabilities, as the two B operands (16 keys each) of the PV product
   f32x16 o_acc[RB][DB];        // O^T: lane = row j32, register r = dim 8 (r / 4) + 4 hh + r % 4 of the 32-dim block
   f32x16 l_acc[RB];            // row sums, from the matrix cores: every register of lane j32 holds the sum of row j32
-  float m_ref[RB], m_neg[RB], lmx[RB];
+  float m_ref[RB], lmx[RB];
+  float m_neg[RB];             // what is added to a scaled score ahead of the exponential: -m_ref (with a soft cap: cap - m_ref)
   float thr[RB];               // (m_ref + slack) in units of the raw scores: what a block's maximum is compared with
   u32x4 ops[PD];               // operands read ahead of their MFMAs
 #pragma unroll
@@ -332,8 +356,24 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       o_acc[rb][db] = z;
     }
   }
+  // Without a soft cap a probability is exp2(s sc_mul + m_neg).  With one, the capped score in log2 units is
+  // cap_out tanh(s cap_in) = cap_out (1 - 2 / (exp2(s cap_in2) + 1)), so the probability is exp2(r cap_m2 + m_neg) with
+  // r = 1 / (exp2(s cap_in2) + 1) and m_neg = cap_out - m_ref.
   const float sc_mul = p.scale_log2;
   const float inv_sc = 1.f / sc_mul;
+  const float cap_out = CAP ? p.softcap * 1.4426950408889634f : 0.f;
+  const float cap_in = CAP ? p.scale / p.softcap : 0.f;
+  const float cap_in2 = cap_in * 2.8853900817779268f;
+  const float cap_m2 = -2.f * cap_out;
+  auto capped = [&](float s) -> float { return cap_out * fast_tanh(s * cap_in); };  // a raw score to log2 units
+  auto prob = [&](float s, float mn) __attribute__((always_inline)) -> float {
+    if constexpr (CAP) {
+      const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s * cap_in2) + 1.f);
+      return s == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(r, cap_m2, mn));  // a masked key is not the cap's lower end
+    } else {
+      return __builtin_amdgcn_exp2f(__builtin_fmaf(s, sc_mul, mn));
+    }
+  };
   // The A operand of the row sums: ones, written to registers once, here.  (Left to the compiler it is rebuilt from
   // scalar registers right in front of the MFMA that reads it, and an MFMA issued through an assembly statement gets
   // no pause behind a vector instruction that writes one of its operands: it read the old register contents.)
@@ -356,13 +396,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       vaddr[db] = lds_base + (uint32_t)(KN * HALF + key * RKL + ((((off >> 4) ^ swz_key_v32<RKL>(key))) << 4) + (off & 15));
     }
   }
-  // operand kk of the block in half `half` of K slot `kslot` (offsets that are constants fold into the instruction)
-  auto read_k = [&](int kslot, int half, int kk) __attribute__((always_inline)) -> u32x4 {
-    return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)(kaddr[kk] + (uint32_t)(kslot * HALF + half * BK * RKL));
-  };
-  auto read_v = [&](int vslot, int half, int o) __attribute__((always_inline)) -> u32x4 {  // operand o = (db, s)
-    const int db = o / 2, s = o % 2;
-    const uint32_t a = vaddr[db] + (uint32_t)(vslot * HALF + (half * BK + 16 * s) * RKL);
+  auto rv_at = [&](uint32_t a) __attribute__((always_inline)) -> u32x4 {  // one V operand: 16 keys x 32 dims, transposed on the way
     const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)a));
     const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)(a + 8 * RKL)));
     return (u32x4){lo[0], lo[1], hi[0], hi[1]};
@@ -378,12 +412,19 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);  // the accumulators may still be on their way
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        const float mx = xor32_max(lmx[rb]) * sc_mul;
+        const float raw = xor32_max(lmx[rb]);
+        const float mx = CAP ? (raw == -INFINITY ? -INFINITY : capped(raw)) : raw * sc_mul;
         const float m_new = fmaxf(m_ref[rb], ceilf(mx));
         float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref[rb] - m_new);  // a power of two, or 0
         m_ref[rb] = m_new;
-        thr[rb] = (m_new + kMaxSlack) * inv_sc;
-        m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
+        if constexpr (CAP) {  // the raw score whose capped value is m_new + slack, if there is one
+          const float y = (m_new + kMaxSlack) / cap_out;
+          thr[rb] = (m_new == -INFINITY) ? -INFINITY : (y >= 0.999f ? INFINITY : 0.5f * __logf((1.f + y) / (1.f - y)) / cap_in);
+          m_neg[rb] = (m_new == -INFINITY) ? 0.f : cap_out - m_new;
+        } else {
+          thr[rb] = (m_new + kMaxSlack) * inv_sc;
+          m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
+        }
         asm volatile("s_nop 1" : "+v"(alpha));
         {
           f32x16 l = l_acc[rb];
@@ -410,23 +451,18 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // ---- the pinned step ---------------------------------------------------------------------------------------
   // PAR = (b + 1) % 2: the buffer of block b+1 (the other receives block b+2 and held block b).  ka: lane addresses of
   // the K operands of block b+2; kn: of the first PD operands of block b+3 (read at the end); va: lane addresses of the V
-  // operands of block b.
-  auto fast_step = [&](auto par_tag, const uint32_t (&ka)[NKK], const uint32_t (&kn)[PD], const uint32_t (&va)[DB], uint32_t dma_lds,
-                       const uint32_t (&dma_voff)[NLH], const char* dma_base) __attribute__((always_inline)) {
+  // operands of block b.  dl / dv0, dv1 / dg: LDS address, lane offsets and global base of the NG half tiles the step requests.
+  auto fast_step = [&](auto par_tag, const uint32_t (&ka)[NKK], const uint32_t (&kn)[PD], const uint32_t (&va)[DB], const uint32_t (&dl)[NG],
+                       const uint32_t (&dv0)[NLH], const uint32_t (&dv1)[NLH], const char* const (&dg)[NG]) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;
     f32x16 (&s_cur)[RB] = sa[PAR];              // S(b+1), consumed by the softmax
     f32x16 (&s_nxt)[RB] = sa[PAR ^ 1];          // S(b+2), produced
     u32x4 (&p_cur)[RB][2] = pb[PAR ^ 1];        // P(b), consumed by the PV product
     u32x4 (&p_nxt)[RB][2] = pb[PAR];            // P(b+1), produced
     auto rk = [&](uint32_t a) __attribute__((always_inline)) -> u32x4 { return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)a; };
-    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 {
-      const int db = o / 2, s = o % 2;
-      const uint32_t a = va[db] + (uint32_t)(16 * s * RKL);
-      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)a));
-      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)(a + 8 * RKL)));
-      return (u32x4){lo[0], lo[1], hi[0], hi[1]};
-    };
-    float xa = 0.f, xb = 0.f, ea = 0.f, eb = 0.f;  // softmax values in flight between slots
+    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 { return rv_at(va[o / 2] + (uint32_t)(16 * (o % 2) * RKL)); };
+    auto dma = [&](int j) __attribute__((always_inline)) { dma16_at(dl[j / NLH], j % NLH, j < NLH ? dv0[j % NLH] : dv1[j % NLH], dg[j / NLH]); };
+    float xa = 0.f, xb = 0.f, ea = 0.f, eb = 0.f, fa = 0.f, fb = 0.f;  // softmax values in flight between slots
     float mx_part[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) mx_part[rb] = -INFINITY;
@@ -448,9 +484,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       } else if (k < NQ + NSUM) {
         const int e = k - NQ, rb = e % RB, sh = e / RB;
         W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
-        // These slots carry no softmax and no operand read: the step's share of the tile loads is requested here (half
-        // a tile: NLH instructions), where the time the load unit takes to accept 1 KiB of addresses hides behind an MFMA.
-        if (e < NLH) dma16_at(dma_lds, e, dma_voff[e], dma_base);
+        // These slots carry no softmax and no operand read: the step's tile loads are requested from here on, where the
+        // time the load unit takes to accept 1 KiB of addresses hides behind an MFMA.
+        if (e < NDI) dma(e);
       } else {
         const int kk2 = k - NQ - NSUM, v = kk2 / RB, rb = kk2 % RB, db = v / 2, sh = v % 2, g = NKK + v;
         if (rb == 0 && g % 2 == 0) asm volatile("" ::"v"(ops[g % PD]), "v"(ops[(g + 1) % PD]));
@@ -460,34 +496,62 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           if (nx < NKK + NVO) ops[g % PD] = rv(nx - NKK);
           else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
         }
+        if (kk2 % 2 == 1 && NSUM + kk2 / 2 < NDI) dma(NSUM + kk2 / 2);
       }
-      // -- the softmax of block b+1, on the slots of the two products: pair i = (row block, register pair); first half
-      //    on even slots (the scaled differences of pair i, and pair i-1 packed), second half on odd slots (exponentials)
+      // -- the softmax of block b+1, on the slots of the two products: pair ip = (row block, register pair) owns SPP slots
       if (k < NQ || k >= NQ + NSUM) {
         const int ks = k < NQ ? k : k - NSUM;
-        const int ip = ks / 2;
-        if ((ks & 1) == 0) {
-          const int srb = ip / 8, sr2 = ip % 8;
-          xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
-          xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc_mul, m_neg[srb]);
-          if (ip > 0) {  // behind the two multiply-adds: they are the distance an exponential wants from its reader
-            const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;
-            p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
+        const int ip = ks / SPP, st = ks % SPP;
+        const int srb = ip / 8, sr2 = ip % 8;
+        const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;  // the pair before
+        if constexpr (!CAP) {
+          // first the scaled differences of the pair, and the pair before packed (behind the two multiply-adds: they are
+          // the distance an exponential wants from its reader); half the pair's slots on, the exponentials
+          if (st == 0) {
+            xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
+            xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc_mul, m_neg[srb]);
+            if (ip > 0) p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
+          } else if (st == SPP / 2) {
+            ea = __builtin_amdgcn_exp2f(xa);
+            eb = __builtin_amdgcn_exp2f(xb);
           }
         } else {
-          ea = __builtin_amdgcn_exp2f(xa);
-          eb = __builtin_amdgcn_exp2f(xb);
+          // four stages, one slot each; the last exponentials and the packing of a pair ride on the first two slots of the next
+          if (st == 0) {
+            xa = s_cur[srb][2 * sr2] * cap_in2;
+            xb = s_cur[srb][2 * sr2 + 1] * cap_in2;
+            if (ip > 0) {
+              fa = __builtin_amdgcn_exp2f(ea);
+              fb = __builtin_amdgcn_exp2f(eb);
+            }
+          } else if (st == 1) {
+            xa = __builtin_amdgcn_exp2f(xa);
+            xb = __builtin_amdgcn_exp2f(xb);
+            if (ip > 0) p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(fa, fb);
+          } else if (st == 2) {
+            xa += 1.f;
+            xb += 1.f;
+            xa = __builtin_amdgcn_rcpf(xa);
+            xb = __builtin_amdgcn_rcpf(xb);
+          } else {
+            ea = __builtin_fmaf(xa, cap_m2, m_neg[srb]);
+            eb = __builtin_fmaf(xb, cap_m2, m_neg[srb]);
+          }
         }
       }
-      // -- row maxima of S(b+2), whose MFMAs lie at least five slots back: one three-way maximum per PV slot
-      if (k >= NQ + NSUM) {
-        const int e = k - NQ - NSUM, mrb = e / 8, mr2 = e % 8;
+      // -- row maxima of S(b+2), whose MFMAs lie at least NSUM slots back: one three-way maximum per MSP PV slots
+      if (k >= NQ + NSUM && (k - NQ - NSUM) % MSP == 0) {
+        const int e = (k - NQ - NSUM) / MSP, mrb = e / 8, mr2 = e % 8;
         mx_part[mrb] = __builtin_fmaxf(__builtin_fmaxf(mx_part[mrb], s_nxt[mrb][2 * mr2]), s_nxt[mrb][2 * mr2 + 1]);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     {  // the last pair
       constexpr int jp = NPAIR - 1, prb = jp / 8, pr2 = jp % 8;
+      if constexpr (CAP) {
+        ea = __builtin_amdgcn_exp2f(ea);
+        eb = __builtin_amdgcn_exp2f(eb);
+      }
       p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
     }
 #pragma unroll
@@ -497,7 +561,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // ---- the same step written plainly, with run-time flags ---------------------------------------------------------
   // do_qk: block b+2 exists; do_sm: block b+1 exists; do_pv: block b >= 0; next_k: block b+3 exists (its first operands
   // are read at the end); first: the first operands of block b+2 have not been read ahead.  kb2: first key of block b+2.
-  // koff / nkoff / voff: byte offsets (slot and half) of blocks b+2 / b+3 in the K ring and of block b in the V ring.
+  // koff / nkoff / voff: byte offsets (slot and part) of blocks b+2 / b+3 in the K ring and of block b in the V ring.
   auto slow_step = [&](auto par_tag, uint32_t koff, uint32_t nkoff, uint32_t voff, bool do_qk, bool do_sm, bool do_pv, bool next_k, bool first, int kb2) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;
     f32x16 (&s_cur)[RB] = sa[PAR];
@@ -507,13 +571,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     auto rk = [&](uint32_t off, int kk) __attribute__((always_inline)) -> u32x4 {
       return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)(kaddr[kk] + off);
     };
-    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 {
-      const int db = o / 2, s = o % 2;
-      const uint32_t a = vaddr[db] + voff + (uint32_t)(16 * s * RKL);
-      const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)a));
-      const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(uintptr_t)(a + 8 * RKL)));
-      return (u32x4){lo[0], lo[1], hi[0], hi[1]};
-    };
+    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 { return rv_at(vaddr[o / 2] + voff + (uint32_t)(16 * (o % 2) * RKL)); };
     if (do_qk) {
       if (first) {
 #pragma unroll
@@ -534,8 +592,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int r2 = 0; r2 < 8; ++r2) {
-          const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[rb][2 * r2], sc_mul, m_neg[rb]));
-          const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[rb][2 * r2 + 1], sc_mul, m_neg[rb]));
+          const float e0 = prob(s_cur[rb][2 * r2], m_neg[rb]);
+          const float e1 = prob(s_cur[rb][2 * r2 + 1], m_neg[rb]);
           p_nxt[rb][r2 / 4][r2 % 4] = H::pack(e0, e1);
         }
     }
@@ -558,7 +616,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       }
     }
     if (do_qk) {  // mask S(b+2) in place and take the row maxima
-      mfma_settle(s_nxt[0], s_nxt[RB - 1]);
+      mfma_settle(s_nxt);
       const bool plain = kb2 >= wave_lo && kb2 + BK <= wave_hi;  // no row of the wave masks a key of this block
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
@@ -585,53 +643,44 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   };
 
   // ---- the walk over the key range -------------------------------------------------------------------------
-  // Trip tt (tt = -1 .. n_tiles - 1) is the two steps b = 2 tt, 2 tt + 1: scores of tile tt+1, PV products of tile tt.
-  // It starts at a barrier behind which K(tt+2) and V(tt) are visible and the slots of K(tt) and V(tt-1) are free:
-  // V(tt+3) and K(tt+4) are requested into them.  Requests so far, in order: K0 V0 K1 V1 K2 | V2 K3 | V3 K4 | ...
-  issue_k(0);
-  issue_v(0);
-  issue_k(1);
-  issue_v(1);
-  issue_k(2);
-  // trips the pinned code may serve: tt >= 0, tile tt+2 exists, tile tt+1 unmasked for the whole wave
-  const int tt_fast_lo = max(0, (wave_lo - kv_lo + TT - 1) / TT - 1);
-  // ... and tile tt+4 exists and lies wholly inside the context: the pinned steps request V(tt+3) and K(tt+4) themselves,
-  // with plain lane offsets
-  const int n_whole = min(n_tiles, (sp.ctx - kv_lo) / TT);  // tiles without a row past the context
-  const int tt_fast_hi = max(tt_fast_lo, min(n_whole - 4, (wave_hi - kv_lo) / TT - 1));  // first trip behind them
-  const int n_blocks = 2 * n_tiles;
-  auto trip_head = [&](int tt) __attribute__((always_inline)) {
-    // in flight may stay what the previous trip requested: V(tt+2) and K(tt+3)
-    const int vin = (tt + 2 < n_tiles && tt + 2 >= 2) ? 1 : 0, kin = (tt + 3 < n_tiles && tt + 3 >= 3) ? 1 : 0;
-    if (vin + kin == 2) wait_loads_and_barrier<2 * NLH>();
-    else if (vin + kin == 1) wait_loads_and_barrier<NLH>();
-    else wait_loads_and_barrier<0>();
-    issue_v(tt + 3);
-    issue_k(tt + 4);
-  };
-  auto slow_trip = [&](int tt) __attribute__((always_inline)) {
-    trip_head(tt);
+  // Step b (b = -2 .. n_blocks - 1): scores of block b+2, softmax of block b+1, PV product of block b.  Requests so far,
+  // in order: K and V of the tiles the first barrier expects behind it, then per barrier V(u + VAH), K(u + KAH).
+  const int n_blocks = SPT * n_tiles;
 #pragma unroll
-    for (int hb = 0; hb < 2; ++hb) {  // step b = 2 tt + hb: block b+2 = (tile tt+1, half hb), block b+3, block b = (tile tt, half hb)
-      const int b = 2 * tt + hb;
-      const bool do_qk = b + 2 < n_blocks, do_sm = b + 1 >= 0 && b + 1 < n_blocks, do_pv = b >= 0;
-      const bool next_k = b + 3 < n_blocks, first = b == -2;
-      const uint32_t koff = (uint32_t)(((tt + 1) & 3) * HALF + hb * BK * RKL);
-      const uint32_t nkoff = hb == 0 ? koff + BK * RKL : (uint32_t)(((tt + 2) & 3) * HALF);
-      const uint32_t voff = (uint32_t)((tt & 3) * HALF + hb * BK * RKL);
-      const int kb2 = kv_lo + (b + 2) * BK;
-      // buffers: block b+1 in (b + 1) % 2 = 1 - hb
-      if (hb == 0) {
-        if (do_sm) check(pb[0], do_pv);
-        slow_step(std::integral_constant<int, 1>{}, koff, nkoff, voff, do_qk, do_sm, do_pv, next_k, first, kb2);
-      } else {
-        if (do_sm) check(pb[1], do_pv);
-        slow_step(std::integral_constant<int, 0>{}, koff, nkoff, voff, do_qk, do_sm, do_pv, next_k, first, kb2);
-      }
-    }
+  for (int t = 0; t < U0 + KAH; ++t) {
+    next_tile();
+    if (t < n_tiles) issue_half(false, t % KN, td[0]);
+    if (t < U0 + VAH && t < n_tiles) issue_half(true, t % KN, td[0]);
+  }
+  auto ring_off = [&](int x) -> uint32_t { return (uint32_t)(((x / SPT) % KN) * HALF + (x % SPT) * BK * RKL); };  // block x >= 0 in its ring
+  auto head = [&](int u) __attribute__((always_inline)) {  // barrier u, written plainly
+    // in flight may stay the requests of the FLYB barriers before, where they made them in full
+    if (u - FLYB >= U0 && u - 1 + KAH < n_tiles) wait_loads_and_barrier<2 * FLYB * NLH>();
+    else wait_loads_and_barrier<0>();
+    const int vt = u + VAH, kt = u + KAH;
+    if (vt < n_tiles) issue_half(true, vt % KN, td[DQ - 1]);
+    next_tile();
+    if (kt < n_tiles) issue_half(false, kt % KN, td[0]);
   };
-  int tt = -1;
-  for (; tt < tt_fast_lo; ++tt) slow_trip(tt);
+  auto slow_step_at = [&](auto par_tag, int b) __attribute__((always_inline)) {
+    if (b % SPT == 0) head(b / SPT);  // (b is even wherever SPT is 2 and b is negative)
+    const bool do_qk = b + 2 < n_blocks, do_sm = b + 1 >= 0 && b + 1 < n_blocks, do_pv = b >= 0 && b < n_blocks;
+    const bool next_k = b + 3 < n_blocks, first = b == -2;
+    constexpr int PAR = decltype(par_tag)::value;
+    if (do_sm) check(pb[PAR ^ 1], do_pv);
+    slow_step(par_tag, ring_off(b + 2), ring_off(b + 3), ring_off(max(b, 0)), do_qk, do_sm, do_pv, next_k, first, kv_lo + (b + 2) * BK);
+  };
+  // Pairs of steps (b, b + 1), b even, the pinned code may serve: b >= 0, the barriers whose requests may be in flight
+  // were regular ones, blocks b+2 and b+3 exist and are unmasked for the whole wave ...
+  const int b_fast_lo = max(0, (((wave_lo - kv_lo + BK - 1) / BK - 2 + 1) >> 1) << 1);
+  // ... and the tiles its barriers request exist and lie wholly inside the context (requested with plain lane offsets)
+  const int n_whole = min(n_tiles, (sp.ctx - kv_lo) / TT);  // tiles without a row past the context
+  const int b_fast_hi = max(b_fast_lo, min((wave_hi - kv_lo) / BK - 3, SPT == 2 ? 2 * (n_whole - KAH) : n_whole - KAH - 1));  // first even b behind them
+  int b = -2;
+  for (; b < b_fast_lo; b += 2) {
+    slow_step_at(std::integral_constant<int, 1>{}, b);
+    slow_step_at(std::integral_constant<int, 0>{}, b + 1);
+  }
   // What the pinned loop reads but never writes is touched once here: should the compiler have parked any of it in
   // memory across the code above, its wait for the reload lands here and not inside the loop, where a wait on the
   // vector-memory counter would also wait for the tiles in flight.
@@ -642,39 +691,81 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
   for (int u = 0; u < NLH; ++u) asm volatile("" : "+v"(voff_k[u]), "+v"(voff_v[u]));
   asm volatile("" : "+v"(pages_vec));
-  for (; tt < tt_fast_hi; ++tt) {
-    // tiles up to K(tt+2) and V(tt) have landed; in flight stay the requests of the trip before, V(tt+2) and K(tt+3)
-    wait_loads_and_barrier<2 * NLH>();
-    // this trip requests V(tt+3), from inside its first step, and K(tt+4), from inside its second
-    const char* v_ptr = v_base + tile_off;  // tile tt+3: described when its K rows were requested
-    next_tile();
-    const char* k_ptr = k_base + tile_off;  // tile tt+4
-    const uint32_t v_lds = lds_base + (uint32_t)(KN + ((tt + 3) & 3)) * HALF + dma_wave_lds;
-    const uint32_t k_lds = lds_base + (uint32_t)((tt + 4) & 3) * HALF + dma_wave_lds;
-    // lane addresses of this trip's operands: K of tile tt+1, the first K operands of tile tt+2, V of tile tt
-    const uint32_t k_off = (uint32_t)(((tt + 1) & 3) * HALF), kn_off = (uint32_t)(((tt + 2) & 3) * HALF), v_off = (uint32_t)((tt & 3) * HALF);
-    uint32_t ka0[NKK], ka1[NKK], kn0[PD], kn1[PD], va0[DB], va1[DB];
+  if (b < b_fast_hi) {
+    int ru = (b / SPT) % KN;  // ring slot of tile u, u the index of the next barrier
+    auto slot_of = [&](auto c_tag) __attribute__((always_inline)) -> uint32_t {  // ring slot of tile u + c
+      constexpr int c = decltype(c_tag)::value % KN;
+      if constexpr ((KN & (KN - 1)) == 0) return (uint32_t)((ru + c) & (KN - 1));
+      else return (uint32_t)(ru + c >= KN ? ru + c - KN : ru + c);
+    };
+#define RPA_SLOT(c) slot_of(std::integral_constant<int, (c)>{})
+    // one barrier and the SPT steps behind it; PAR0: the buffer the first of them hands its softmax
+    auto fast_trip = [&](auto par_tag) __attribute__((always_inline)) {
+      constexpr int PAR0 = decltype(par_tag)::value;
+      // visible now: K tiles up to u + KNO, V tiles up to u; in flight stay the requests of the FLYB barriers before
+      wait_loads_and_barrier<2 * FLYB * NLH>();
+      // this barrier's requests, made from inside its steps: V(u + VAH), described DQ tiles ago, and K(u + KAH)
+      const char* v_ptr = v_base + td[DQ - 1].off;
+      next_tile(false);
+      const char* k_ptr = k_base + td[0].off;
+      const uint32_t v_lds = lds_base + (uint32_t)(KN + RPA_SLOT(VAH)) * HALF + dma_wave_lds;
+      const uint32_t k_lds = lds_base + RPA_SLOT(KAH) * HALF + dma_wave_lds;
+      if constexpr (SPT == 2) {
+        // operands: K of tile u+1, the first K operands of tile u+2, V of tile u
+        const uint32_t k_off = RPA_SLOT(1) * HALF, kn_off = RPA_SLOT(2) * HALF, v_off = RPA_SLOT(0) * HALF;
+        uint32_t ka0[NKK], ka1[NKK], kn0[PD], kn1[PD], va0[DB], va1[DB];
 #pragma unroll
-    for (int kk = 0; kk < NKK; ++kk) {
-      ka0[kk] = kaddr[kk] + k_off;
-      ka1[kk] = ka0[kk] + BK * RKL;  // a constant apart: folds into the instruction's offset
-    }
+        for (int kk = 0; kk < NKK; ++kk) {
+          ka0[kk] = kaddr[kk] + k_off;
+          ka1[kk] = ka0[kk] + BK * RKL;  // a constant apart: folds into the instruction's offset
+        }
 #pragma unroll
-    for (int o = 0; o < PD; ++o) {
-      kn0[o] = ka1[o];
-      kn1[o] = kaddr[o] + kn_off;
-    }
+        for (int o = 0; o < PD; ++o) {
+          kn0[o] = ka1[o];
+          kn1[o] = kaddr[o] + kn_off;
+        }
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
-      va0[db] = vaddr[db] + v_off;
-      va1[db] = va0[db] + BK * RKL;
+        for (int db = 0; db < DB; ++db) {
+          va0[db] = vaddr[db] + v_off;
+          va1[db] = va0[db] + BK * RKL;
+        }
+        const uint32_t dl0[1] = {v_lds}, dl1[1] = {k_lds};
+        const char* const dg0[1] = {v_ptr};
+        const char* const dg1[1] = {k_ptr};
+        check(pb[PAR0 ^ 1], true);
+        fast_step(std::integral_constant<int, PAR0>{}, ka0, kn0, va0, dl0, voff_v, voff_v, dg0);
+        check(pb[PAR0], true);
+        fast_step(std::integral_constant<int, PAR0 ^ 1>{}, ka1, kn1, va1, dl1, voff_k, voff_k, dg1);
+      } else {
+        // operands: K of tile u+2, the first K operands of tile u+3, V of tile u
+        const uint32_t k_off = RPA_SLOT(2) * HALF, kn_off = RPA_SLOT(3) * HALF, v_off = RPA_SLOT(0) * HALF;
+        uint32_t ka0[NKK], kn0[PD], va0[DB];
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk) ka0[kk] = kaddr[kk] + k_off;
+#pragma unroll
+        for (int o = 0; o < PD; ++o) kn0[o] = kaddr[o] + kn_off;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) va0[db] = vaddr[db] + v_off;
+        const uint32_t dl0[2] = {v_lds, k_lds};
+        const char* const dg0[2] = {v_ptr, k_ptr};
+        check(pb[PAR0 ^ 1], true);
+        fast_step(std::integral_constant<int, PAR0>{}, ka0, kn0, va0, dl0, voff_v, voff_k, dg0);
+      }
+      ru = ru + 1 == KN ? 0 : ru + 1;
+    };
+#undef RPA_SLOT
+    for (; b < b_fast_hi; b += 2) {
+      // No branch between the steps of an iteration: instructions of a pinned step must not find a later block to sink
+      // into.  An iteration moves the cursor by at most one column (pages hold two tiles or more).
+      refill_pages(1);
+      fast_trip(std::integral_constant<int, 1>{});
+      if constexpr (SPT == 1) fast_trip(std::integral_constant<int, 0>{});
     }
-    check(pb[0], true);
-    fast_step(std::integral_constant<int, 1>{}, ka0, kn0, va0, v_lds, voff_v, v_ptr);
-    check(pb[1], true);
-    fast_step(std::integral_constant<int, 0>{}, ka1, kn1, va1, k_lds, voff_k, k_ptr);
   }
-  for (; tt < n_tiles; ++tt) slow_trip(tt);
+  for (; b < n_blocks; b += 2) {
+    slow_step_at(std::integral_constant<int, 1>{}, b);
+    slow_step_at(std::integral_constant<int, 0>{}, b + 1);
+  }
 
   // ---- epilogue -----------------------------------------------------------------------------------------
   mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);
@@ -714,24 +805,31 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   }
 }
 
-template <int D, int NW, int RB, int HT>
+template <int D, int NW, int RB, int HT, bool CAP>
 static int launch_x32(hipStream_t stream, const AttnParams& p) {
-  const int64_t slots = ((int64_t)p.T * p.group) / kWideRows + p.S;  // upper bound on row tiles of the batch
+  constexpr int ROWS = NW * RB * 32;
+  if (p.pre_rows != ROWS) return (int)hipErrorInvalidValue;  // the plan and merge kernels are told this row-tile height
+  const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
   const int64_t blocks = slots * p.Hkv * p.pre_max_chunks;
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL((attn_prefill_x32_kernel<D, NW, RB, HT>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  hipLaunchKernelGGL((attn_prefill_x32_kernel<D, NW, RB, HT, CAP>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
   return (int)hipGetLastError();
 }
 
-// bf16 (or float16) pages of a multiple of 64 tokens, head size 128, no soft cap
-bool prefill_x32_supported(const AttnParams& p) {
-  return (p.kv_dtype == RPA_BF16 || p.kv_dtype == RPA_F16) && p.page_size % 64 == 0 && p.D == 128 && !(p.softcap > 0.f) &&
-         (int64_t)64 * p.token_stride < ((int64_t)1 << 31);
+// Query rows one workgroup of this kernel owns at the call's shape, 0 where the kernel does not apply.  Served: bf16 or
+// float16 pages of head size 128 without a soft cap (256 rows), bf16 pages of head size 256 with or without one (128
+// rows); page sizes that are multiples of 64 tokens.
+int prefill_x32_rows(const AttnParams& p) {
+  if (p.page_size % 64 != 0 || (int64_t)64 * p.token_stride >= ((int64_t)1 << 31)) return 0;
+  if (p.D == 128 && (p.kv_dtype == RPA_BF16 || p.kv_dtype == RPA_F16) && !(p.softcap > 0.f)) return 256;
+  if (p.D == 256 && p.kv_dtype == RPA_BF16) return 128;
+  return 0;
 }
 
 int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p) {
-  if (p.kv_dtype == RPA_F16) return launch_x32<128, 4, 2, RPA_F16>(stream, p);
-  return launch_x32<128, 4, 2, RPA_BF16>(stream, p);
+  if (p.D == 256) return p.softcap > 0.f ? launch_x32<256, 4, 1, RPA_BF16, true>(stream, p) : launch_x32<256, 4, 1, RPA_BF16, false>(stream, p);
+  if (p.kv_dtype == RPA_F16) return launch_x32<128, 4, 2, RPA_F16, false>(stream, p);
+  return launch_x32<128, 4, 2, RPA_BF16, false>(stream, p);
 }
 
 }  // namespace rpa

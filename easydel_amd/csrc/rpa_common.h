@@ -63,6 +63,7 @@ struct AttnParams {
   int pre_auto;        // 1: the plan kernel sets the chunk length from the batch's lengths; 0: pre_chunk as given
   int pre_slots;       // workgroups of the prefill kernel the chip holds at once
   int pre_rows;        // query rows (token x group head) one workgroup of the call's prefill kernel owns: 128 or 256
+  int pre_x32;         // 1: the 32x32-tile prefill kernel serves the call (pre_rows is its row-tile height)
   int decode_sync;   // decode workgroups re-align their waves with a barrier every this many tiles (power of two), 0 = never
   int decode_pace;   // 0: the decode kernel never pauses a wave (see PACE there); default 1
   int decode_dma;    // 1: bf16 decode tiles go global -> LDS directly where that kernel applies; 0: always through registers
@@ -277,8 +278,8 @@ int decode_row_limit(int T, int S, int D, int kv_dtype);
 bool prefill_supported(const AttnParams& p);
 bool prefill_dma_supported(const AttnParams& p);
 int launch_attn_prefill_dma8(hipStream_t stream, const AttnParams& p);  // 8-bit pages: codes loaded straight into LDS, widened there
-int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p);   // bf16 pages, 32x32x16 tiles, 256-row workgroups
-bool prefill_x32_supported(const AttnParams& p);
+int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p);   // 16-bit pages, 32x32x16 tiles, one workgroup per CU
+int prefill_x32_rows(const AttnParams& p);  // its row-tile height at the call's shape, 0 where it does not apply
 bool prefill_dma8_supported(const AttnParams& p);
 
 }  // namespace rpa
