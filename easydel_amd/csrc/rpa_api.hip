@@ -129,7 +129,7 @@ void prefill_split(int T, int S, int M, int page_size, int Hq, int Hkv, int D, i
   *max_chunks = chunks;
 }
 
-size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + 2 * ((size_t)S + 1) + rpa::kMaxDecodeWgs) * 4); }
+size_t plan_bytes(int S) { return align256(((size_t)rpa::kPlanHeader + 2 * ((size_t)S + 1) + rpa::kMaxDecodeWgs + 2 * rpa::kMaxSortedSeqs + 1) * 4); }
 
 // Static bound on query tokens the decode kernel can own: sequences with at most dec_rows rows per KV head.
 int decode_token_bound(int T, int S, int Hq, int Hkv, int dec_rows) {

@@ -524,6 +524,12 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     toks = sp.q_len;
     return (sp.hi - sp.lo + 63) & ~63;
   };
+  // Large-row sequences ordered longest first (by the keys an average row tile of theirs visits): the large-row
+  // kernel's workgroups are dealt to the chip in grid order, and the chip then idles for at most the shortest
+  // workgroup's time at the end, not the longest's.  One sequence per thread, ranks by counting.
+  __shared__ int s_key[kMaxSortedSeqs], s_tiles_of[kMaxSortedSeqs], s_rank_tiles[kMaxSortedSeqs];
+  const bool sorted = S <= kMaxSortedSeqs;
+  int my_key = -1, my_tiles = 0;
   int sum = 0, tsum = 0, toks;
   unsigned long long work = 0;  // keys the large-row kernel visits per KV head, over its row tiles (an estimate)
   int reach = 0;                // a bound on the keys one of its row tiles visits
@@ -541,7 +547,14 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
       span_min = min(span_min, span);
       span_max = max(span_max, span);
       n_tiles += tiles;
+      my_key = span;
+      my_tiles = tiles;
     }
+  }
+  if (sorted) {  // (per == 1: thread tid owns sequence tid)
+    s_key[tid] = my_key;
+    s_tiles_of[tid] = my_tiles;
+    s_rank_tiles[tid] = 0;
   }
   if (work) atomicAdd(&s_work, work);
   if (reach) {
@@ -567,6 +580,33 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     P[S + 1 + i] = min(trun, max(p.t_dec_max - 1, 0));
     run += span_of(i, seq_plan(p, i), toks);
     trun += toks;
+  }
+  {
+    int32_t* order = plan + kPlanHeader + 2 * (S + 1) + kMaxDecodeWgs;
+    int32_t* tile_start = order + kMaxSortedSeqs;
+    if (!sorted) {
+      if (tid == 0) plan[5] = -1;
+    } else if (s_large) {  // (uniform: written before the scans' barriers)
+      int rank = 0, n_large = 0;
+      for (int j = 0; j < S; ++j) {
+        const int kj = s_key[j];
+        n_large += kj >= 0;
+        rank += (kj > my_key) || (kj == my_key && j < tid);
+      }
+      if (my_key >= 0) {
+        order[rank] = tid;
+        s_rank_tiles[rank] = my_tiles;
+      }
+      __syncthreads();
+      if (tid <= n_large) {
+        int start = 0;
+        for (int r = 0; r < tid; ++r) start += s_rank_tiles[r];
+        tile_start[tid] = start;
+      }
+      if (tid == 0) plan[5] = n_large;
+    } else if (tid == 0) {
+      plan[5] = 0;
+    }
   }
   const int W = part[1023];
   if (tid == 0) {

@@ -152,8 +152,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   static_assert(!CAP || SPP == 4, "the soft cap's stages take four slots per pair");
   static_assert(NKK >= PD && NVO >= PD, "the operand ring is shorter than either phase");
   constexpr int NG = SPT == 2 ? 1 : 2;   // half tiles a step requests: at two steps per tile V in the first, K in the second
-  constexpr int NDI = NG * NLH;          // DMA instructions of a step: in the slots of the row sums, then every other PV slot
-  static_assert(NDI <= NSUM + NP / 2, "slots for the step's DMA instructions");
+  constexpr int NDI = NG * NLH;          // DMA instructions of a step: in the slots of the row sums ...
+  constexpr int DSP = (NQ + NP) / NDI;   // where they outnumber the slots of the row sums: one per DSP slots of the two products
 
   __shared__ __attribute__((aligned(1024))) unsigned char lds_all[2 * KN * HALF];
 
@@ -172,15 +172,32 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   if (p.plan[2] == 0) return;
   const int n_live = live_rows(p);
   if (n_live <= 0) return;
-  int lo_i = 0, hi_i = n_live;
-  while (hi_i - lo_i > 1) {
-    const int mid = (lo_i + hi_i) >> 1;
-    if ((int)(((int64_t)p.qsl[mid] * G) / ROWS) + mid <= slot) lo_i = mid; else hi_i = mid;
+  // Slot -> (sequence, row tile): through the plan's longest-first order where the plan kernel made one (the grid deals
+  // workgroups to the chip in this order), else sequence i starts at slot floor(qsl[i] G / ROWS) + i.
+  int i, tile_in_seq;
+  const int n_sorted = p.plan[5];
+  if (n_sorted >= 0) {
+    const int32_t* order = p.plan + kPlanHeader + 2 * (p.S + 1) + kMaxDecodeWgs;
+    const int32_t* tile_start = order + kMaxSortedSeqs;
+    if (n_sorted == 0 || slot >= tile_start[n_sorted]) return;
+    int lo_r = 0, hi_r = n_sorted;
+    while (hi_r - lo_r > 1) {
+      const int mid = (lo_r + hi_r) >> 1;
+      if (tile_start[mid] <= slot) lo_r = mid; else hi_r = mid;
+    }
+    i = order[lo_r];
+    tile_in_seq = slot - tile_start[lo_r];
+  } else {
+    int lo_i = 0, hi_i = n_live;
+    while (hi_i - lo_i > 1) {
+      const int mid = (lo_i + hi_i) >> 1;
+      if ((int)(((int64_t)p.qsl[mid] * G) / ROWS) + mid <= slot) lo_i = mid; else hi_i = mid;
+    }
+    i = lo_i;
+    tile_in_seq = slot - ((int)(((int64_t)p.qsl[i] * G) / ROWS) + i);
   }
-  const int i = lo_i;
   const SeqPlan sp = seq_plan(p, i);
   if (!sp.live || sp.small_rows) return;
-  const int tile_in_seq = slot - ((int)(((int64_t)sp.q0 * G) / ROWS) + i);
   const int rows_total = sp.q_len * G;
   const int R0 = tile_in_seq * ROWS;
   if (tile_in_seq < 0 || R0 >= rows_total) return;
@@ -486,7 +503,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
         // These slots carry no softmax and no operand read: the step's tile loads are requested from here on, where the
         // time the load unit takes to accept 1 KiB of addresses hides behind an MFMA.
-        if (e < NDI) dma(e);
+        if (NDI <= NSUM && e < NDI) dma(e);
       } else {
         const int kk2 = k - NQ - NSUM, v = kk2 / RB, rb = kk2 % RB, db = v / 2, sh = v % 2, g = NKK + v;
         if (rb == 0 && g % 2 == 0) asm volatile("" ::"v"(ops[g % PD]), "v"(ops[(g + 1) % PD]));
@@ -496,11 +513,11 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           if (nx < NKK + NVO) ops[g % PD] = rv(nx - NKK);
           else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
         }
-        if (kk2 % 2 == 1 && NSUM + kk2 / 2 < NDI) dma(NSUM + kk2 / 2);
       }
       // -- the softmax of block b+1, on the slots of the two products: pair ip = (row block, register pair) owns SPP slots
       if (k < NQ || k >= NQ + NSUM) {
         const int ks = k < NQ ? k : k - NSUM;
+        if (NDI > NSUM && ks % DSP == DSP - 1 && ks / DSP < NDI) dma(ks / DSP);  // more tile loads than row-sum slots: spread evenly
         const int ip = ks / SPP, st = ks % SPP;
         const int srb = ip / 8, sr2 = ip % 8;
         const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;  // the pair before

@@ -12,6 +12,7 @@ constexpr int kRowBlock = 16;      // MFMA M/N extent: rows (token, group-head p
 constexpr int kMaxSplitsCap = 256;   // hard upper bound on split-K partials per sequence
 constexpr int kPlanHeader = 16;      // ints before the prefix array in the decode plan
 constexpr int kMaxDecodeWgs = 4096;  // persistent decode workgroups per KV-head group
+constexpr int kMaxSortedSeqs = 1024; // batches of up to this many sequences get their large-row sequences ordered longest first
 constexpr int kPrefillRows = 128;    // query rows (token x group head) one prefill workgroup owns (the 32x32-tile kernel: 256; AttnParams::pre_rows)
 constexpr int kMaxPrefillChunks = 8; // key chunks one prefill row tile may be split into
 constexpr int kMinPrefillChunk = 2048; // fewest keys of such a chunk
@@ -40,7 +41,10 @@ struct AttnParams {
                    // the large-row kernel, [3] = 1 if the merge kernel has work, [4] = keys per split-K chunk of the
                    // large-row kernel, then at kPlanHeader:
                    // P[S+1] exclusive prefix of per-sequence key spans, R[S+1] exclusive prefix of
-                   // decode-class query tokens (row of a token in the partial buffers), first_seq[n_wg]
+                   // decode-class query tokens (row of a token in the partial buffers), first_seq[kMaxDecodeWgs],
+                   // then the large-row sequences longest first: [5] = their number L (-1: the batch has too many
+                   // sequences, not ordered), order[kMaxSortedSeqs] (sequence of rank r), tile_start[kMaxSortedSeqs + 1]
+                   // (exclusive prefix of their row-tile counts in that order)
   int T, S, M, P, page_size, Hq, Hkv, group, D, C;
   int Dq;                // elements of a q / out row.  D is the head size the kernels compute with: Dq itself, or -- on the
                          // MFMA path over padded head storage -- the stored row width (128 / 256), whose padding holds zeros
