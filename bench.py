@@ -96,7 +96,7 @@ def build_workload(name, seed, sequential=False):
 
 KERNEL_SOURCES = {  # the files a kernel is compiled from: a counter run is only valid for the sources it was taken on
     "attn_decode_kernel": ("rpa_attn_decode.hip", "rpa_attn_decode_dma.h", "rpa_mfma.h", "rpa_common.h"),
-    "attn_prefill_kernel": ("rpa_attn_prefill_dma.hip", "rpa_attn_prefill_dma8.hip", "rpa_attn_prefill.hip", "rpa_mfma.h", "rpa_common.h"),
+    "attn_prefill_kernel": ("rpa_attn_prefill_x32.hip", "rpa_attn_prefill_dma.hip", "rpa_attn_prefill_dma8.hip", "rpa_attn_prefill.hip", "rpa_mfma.h", "rpa_common.h"),
 }
 
 

@@ -22,9 +22,14 @@ GEOMETRIES = [(16, 64, BF16), (128, 64, BF16), (20, 32, BF16), (8, 128, BF16), (
 
 # 18 seeds by default; RPA_RANDOM_SEEDS in the environment widens the sweep
 _FIRST_SEED = int(os.environ.get("RPA_RANDOM_FIRST_SEED", "0"))  # a sweep over seeds no earlier sweep has seen starts here
+# Seeds a wider sweep once failed on, kept as regressions.  758: 20 heads, window 32 -- few visible keys whose values
+# cancel; with single bf16 softmax weights in the PV product one output of 3.55 missed by 2.1e-2.
+_REGRESSION_SEEDS = [758]
+_SEEDS = list(range(_FIRST_SEED, _FIRST_SEED + int(os.environ.get("RPA_RANDOM_SEEDS", "18"))))
+_SEEDS += [s for s in _REGRESSION_SEEDS if s not in _SEEDS]
 
 
-@pytest.mark.parametrize("seed", range(_FIRST_SEED, _FIRST_SEED + int(os.environ.get("RPA_RANDOM_SEEDS", "18"))))
+@pytest.mark.parametrize("seed", _SEEDS)
 def test_random_mla_batch(gpu, seed):
     rng = np.random.default_rng(5000 + seed)
     Hq, page_size, dtype = GEOMETRIES[seed % len(GEOMETRIES)]
