@@ -12,7 +12,7 @@ from easydel_amd import kernels
 from easydel_amd.caching import RaggedPagesMetadata
 from easydel_amd.operations import OperationMetadata, OperationRegistry
 from easydel_amd.operations.ragged_page_attention import dp_local_reduce
-from rpa_testlib import BF16, orc
+from rpa_testlib import BF16, FP8, INT8, orc
 
 pytestmark = pytest.mark.gpu
 
@@ -77,6 +77,55 @@ def test_dp_local_shards_sum_to_the_global_result(gpu, n_shards, page_size, Hq, 
     assert np.abs(tl.from_torch(out_global, BF16) - want).max() <= tl.TOL_BF16_MAX
     with pytest.raises(ValueError):
         op.forward_v3_dp_local_shard(q, k, v, pool[:local_pages], meta, 0, 3 if b["S"] % 3 else 7)
+
+
+@pytest.mark.parametrize("kv_dtype", [INT8, FP8])
+def test_dp_local_shards_of_a_scaled_8bit_pool(gpu, kv_dtype):
+    """A rank's share of a scaled 8-bit pool travels with its rows of the scales: the rank's write quantises into its
+    pages and scales, the ranks' outputs sum to the attention over the dequantised global pool, and int8 pages
+    without scales are refused."""
+    n_shards, local_pages, page_size, Hq, Hkv, D = 2, 400, 64, 32, 8, 128
+    b = _sharded_batch(75, n_shards, 5, local_pages, page_size, Hq, Hkv, D)
+    rng = np.random.default_rng(76)
+    P = b["P"]
+    # pages that already hold context: codes and per-(page, combined head) scales
+    codes = rng.integers(0, 255, size=(P, page_size, 2 * Hkv, D), dtype=np.uint8)
+    if kv_dtype == FP8:
+        codes[(codes & 0x7f) == 0x7f] = 0x3c  # no NaN codes in the stale contents
+    hi = 0.03 if kv_dtype == INT8 else 0.008  # the largest code is 127 / 448: stored values stay within a few units
+    scales = rng.uniform(hi / 3, hi, size=(P, 2 * Hkv)).astype(np.float32)
+    up = lambda a: torch.from_numpy(a).to(gpu)  # noqa: E731
+    meta = RaggedPagesMetadata(pages_tables=up(b["tables"]), context_lens=up(b["ctx"]), query_start_loc=up(b["qsl"]),
+                               num_seqs=torch.tensor([b["S"]], dtype=torch.int32, device=gpu),
+                               request_distribution=up(orc.request_distribution_ref(b["q_lens"], b["ctx"])), page_size=page_size)
+    q, k, v = (tl.to_torch(b[x], BF16, gpu) for x in ("q", "k", "v"))
+    torch_kv = {FP8: torch.float8_e4m3fn, INT8: torch.int8}[kv_dtype]
+    pool = up(codes).view(torch_kv)
+    pool_scales = up(scales)
+    op = OperationRegistry.create("ragged_page_attention_v3", OperationMetadata())
+    outs, new_codes, new_scales = [], [], []
+    for sh in range(n_shards):
+        rows = slice(sh * local_pages, (sh + 1) * local_pages)
+        out, pages, sc = op.forward_v3_dp_local_shard(q, k, v, pool[rows].clone(), meta, sh, n_shards,
+                                                      local_kv_scales=pool_scales[rows].clone(), num_kv_heads=Hkv)
+        torch.cuda.synchronize()
+        m = orc.dp_local_shard_ref(sh, n_shards, b["ctx"], b["tables"], b["qsl"], local_pages, b["T"])
+        assert not np.abs(tl.from_torch(out, BF16)[~m["token_mask"]]).any(), f"shard {sh}: rows of other ranks' tokens must be zero"
+        outs.append(out)
+        new_codes.append(pages.view(torch.uint8).cpu().numpy())
+        new_scales.append(sc.cpu().numpy())
+    # the ranks' writes together are the global quantising write, bit for bit
+    want_codes, want_scales = orc.page_scatter_ragged_quantised_ref(orc.bf16_bits_to_f32(b["k"]), orc.bf16_bits_to_f32(b["v"]), codes, scales,
+                                                                    b["ctx"], b["tables"], b["qsl"], [b["S"]], kv_dtype=kv_dtype)
+    assert np.array_equal(np.concatenate(new_scales), want_scales)
+    assert np.array_equal(np.concatenate(new_codes).reshape(want_codes.shape), want_codes)
+    kv_val = orc.decode_codes(want_codes, kv_dtype).astype(np.float64) * want_scales[:, None, :, None]
+    want = orc.ragged_paged_attention_ref(orc.bf16_bits_to_f32(b["q"]).astype(np.float64), kv_val, b["ctx"], b["tables"], b["qsl"], [b["S"]])
+    err = np.abs(tl.from_torch(dp_local_reduce(outs), BF16) - want)
+    assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (err.max(), err.mean())
+    if kv_dtype == INT8:
+        with pytest.raises(ValueError):
+            op.forward_v3_dp_local_shard(q, k, v, pool[:local_pages].clone(), meta, 0, n_shards)
 
 
 def test_mla_dp_local_shards_sum_to_the_global_result(gpu):
