@@ -690,9 +690,16 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // Pairs of steps (b, b + 1), b even, the pinned code may serve: b >= 0, the barriers whose requests may be in flight
   // were regular ones, blocks b+2 and b+3 exist and are unmasked for the whole wave ...
   const int b_fast_lo = max(0, (((wave_lo - kv_lo + BK - 1) / BK - 2 + 1) >> 1) << 1);
-  // ... and the tiles its barriers request exist and lie wholly inside the context (requested with plain lane offsets)
+  // ... and the tiles its barriers request (with plain lane offsets) are not the one that straddles the end of the
+  // context, whose rows past the end must not be fetched as they are.  Tiles past the key range may be requested: the
+  // cursor has moved on into valid pages (the next chunk's keys, or whatever page the table names: ids are clipped),
+  // the bytes land in ring slots nobody reads again, and the count of loads in flight stays what the barriers assume.
+  // The plain steps do not request such tiles, so the plain barriers ahead of the first pinned one must all have had
+  // real tiles to request.
   const int n_whole = min(n_tiles, (sp.ctx - kv_lo) / TT);  // tiles without a row past the context
-  const int b_fast_hi = max(b_fast_lo, min((wave_hi - kv_lo) / BK - 3, SPT == 2 ? 2 * (n_whole - KAH) : n_whole - KAH - 1));  // first even b behind them
+  const int b_req_hi = n_whole == n_tiles ? 0x7ffffff0 : (SPT == 2 ? 2 * (n_whole - KAH) : n_whole - KAH - 1);
+  const bool lead_in_full = b_fast_lo / SPT - 1 + KAH < n_tiles;
+  const int b_fast_hi = lead_in_full ? max(b_fast_lo, min(min((wave_hi - kv_lo) / BK - 3, n_blocks - 3), b_req_hi)) : b_fast_lo;  // first even b behind them
   int b = -2;
   for (; b < b_fast_lo; b += 2) {
     slow_step_at(std::integral_constant<int, 1>{}, b);
