@@ -36,6 +36,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill", "fp8-prefill", "int8-prefill", "gemma-decode",
+                             "decode-hkv4", "decode-hkv1", "decode-16seq", "decode-32seq",
                              "mla-decode-h128", "mla-decode-h16", "mla-prefill-h128"])
     ap.add_argument("--layout", default="interleaved", choices=["interleaved", "unified"],
                     help="interleaved: one pool [P, page, 2*Hkv, D], scatter fused with the attention call (v3); "
@@ -74,6 +75,10 @@ def parse_args():
     return ap.parse_args()
 
 
+DECODE_SHAPES = {"decode-hkv4": dict(Hq=28, Hkv=4), "decode-hkv1": dict(Hq=8, Hkv=1), "decode-16seq": dict(n_seqs=16),
+                 "decode-32seq": dict(n_seqs=32)}
+
+
 def build_workload(name, seed, sequential=False):
     import bench_workloads as workloads
 
@@ -91,6 +96,8 @@ def build_workload(name, seed, sequential=False):
         return workloads.gemma_decode(seed)
     if name == "llama-prefill":  # tuning shape for the prefill kernel, not one of the benchmark configurations
         return workloads.llama_long_prefill(seed)
+    if name in DECODE_SHAPES:  # tuning shapes: decode away from the benchmark's head counts and batch size
+        return workloads.decode_shape(seed, **DECODE_SHAPES[name])
     return workloads.config5_gemma_long_prefill(seed, windowed=(name == "c5-window"))
 
 

@@ -143,6 +143,18 @@ def config2_llama_decode(seed: int = 0, n_seqs: int = 256, num_pages: int = 40_0
                     block_tables=_tables(rng, ctx, 64, num_pages, 128, shuffle_pages), softmax_scale=128.0 ** -0.5)
 
 
+def decode_shape(seed: int = 0, *, Hq: int = 32, Hkv: int = 8, n_seqs: int = 256, num_pages: int | None = None) -> Workload:
+    """Not one of the five benchmark shapes: the pure-decode batch of C2 (contexts of 512..8192 tokens, head size 128,
+    64-token pages) at other head counts -- 28 / 4 and 8 / 1, the shards of a Qwen-shaped and a Llama-70B-shaped model under
+    tensor parallelism over the KV heads -- or at other batch sizes (16 and 32 sequences, where the call is launch-bound)."""
+    rng = np.random.default_rng(seed)
+    ctx = rng.integers(512, 8193, size=n_seqs).astype(np.int32)
+    pages = num_pages if num_pages is not None else int(np.ceil(ctx / 64).sum()) + 64
+    return Workload(f"pure decode, {Hq}/{Hkv} heads, {n_seqs} sequences (tuning shape)", Hq=Hq, Hkv=Hkv, D=128, page_size=64,
+                    num_pages=pages, max_pages_per_seq=128, context_lens=ctx, q_lens=np.ones(n_seqs, dtype=np.int32),
+                    block_tables=_tables(rng, ctx, 64, pages, 128), softmax_scale=128.0 ** -0.5)
+
+
 def config3_mixed_chunked(seed: int = 0, num_pages: int = 48_000) -> Workload:
     rng = np.random.default_rng(seed)
     dec = rng.integers(1024, 16385, size=64)
