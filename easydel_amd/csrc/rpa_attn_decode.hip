@@ -103,18 +103,15 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // With fewer KV heads than waves, the waves of a workgroup form groups of Hkv, and every group walks a span of its
-  // own (wave = head + Hkv * group): all waves stream, where otherwise WPB - Hkv of them would have nothing to do.
-  const int h = p.wave_groups > 1 ? wave % p.Hkv : (int)blockIdx.y * WPB + wave;
-  const int span_id = p.wave_groups > 1 ? (int)blockIdx.x * p.wave_groups + wave / p.Hkv : (int)blockIdx.x;
+  const int h = blockIdx.y * WPB + wave;
   if (h >= p.Hkv) return;
 
-  // ---- this workgroup's (wave group's) span of the flattened key stream -----------------------
+  // ---- this workgroup's span of the flattened key stream --------------------------------------
   const int32_t* __restrict__ plan = p.plan;
   const int W = plan[0], Q = plan[1];
   const int32_t* __restrict__ P = plan + kPlanHeader;
-  if ((int64_t)span_id * Q >= W) return;
-  const int span_begin = span_id * Q;
+  if ((int64_t)blockIdx.x * Q >= W) return;
+  const int span_begin = blockIdx.x * Q;
   const int span_end = min(W, span_begin + Q);
 
   const int G = p.group;
@@ -181,7 +178,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_kernel(AttnParams p) 
       counted = false;
     }
   };
-  Piece cur = make_piece(p, P, plan[kPlanHeader + 2 * (p.S + 1) + span_id], span_begin, span_end, Q);
+  Piece cur = make_piece(p, P, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
   int page_a = page_of(cur.i, cur.t_begin), page_b = 0;  // pages of the tiles in staging buffers 0 and 1
   enter();
   issue(Buf0{}, cur.t_begin, page_a);  // first tile in flight before anything else is set up
@@ -702,12 +699,8 @@ static int launch_rb(hipStream_t stream, AttnParams p) {
   const int head_groups = (p.Hkv + WPB - 1) / WPB;
   int n_wg = resident / head_groups;
   if (p.decode_wgs > 0) n_wg = p.decode_wgs;
-  // Fewer KV heads than waves (a power of two of them): groups of Hkv waves walk spans of their own.  Their tile counts
-  // differ, so the workgroup's re-aligning barrier is off.
-  p.wave_groups = (p.Hkv < WPB && WPB % p.Hkv == 0) ? WPB / p.Hkv : 1;
-  n_wg = max(1, min(n_wg, kMaxDecodeWgs / p.wave_groups));
-  p.n_wg = n_wg * p.wave_groups;
-  if (p.wave_groups > 1) p.decode_sync = 0;
+  n_wg = max(1, min(n_wg, kMaxDecodeWgs));
+  p.n_wg = n_wg;
   if (p.decode_which & 1) hipLaunchKernelGGL(decode_plan_kernel, dim3(p.new_k ? 1 + (p.T + kScatterTokensPerBlock - 1) / kScatterTokensPerBlock : 1), dim3(1024), 0, stream, p);
   if (p.decode_which & 2) {
     if constexpr (kHasDecodeDma<D, KVT, TT, WPB>) {

@@ -87,9 +87,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // (wave groups: see attn_decode_kernel)
-  const int h = p.wave_groups > 1 ? wave % p.Hkv : (int)blockIdx.y * WPB + wave;
-  const int span_id = p.wave_groups > 1 ? (int)blockIdx.x * p.wave_groups + wave / p.Hkv : (int)blockIdx.x;
+  const int h = blockIdx.y * WPB + wave;
   if (h >= p.Hkv) return;
 
   ConstI32 plan = (ConstI32)(uintptr_t)p.plan;
@@ -98,8 +96,8 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
   ConstI32 bt = (ConstI32)(uintptr_t)p.block_tables;
   const int W = plan[0], Q = plan[1];
   ConstI32 P = plan + kPlanHeader;
-  if ((int64_t)span_id * Q >= W) return;
-  const int span_begin = span_id * Q;
+  if ((int64_t)blockIdx.x * Q >= W) return;
+  const int span_begin = blockIdx.x * Q;
   const int span_end = min(W, span_begin + Q);
 
   const int G = p.group;
@@ -127,7 +125,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
   const char* pages_v = (const char*)p.v_pages + (int64_t)h * p.head_stride;
 
   // ---- issue side -------------------------------------------------------------------------------------------
-  DmaPiece ip = make_piece_dma(p, P, ctxs, qsl, plan[kPlanHeader + 2 * (p.S + 1) + span_id], span_begin, span_end, Q);
+  DmaPiece ip = make_piece_dma(p, P, ctxs, qsl, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
   int i_tok = ip.t_begin;     // first token of the next tile to issue
   bool i_live = true;         // false once the span's last tile has been issued
   int i_ks = 0, i_vs = 0;     // ring slots the next K / V half goes to
@@ -203,7 +201,7 @@ __global__ __launch_bounds__(64 * WPB, 1) void attn_decode_dma_kernel(AttnParams
   const float cap_in = CAP ? p.scale / p.softcap : 0.f;
 
   // ---- compute side ------------------------------------------------------------------------------------------
-  DmaPiece cur = make_piece_dma(p, P, ctxs, qsl, plan[kPlanHeader + 2 * (p.S + 1) + span_id], span_begin, span_end, Q);
+  DmaPiece cur = make_piece_dma(p, P, ctxs, qsl, plan[kPlanHeader + 2 * (p.S + 1) + blockIdx.x], span_begin, span_end, Q);
   int tg = 0;  // tiles computed so far in the span: tile tg lives in ring slots tg & 1
   for (;;) {
     const int rows = cur.q_len * G;

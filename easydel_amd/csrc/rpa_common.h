@@ -60,8 +60,7 @@ struct AttnParams {
   int max_splits;    // >= 2: most partial slots one sequence may use
   int dec_rows;      // most query rows per KV head (q_len * group) of a sequence the decode kernel serves: 16 or 32
   int t_dec_max;     // static bound on decode-class query tokens = rows of one partial slot
-  int n_wg;          // spans the flattened key stream is cut into per KV-head group: persistent decode workgroups x wave_groups
-  int wave_groups;   // > 1 (fewer KV heads than waves in a decode workgroup): waves w / Hkv of a workgroup walk spans of their own
+  int n_wg;          // persistent decode workgroups per KV-head group
   int decode_wgs;    // override for n_wg, 0 = as many as are resident at once
   int pre_chunk;     // keys per prefill split-K chunk (multiple of 64) when pre_auto is 0
   int pre_max_chunks;  // chunks the prefill partial buffers hold; 1 = never split
