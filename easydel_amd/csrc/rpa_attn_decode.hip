@@ -500,7 +500,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   const int S = p.S, tid = threadIdx.x;
   const int per = (S + 1023) / 1024;
   const int i0 = min(S, tid * per), i1 = min(S, i0 + per);
-  __shared__ int s_large, s_merge, s_reach, s_span_min, s_span_max, s_tiles;
+  __shared__ int s_large, s_merge, s_reach, s_span_min, s_span_max, s_tiles, s_chunk;
   __shared__ unsigned long long s_work;
   if (tid == 0) {
     s_large = 0;
@@ -524,9 +524,10 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     toks = sp.q_len;
     return (sp.hi - sp.lo + 63) & ~63;
   };
-  // Large-row sequences ordered longest first (by the keys an average row tile of theirs visits): the large-row
-  // kernel's workgroups are dealt to the chip in grid order, and the chip then idles for at most the shortest
-  // workgroup's time at the end, not the longest's.  One sequence per thread, ranks by counting.
+  // Large-row sequences ordered by the length of their workgroups, longest first (the keys an average row tile of
+  // theirs visits over the chunks it is cut into): the large-row kernel's workgroups are dealt to the chip in grid
+  // order, and the chip then idles for at most the shortest workgroup's time at the end, not the longest's.  One
+  // sequence per thread, ranks by counting, once the chunk length is known.
   __shared__ int s_key[kMaxSortedSeqs], s_tiles_of[kMaxSortedSeqs], s_rank_tiles[kMaxSortedSeqs];
   const bool sorted = S <= kMaxSortedSeqs;
   int my_key = -1, my_tiles = 0;
@@ -581,33 +582,6 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     run += span_of(i, seq_plan(p, i), toks);
     trun += toks;
   }
-  {
-    int32_t* order = plan + kPlanHeader + 2 * (S + 1) + kMaxDecodeWgs;
-    int32_t* tile_start = order + kMaxSortedSeqs;
-    if (!sorted) {
-      if (tid == 0) plan[5] = -1;
-    } else if (s_large) {  // (uniform: written before the scans' barriers)
-      int rank = 0, n_large = 0;
-      for (int j = 0; j < S; ++j) {
-        const int kj = s_key[j];
-        n_large += kj >= 0;
-        rank += (kj > my_key) || (kj == my_key && j < tid);
-      }
-      if (my_key >= 0) {
-        order[rank] = tid;
-        s_rank_tiles[rank] = my_tiles;
-      }
-      __syncthreads();
-      if (tid <= n_large) {
-        int start = 0;
-        for (int r = 0; r < tid; ++r) start += s_rank_tiles[r];
-        tile_start[tid] = start;
-      }
-      if (tid == 0) plan[5] = n_large;
-    } else if (tid == 0) {
-      plan[5] = 0;
-    }
-  }
   const int W = part[1023];
   if (tid == 0) {
     P[S] = W;
@@ -641,9 +615,46 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     plan[3] = s_merge;  // anything for the merge kernel?
     plan[4] = (int)chunk;
     s_Q = q;
+    s_chunk = (int)min(chunk, (long long)0x7fffffff);
   }
   __threadfence_block();
   __syncthreads();
+  {
+    int32_t* order = plan + kPlanHeader + 2 * (S + 1) + kMaxDecodeWgs;
+    int32_t* tile_start = order + kMaxSortedSeqs;
+    if (!sorted) {
+      if (tid == 0) plan[5] = -1;
+    } else if (s_large) {  // (uniform: written before the scans' barriers)
+      // the key: the keys one workgroup of the sequence visits, i.e. its span over the number of chunks it is cut into
+      // (prefill_tile's rule, on the sequence's average row tile)
+      if (my_key >= 0) {
+        const int target = s_chunk;
+        const int n = min(max((int)(((int64_t)my_key + target / 2) / target), 1), p.pre_max_chunks);
+        my_key = (my_key + n - 1) / n;
+      }
+      s_key[tid] = my_key;
+      __syncthreads();
+      int rank = 0, n_large = 0;
+      for (int j = 0; j < S; ++j) {
+        const int kj = s_key[j];
+        n_large += kj >= 0;
+        rank += (kj > my_key) || (kj == my_key && j < tid);
+      }
+      if (my_key >= 0) {
+        order[rank] = tid;
+        s_rank_tiles[rank] = my_tiles;
+      }
+      __syncthreads();
+      if (tid <= n_large) {
+        int start = 0;
+        for (int r = 0; r < tid; ++r) start += s_rank_tiles[r];
+        tile_start[tid] = start;
+      }
+      if (tid == 0) plan[5] = n_large;
+    } else if (tid == 0) {
+      plan[5] = 0;
+    }
+  }
   // first sequence of every workgroup: the last i with P[i] <= j*Q (the kernel then skips empty ones)
   const int Q = s_Q;
   for (int j = tid; j < p.n_wg; j += 1024) {
