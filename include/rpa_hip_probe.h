@@ -82,8 +82,9 @@ double rpa_mfma_probe(rpa_stream_t stream, int shape, int source, int mfmas_per_
  *                    fixed from the block-table bound (1 = never split); set it before sizing the workspace
  *   "prefill_dma"    1 (default): prefill tiles are loaded global -> LDS by the load unit where those kernels apply
  *                    (page_size % 32 == 0); 0: every prefill tile is staged through registers (bf16 / 8-bit pages only)
- *   "prefill_x32"    1 (default): bf16 / float16 pages of a multiple of 64 tokens at head size 128, without soft cap, take the
- *                    prefill kernel built on 32x32x16 tiles (256-row workgroups); 0: never
+ *   "prefill_x32"    1 (default): pages of a multiple of 64 tokens take the prefill kernel built on 32x32x16 tiles, one
+ *                    workgroup per CU, at head size 128 (bf16 / float16 pages, no soft cap: 256-row workgroups) and at
+ *                    head size 256 (bf16 pages, with or without soft cap: 128-row workgroups); 0: never
  *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
  *                    the shapes, and batches of few row tiles cut by a chunk length chosen on the device from their
  *                    own lengths); set it before sizing the workspace

@@ -287,6 +287,46 @@ def test_prefill_register_staged_kernel_serves_bf16_too(gpu, D, page_size, Hq, H
     assert np.abs(direct[tl.valid_rows(b)] - staged[tl.valid_rows(b)]).max() <= 2e-2
 
 
+@pytest.mark.parametrize("D,page_size,Hq,Hkv,cap", [(128, 64, 32, 8, None), (256, 128, 16, 8, 50.0), (256, 64, 8, 4, None)])
+@pytest.mark.parametrize("window", [None, 333])
+def test_prefill_kernel_on_32x32_tiles(gpu, D, page_size, Hq, Hkv, cap, window):
+    # The large-row kernel built on 32x32x16 tiles (one workgroup per CU; 256 rows at head size 128, 128 at 256): contexts
+    # that end on every residue of its 32-key blocks and make odd and even block counts, a chunk deep in a context, a row
+    # tile with a single live row, key ranges cut into chunks by the device's rule and by a fixed count -- against the
+    # oracle, and against the kernel on 16x16x32 tiles that serves these shapes when this one is switched off.
+    from easydel_amd import _lib
+
+    ctx = [1, 31, 32, 33, 95, 96, 97, 161, 640, 2100, 1500, 4000]
+    q_lens = [1, 31, 32, 33, 95, 96, 97, 129, 640, 70, 513, 300]
+    b = tl.make_batch(61 + D, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, pad_rows=1, pad_tokens=3, max_pages=-(-4000 // page_size))
+    kw = dict(sliding_window=window, logits_soft_cap=cap, softmax_scale=D ** -0.5)
+    rows = tl.valid_rows(b)
+    want = tl.oracle_out(b, **kw)
+
+    def run(what):
+        got = tl.run_gpu_attention(b, **kw)
+        mx, mean = tl.assert_close(got, want, b, what)
+        print(f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+        return got
+
+    wide = run(f"32x32 prefill D{D} window {window}")
+    for chunks in (3, 8):  # fixed chunk counts: every row tile of the long sequences leaves partials for the merge
+        prev = _lib.set_tunable("prefill_chunks", chunks)
+        try:
+            cut = run(f"32x32 prefill D{D} window {window}, {chunks} key chunks")
+        finally:
+            _lib.set_tunable("prefill_chunks", prev)
+        assert np.abs(cut[rows] - wide[rows]).max() <= 2e-2
+    prev = _lib.set_tunable("prefill_x32", 0)
+    try:
+        narrow = run(f"16x16 prefill D{D} window {window}")
+    finally:
+        _lib.set_tunable("prefill_x32", prev)
+    assert np.abs(wide[rows] - narrow[rows]).max() <= 2e-2
+    again = tl.run_gpu_attention(b, **kw)
+    assert np.array_equal(again[rows], wide[rows]), "two runs of the same call must agree bit for bit"
+
+
 def test_chunked_prefill_equals_rows_of_single_shot_prefill(gpu):
     # the same keys, queried as one 384-token prefill and as its last 128-token chunk
     b_full = tl.make_batch(53, [384], [384], Hq=32, Hkv=8, D=128, page_size=64)
