@@ -478,7 +478,10 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     u32x4 (&p_nxt)[RB][2] = pb[PAR];            // P(b+1), produced
     auto rk = [&](uint32_t a) __attribute__((always_inline)) -> u32x4 { return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)a; };
     auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 { return rv_at(va[o / 2] + (uint32_t)(16 * (o % 2) * RKL)); };
-    auto dma = [&](int j) __attribute__((always_inline)) { dma16_at(dl[j / NLH], j % NLH, j < NLH ? dv0[j % NLH] : dv1[j % NLH], dg[j / NLH]); };
+    auto dma = [&](int j) __attribute__((always_inline)) {  // m0 is set by a half tile's first request and kept for its others
+      if (j % NLH == 0) dma16_at(dl[j / NLH], 0, j < NLH ? dv0[0] : dv1[0], dg[j / NLH]);
+      else dma16_at_same_m0(j % NLH, j < NLH ? dv0[j % NLH] : dv1[j % NLH], dg[j / NLH]);
+    };
     float xa = 0.f, xb = 0.f, ea = 0.f, eb = 0.f, fa = 0.f, fb = 0.f;  // softmax values in flight between slots
     float mx_part[RB];
 #pragma unroll
@@ -514,6 +517,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
         }
       }
+      // The MFMA leads its slot: left free, the compiler moves a slot's pack ahead of it, directly behind the exponentials
+      // of the slot before, where it needs a wait state of its own and then waits for their results.
+      __builtin_amdgcn_sched_barrier(0);
       // -- the softmax of block b+1, on the slots of the two products: pair ip = (row block, register pair) owns SPP slots
       if (k < NQ || k >= NQ + NSUM) {
         const int ks = k < NQ ? k : k - NSUM;

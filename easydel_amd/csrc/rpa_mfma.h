@@ -157,6 +157,15 @@ __device__ __forceinline__ void dma16_at(uint32_t lds_addr, int u, uint32_t voff
   else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 offset:3072" ::"s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
+// ... and with m0 left as the instruction before of the same group set it (u > 0).  Only for instruction streams in
+// which nothing between the group's instructions writes m0: the compiler does so for indexed register moves, lane reads
+// by a vector index and LDS DMA of its own, none of which the pinned steps that use this contain.
+__device__ __forceinline__ void dma16_at_same_m0(int u, uint32_t voff, const void* base) {
+  if (u == 1) asm volatile("global_load_lds_dwordx4 %0, %1 offset:1024" ::"v"(voff), "s"(base) : "memory");
+  else if (u == 2) asm volatile("global_load_lds_dwordx4 %0, %1 offset:2048" ::"v"(voff), "s"(base) : "memory");
+  else asm volatile("global_load_lds_dwordx4 %0, %1 offset:3072" ::"v"(voff), "s"(base) : "memory");
+}
+
 // ... with the non-temporal hint, for data no wave will ask for again (the pages a decode kernel streams): kept out
 // of the caches' longer-lived lines, such a stream reads HBM measurably faster.
 __device__ __forceinline__ void dma16_nt(uint32_t lds_addr, uint32_t voff, const void* base) {
