@@ -116,6 +116,54 @@ def test_product_build_has_no_probes_and_no_stage_knob(tmp_path):
     assert "decode_sync" in strings  # the tuning knobs stay
 
 
+def test_the_pinned_prefill_steps_are_what_the_source_says(tmp_path):
+    """The 32x32-tile prefill kernel issues its MFMAs and its tile requests through assembly statements, which the
+    compiler neither pads nor sees into; two things it relies on are checked on the generated code.  (1) m0, which a
+    half tile's first request sets for the others, is written by nothing but those statements.  (2) Inside the pinned
+    loops (the blocks that hold a whole step's MFMAs) there is no scratch-memory access and no wait on the vector-memory
+    counter other than the steps' own: either would wait for the tiles in flight."""
+    import re
+    import subprocess
+
+    from easydel_amd import build
+
+    asm = tmp_path / "x32.s"
+    cmd = [build._hipcc(), *build.HIPCC_FLAGS, "-S", "--cuda-device-only", str(build.CSRC / "rpa_attn_prefill_x32.hip"), "-o", str(asm)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-2000:]
+    lines = asm.read_text().splitlines()
+    in_asm, kernel, block, blocks = False, None, None, {}
+    for n, line in enumerate(lines, 1):
+        text = line.strip()
+        if "#ASMSTART" in text:
+            in_asm = True
+        elif "#ASMEND" in text:
+            in_asm = False
+        m = re.match(r"^(_ZN3rpa23attn_prefill_x32_kernel\w+):", line)
+        if m:
+            kernel = m.group(1)
+        m = re.match(r"^(\.LBB\d+_\d+):", line)
+        if m and kernel:
+            block = (kernel, m.group(1))
+            blocks[block] = []
+        if not text or text.startswith(";") or text.startswith("."):
+            continue
+        if not in_asm:
+            assert not re.search(r"\bm0\b", text), f"line {n}: the compiler's own code touches m0: {text}"
+        if block:
+            blocks[block].append((text, in_asm))
+    pinned = {b: ins for b, ins in blocks.items() if sum(t.startswith("v_mfma") for t, _ in ins) >= 30}
+    bf16 = [b for b in pinned if "ELi1ELb" in b[0]]  # the bf16 instantiations: the benchmark shapes
+    assert len(bf16) >= 6, sorted(pinned)  # two pinned steps each at head size 128, 256 and 256 with soft cap
+    for b in bf16:
+        ins = pinned[b]
+        last = max(i for i, (t, _) in enumerate(ins) if t.startswith("v_mfma"))
+        first = min(i for i, (t, _) in enumerate(ins) if t.startswith("v_mfma"))
+        for t, from_asm in ins[first:last + 1]:
+            assert not t.startswith("scratch_"), f"{b}: scratch access inside a pinned step: {t}"
+            assert from_asm or "vmcnt" not in t, f"{b}: the compiler waits on vector memory inside a pinned step: {t}"
+
+
 def test_multi_latent_entry_points_validate_before_any_device_work():
     lib = _lib.load()
     a = 0x7000_0000_0000
