@@ -456,8 +456,10 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     int err = 0;
     if (stages & 3) err = rpa::launch_attn_decode(s, p, stages & 3);
     if (err) return hip_fail(err, "decode kernel launch");
-    // Rows too large for the decode kernel: MFMA prefill kernel where it applies, fp32 kernel otherwise.
-    if (stages & 4) err = rpa::prefill_supported(p) ? rpa::launch_attn_prefill(s, p) : rpa::launch_attn_generic(s, p);
+    // Rows too large for the decode kernel: MFMA prefill kernel where it applies, fp32 kernel otherwise.  No launch where
+    // the call's bounds rule such rows out (all its tokens together make no more rows per KV head than the decode kernel takes).
+    const bool large_rows_possible = (int64_t)T * p.group > p.dec_rows;
+    if ((stages & 4) && large_rows_possible) err = rpa::prefill_supported(p) ? rpa::launch_attn_prefill(s, p) : rpa::launch_attn_generic(s, p);
     if (err) return hip_fail(err, "prefill kernel launch");
   } else {
     int err = (stages & 4) ? rpa::launch_attn_generic(s, p) : 0;
