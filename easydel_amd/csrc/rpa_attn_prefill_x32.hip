@@ -469,7 +469,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // PAR = (b + 1) % 2: the buffer of block b+1 (the other receives block b+2 and held block b).  ka: lane addresses of
   // the K operands of block b+2; kn: of the first PD operands of block b+3 (read at the end); va: lane addresses of the V
   // operands of block b.  dl / dv0, dv1 / dg: LDS address, lane offsets and global base of the NG half tiles the step requests.
-  auto fast_step = [&](auto par_tag, const uint32_t (&ka)[NKK], const uint32_t (&kn)[PD], const uint32_t (&va)[DB], const uint32_t (&dl)[NG],
+  auto fast_step = [&](auto par_tag, auto&& ka, auto&& kn, auto&& va, auto&& in_slot, const uint32_t (&dl)[NG],
                        const uint32_t (&dv0)[NLH], const uint32_t (&dv1)[NLH], const char* const (&dg)[NG]) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;
     f32x16 (&s_cur)[RB] = sa[PAR];              // S(b+1), consumed by the softmax
@@ -477,7 +477,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     u32x4 (&p_cur)[RB][2] = pb[PAR ^ 1];        // P(b), consumed by the PV product
     u32x4 (&p_nxt)[RB][2] = pb[PAR];            // P(b+1), produced
     auto rk = [&](uint32_t a) __attribute__((always_inline)) -> u32x4 { return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)a; };
-    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 { return rv_at(va[o / 2] + (uint32_t)(16 * (o % 2) * RKL)); };
+    auto rv = [&](int o) __attribute__((always_inline)) -> u32x4 { return rv_at(va(o / 2) + (uint32_t)(16 * (o % 2) * RKL)); };
     auto dma = [&](int j) __attribute__((always_inline)) {  // m0 is set by a half tile's first request and kept for its others
       if (j % NLH == 0) dma16_at(dl[j / NLH], 0, j < NLH ? dv0[0] : dv1[0], dg[j / NLH]);
       else dma16_at_same_m0(j % NLH, j < NLH ? dv0[j % NLH] : dv1[j % NLH], dg[j / NLH]);
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         else W::mfma_s(s_nxt[rb], ops[g % PD], qf[rb][g]);
         if (rb == RB - 1) {
           const int nx = g + PD;
-          if (nx < NKK) ops[g % PD] = rk(ka[nx]);
+          if (nx < NKK) ops[g % PD] = rk(ka(nx));
           else ops[g % PD] = rv(nx - NKK);
         }
       } else if (k < NQ + NSUM) {
@@ -514,7 +514,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         if (rb == RB - 1) {
           const int nx = g + PD;
           if (nx < NKK + NVO) ops[g % PD] = rv(nx - NKK);
-          else ops[g % PD] = rk(kn[nx - NKK - NVO]);  // the next step's first operands
+          else ops[g % PD] = rk(kn(nx - NKK - NVO));  // the next step's first operands
         }
       }
       // The MFMA leads its slot: left free, the compiler moves a slot's pack ahead of it, directly behind the exponentials
@@ -561,12 +561,16 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
             eb = __builtin_fmaf(xb, cap_m2, m_neg[srb]);
           }
         }
+        // (the last pair's stages have no reader inside the step: unpinned they gather behind its last MFMA)
+        if (ip == NPAIR - 1) asm volatile("" : "+v"(xa), "+v"(xb), "+v"(ea), "+v"(eb));
       }
       // -- row maxima of S(b+2), whose MFMAs lie at least NSUM slots back: one three-way maximum per MSP PV slots
       if (k >= NQ + NSUM && (k - NQ - NSUM) % MSP == 0) {
         const int e = (k - NQ - NSUM) / MSP, mrb = e / 8, mr2 = e % 8;
         mx_part[mrb] = __builtin_fmaxf(__builtin_fmaxf(mx_part[mrb], s_nxt[mrb][2 * mr2]), s_nxt[mrb][2 * mr2 + 1]);
+        asm volatile("" : "+v"(mx_part[mrb]));  // in this slot: left free, the chain of maxima gathers behind the step's last MFMA
       }
+      in_slot(k);  // what the caller wants done during this slot: the lane addresses of the steps to come
       __builtin_amdgcn_sched_barrier(0);
     }
     {  // the last pair
@@ -722,68 +726,78 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   for (int u = 0; u < NLH; ++u) asm volatile("" : "+v"(voff_k[u]), "+v"(voff_v[u]));
   asm volatile("" : "+v"(pages_vec));
   if (b < b_fast_hi) {
-    int ru = (b / SPT) % KN;  // ring slot of tile u, u the index of the next barrier
-    auto slot_of = [&](auto c_tag) __attribute__((always_inline)) -> uint32_t {  // ring slot of tile u + c
-      constexpr int c = decltype(c_tag)::value % KN;
-      if constexpr ((KN & (KN - 1)) == 0) return (uint32_t)((ru + c) & (KN - 1));
-      else return (uint32_t)(ru + c >= KN ? ru + c - KN : ru + c);
+    // Ring offsets of the tiles u .. u + KN - 1, u the index of the next barrier (r[c]: tile u + c), turned once per barrier.
+    uint32_t r[KN];
+#pragma unroll
+    for (int c = 0; c < KN; ++c) r[c] = (uint32_t)(((b / SPT + c) % KN) * HALF);
+    // Lane addresses the steps read their operands through: ring offset added.  A: K of tile u + KC (the tile whose
+    // scores the barrier's steps take); VA: V of tile u.  Operands 8 k-steps, or 4 dim blocks, apart lie 256 bytes apart
+    // whatever the lane's swizzle key, and the parts of a tile a constant apart: those fold into the instructions' offsets.
+    // Each is replaced by the next barrier's value behind its last use, by an addition pinned to a slot of the step:
+    // computed at the head of a step, ahead of its first MFMA, the additions are time the matrix pipe stands idle.
+    constexpr int KC = SPT == 2 ? 1 : 2;
+    constexpr int NKA = NKK < 8 ? NKK : 8, NVA = DB < 4 ? DB : 4;
+    static_assert(NKK % NKA == 0 && DB % NVA == 0 && NKA >= PD, "");
+    uint32_t A[NKA], VA[NVA];
+#pragma unroll
+    for (int kk = 0; kk < NKA; ++kk) A[kk] = kaddr[kk] + r[KC];
+#pragma unroll
+    for (int db = 0; db < NVA; ++db) VA[db] = vaddr[db] + r[0];
+    const uint32_t k_lds0 = lds_base + dma_wave_lds, v_lds0 = k_lds0 + (uint32_t)(KN * HALF);
+    auto pinned_add = [&](uint32_t sgpr, uint32_t vgpr) __attribute__((always_inline)) -> uint32_t {
+      uint32_t d;
+      asm volatile("v_add_u32 %0, %1, %2" : "=v"(d) : "s"(sgpr), "v"(vgpr));
+      return d;
     };
-#define RPA_SLOT(c) slot_of(std::integral_constant<int, (c)>{})
+    // The last step of a barrier moves the addresses on: K once the step's own K operands are read (the row-sum slots on;
+    // the operands read at its end are the next barrier's), V behind the last V operand.
+    constexpr int K_UPD0 = NQ, K_UPD_SLOTS = NSUM + 4, V_UPD0 = NQ + NSUM + NP - 4;
+    constexpr int K_PER = (NKA + K_UPD_SLOTS - 1) / K_UPD_SLOTS;
+    auto move_on = [&](int k) __attribute__((always_inline)) {
+#pragma unroll
+      for (int kk = 0; kk < NKA; ++kk)
+        if (k == K_UPD0 + kk / K_PER) A[kk] = pinned_add(r[(KC + 1) % KN], kaddr[kk]);
+#pragma unroll
+      for (int db = 0; db < NVA; ++db)
+        if (k == V_UPD0 + db) VA[db] = pinned_add(r[1 % KN], vaddr[db]);
+    };
+    auto nothing = [&](int) __attribute__((always_inline)) {};
     // one barrier and the SPT steps behind it; PAR0: the buffer the first of them hands its softmax
     auto fast_trip = [&](auto par_tag) __attribute__((always_inline)) {
       constexpr int PAR0 = decltype(par_tag)::value;
       // visible now: K tiles up to u + KNO, V tiles up to u; in flight stay the requests of the FLYB barriers before
       wait_loads_and_barrier<2 * FLYB * NLH>();
+      check(pb[PAR0 ^ 1], true);
       // this barrier's requests, made from inside its steps: V(u + VAH), described DQ tiles ago, and K(u + KAH)
       const char* v_ptr = v_base + td[DQ - 1].off;
       next_tile(false);
       const char* k_ptr = k_base + td[0].off;
-      const uint32_t v_lds = lds_base + (uint32_t)(KN + RPA_SLOT(VAH)) * HALF + dma_wave_lds;
-      const uint32_t k_lds = lds_base + RPA_SLOT(KAH) * HALF + dma_wave_lds;
+      const uint32_t v_lds = v_lds0 + r[VAH % KN];
+      const uint32_t k_lds = k_lds0 + r[KAH % KN];
       if constexpr (SPT == 2) {
-        // operands: K of tile u+1, the first K operands of tile u+2, V of tile u
-        const uint32_t k_off = RPA_SLOT(1) * HALF, kn_off = RPA_SLOT(2) * HALF, v_off = RPA_SLOT(0) * HALF;
-        uint32_t ka0[NKK], ka1[NKK], kn0[PD], kn1[PD], va0[DB], va1[DB];
-#pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) {
-          ka0[kk] = kaddr[kk] + k_off;
-          ka1[kk] = ka0[kk] + BK * RKL;  // a constant apart: folds into the instruction's offset
-        }
-#pragma unroll
-        for (int o = 0; o < PD; ++o) {
-          kn0[o] = ka1[o];
-          kn1[o] = kaddr[o] + kn_off;
-        }
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          va0[db] = vaddr[db] + v_off;
-          va1[db] = va0[db] + BK * RKL;
-        }
+        constexpr uint32_t PART = BK * RKL;
         const uint32_t dl0[1] = {v_lds}, dl1[1] = {k_lds};
         const char* const dg0[1] = {v_ptr};
         const char* const dg1[1] = {k_ptr};
-        check(pb[PAR0 ^ 1], true);
-        fast_step(std::integral_constant<int, PAR0>{}, ka0, kn0, va0, dl0, voff_v, voff_v, dg0);
+        fast_step(std::integral_constant<int, PAR0>{},
+                  [&](int nx) { return A[nx]; }, [&](int o) { return A[o] + PART; }, [&](int db) { return VA[db]; }, nothing,
+                  dl0, voff_v, voff_v, dg0);
         check(pb[PAR0], true);
-        fast_step(std::integral_constant<int, PAR0 ^ 1>{}, ka1, kn1, va1, dl1, voff_k, voff_k, dg1);
+        fast_step(std::integral_constant<int, PAR0 ^ 1>{},
+                  [&](int nx) { return A[nx] + PART; }, [&](int o) { return A[o]; }, [&](int db) { return VA[db] + PART; }, move_on,
+                  dl1, voff_k, voff_k, dg1);
       } else {
-        // operands: K of tile u+2, the first K operands of tile u+3, V of tile u
-        const uint32_t k_off = RPA_SLOT(2) * HALF, kn_off = RPA_SLOT(3) * HALF, v_off = RPA_SLOT(0) * HALF;
-        uint32_t ka0[NKK], kn0[PD], va0[DB];
-#pragma unroll
-        for (int kk = 0; kk < NKK; ++kk) ka0[kk] = kaddr[kk] + k_off;
-#pragma unroll
-        for (int o = 0; o < PD; ++o) kn0[o] = kaddr[o] + kn_off;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) va0[db] = vaddr[db] + v_off;
         const uint32_t dl0[2] = {v_lds, k_lds};
         const char* const dg0[2] = {v_ptr, k_ptr};
-        check(pb[PAR0 ^ 1], true);
-        fast_step(std::integral_constant<int, PAR0>{}, ka0, kn0, va0, dl0, voff_v, voff_k, dg0);
+        fast_step(std::integral_constant<int, PAR0>{},
+                  [&](int nx) { return A[nx % NKA] + (uint32_t)(256 * (nx / NKA)); }, [&](int o) { return A[o]; },
+                  [&](int db) { return VA[db % NVA] + (uint32_t)(256 * (db / NVA)); }, move_on, dl0, voff_v, voff_k, dg0);
       }
-      ru = ru + 1 == KN ? 0 : ru + 1;
+      const uint32_t r0 = r[0];
+#pragma unroll
+      for (int c = 0; c + 1 < KN; ++c) r[c] = r[c + 1];
+      r[KN - 1] = r0;
     };
-#undef RPA_SLOT
     for (; b < b_fast_hi; b += 2) {
       // No branch between the steps of an iteration: instructions of a pinned step must not find a later block to sink
       // into.  An iteration moves the cursor by at most one column (pages hold two tiles or more).
