@@ -223,6 +223,19 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   const int n_tiles = (kv_hi - kv_lo + TT - 1) / TT;
   const bool single = pt.n_chunks == 1;
 
+  // ---- the page table ------------------------------------------------------------------------------
+  // (Requested ahead of the query rows: the first tile loads wait for it.)
+  // Block-table entries are held 64 columns at a time, one per lane, and picked with v_readlane: the loop then holds no
+  // scalar memory load, whose out-of-order return would turn every wait for an LDS operand into a wait for all of them.
+  const int32_t* bt_row = p.block_tables + (int64_t)i * p.M;
+  int col_base = kv_lo / p.page_size;
+  // (held as the page's offset in the pool in units of 256 bytes: ids clipped and multiplied once per 64 columns here,
+  //  not once per tile in scalar arithmetic; a page is a multiple of 64 rows of 16 bytes or more, the pool is below 2^40 bytes)
+  const uint32_t page_units = (uint32_t)(p.page_stride >> 8);
+  auto page_offsets = [&](int col0) -> uint32_t { return (uint32_t)min(max(bt_row[min(col0 + lane, p.M - 1)], 0), p.P - 1) * page_units; };
+  uint32_t pages_vec = page_offsets(col_base);
+  int cur_col = col_base, cur_off = kv_lo - col_base * p.page_size, cur_tb = kv_lo;
+
   // ---- per row-block lane state --------------------------------------------------------------------
   int row_lo[RB], row_hi[RB];
   bool row_ok[RB];
@@ -252,16 +265,6 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       qf[rb][kk] = v;
     }
   }
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-    for (int kk = 0; kk < NKK; ++kk) {  // waited for here, not inside the loop; kept in the accumulation file from here on
-      u32x4 v = qf[rb][kk];
-#pragma unroll
-      for (int w = 0; w < 4; ++w) v[w] = W::scale_pair(v[w], q_mul);
-      asm volatile("" : "+a"(v));
-      qf[rb][kk] = v;
-    }
   {
     int lo_max = 0, hi_min = 0x7fffffff;
 #pragma unroll
@@ -299,12 +302,6 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     voff_k[u] = roff + (uint32_t)(dma_chunk(u, false) << 4);
     voff_v[u] = roff + (uint32_t)(dma_chunk(u, true) << 4);
   }
-  // Block-table entries are held 64 columns at a time, one per lane, and picked with v_readlane: the loop then holds no
-  // scalar memory load, whose out-of-order return would turn every wait for an LDS operand into a wait for all of them.
-  const int32_t* bt_row = p.block_tables + (int64_t)i * p.M;
-  int col_base = kv_lo / pg;
-  int pages_vec = bt_row[min(col_base + lane, p.M - 1)];
-  int cur_col = col_base, cur_off = kv_lo - col_base * pg, cur_tb = kv_lo;
   // Descriptors of the tiles the cursor was last at, newest first: a tile's V rows are requested DQ tiles behind its K rows.
   struct TileDesc {
     int64_t off;
@@ -318,16 +315,16 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   auto refill_pages = [&](int margin) __attribute__((always_inline)) {
     if (cur_col - col_base >= 64 - margin) {
       col_base = cur_col;
-      pages_vec = bt_row[min(col_base + lane, p.M - 1)];
+      pages_vec = page_offsets(col_base);
       asm volatile("" : "+v"(pages_vec));  // waited for here, once in 64 columns, not at the look-up every tile shares
     }
   };
   auto next_tile = [&](bool refill = true) __attribute__((always_inline)) {  // (also for tiles past the range: the cursor then only counts)
     if (refill) refill_pages(0);
-    const int page = min(max(__builtin_amdgcn_readlane(pages_vec, cur_col - col_base), 0), p.P - 1);
+    const uint64_t page_off = (uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)pages_vec, cur_col - col_base) << 8;
 #pragma unroll
     for (int j = DQ - 1; j > 0; --j) td[j] = td[j - 1];
-    td[0].off = (int64_t)page * p.page_stride + (int64_t)((uint32_t)cur_off * tok_stride);
+    td[0].off = (int64_t)(page_off + (uint32_t)cur_off * tok_stride);
     td[0].edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
     td[0].tb = cur_tb;
     cur_tb += TT;
@@ -722,6 +719,17 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     if (t < n_tiles) issue_half(false, t % KN, td[0]);
     if (t < U0 + VAH && t < n_tiles) issue_half(true, t % KN, td[0]);
   }
+  // The query rows, requested at the top: scaled, and from here on in the accumulation file.
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {  // waited for here, behind the first tile requests and not inside the loop; kept in the accumulation file from here on
+      u32x4 v = qf[rb][kk];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) v[w] = W::scale_pair(v[w], q_mul);
+      asm volatile("" : "+a"(v));
+      qf[rb][kk] = v;
+    }
   auto ring_off = [&](int x) -> uint32_t { return (uint32_t)(((x / SPT) % KN) * HALF + (x % SPT) * BK * RKL); };  // block x >= 0 in its ring
   auto head = [&](int u) __attribute__((always_inline)) {  // barrier u, written plainly
     // in flight may stay the requests of the FLYB barriers before, where they made them in full
@@ -909,6 +917,7 @@ static int launch_x32(hipStream_t stream, const AttnParams& p) {
 // rows); page sizes that are multiples of 64 tokens.
 int prefill_x32_rows(const AttnParams& p) {
   if (p.page_size % 64 != 0 || (int64_t)64 * p.token_stride >= ((int64_t)1 << 31)) return 0;
+  if (p.page_stride % 256 != 0 || (int64_t)p.P * (p.page_stride >> 8) >= ((int64_t)1 << 32)) return 0;  // page offsets are held in units of 256 bytes
   if (p.D == 128 && (p.kv_dtype == RPA_BF16 || p.kv_dtype == RPA_F16) && !(p.softcap > 0.f)) return 256;
   if (p.D == 256 && p.kv_dtype == RPA_BF16) return 128;
   return 0;
