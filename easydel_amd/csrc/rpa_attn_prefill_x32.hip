@@ -864,38 +864,91 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   }
 
   // ---- epilogue -----------------------------------------------------------------------------------------
+  // A lane holds 4-dim pieces of its own row: stored as they are, every store instruction would scatter 16- or 32-byte
+  // pieces over 32 rows.  The rows go through the wave's share of the (now idle) rings instead and leave as whole rows,
+  // 16 bytes per lane over consecutive lanes.  Rows narrower than the padded head (Dq < D) are stored piecewise.
   mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);
+  const bool staged = p.Dq == D;
+  constexpr int RS32 = D * 4 + 16, RS16 = D * 2 + 16;  // row strides of the staging area: 16 bytes of padding spread the rows over the banks
+  static_assert(NW * 32 * RS32 <= 2 * KN * HALF, "the staging areas of the waves fit the rings");
+  const uint32_t stage = lds_base + (uint32_t)wave * (uint32_t)(32 * RS32);
+  if (staged) wait_loads_and_barrier<0>();  // every wave is through with the rings, and no tile is still on its way into them
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const float l_tot = l_acc[rb][0];
-    if (row_ok[rb]) {
-      if (single) {
-        const float l_fin = with_sink(p, out_head[rb], m_ref[rb], l_tot);
-        const float inv = l_fin > 0.f ? 1.f / l_fin : 0.f;
-        uint16_t* orow = (uint16_t*)p.out + ((int64_t)out_tok[rb] * p.Hq + out_head[rb]) * p.Dq + 4 * hh;
+    // where the lane's row goes: its index among the [T][Hq] rows of the output (or of a chunk's partial rows), -1: nowhere
+    const int my_slot = row_ok[rb] ? out_tok[rb] * p.Hq + out_head[rb] : -1;
+    if (single) {
+      const float l_fin = with_sink(p, out_head[rb], m_ref[rb], l_tot);
+      const float inv = l_fin > 0.f ? 1.f / l_fin : 0.f;
+      if (!staged) {
+        if (row_ok[rb]) {
+          uint16_t* orow = (uint16_t*)p.out + (int64_t)my_slot * p.Dq + 4 * hh;
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const f32x16 o = o_acc[rb][db];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {  // registers 4 q4 .. 4 q4 + 3 are dims 32 db + 8 q4 + 4 hh + 0..3
+              const u32x2 w = {H::pack(o[4 * q4] * inv, o[4 * q4 + 1] * inv), H::pack(o[4 * q4 + 2] * inv, o[4 * q4 + 3] * inv)};
+              if (32 * db + 8 * q4 + 4 * hh < p.Dq) *(u32x2*)(orow + 32 * db + 8 * q4) = w;
+            }
+          }
+        }
+      } else {
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const f32x16 o = o_acc[rb][db];
 #pragma unroll
-          for (int q4 = 0; q4 < 4; ++q4) {  // registers 4 q4 .. 4 q4 + 3 are dims 32 db + 8 q4 + 4 hh + 0..3
+          for (int q4 = 0; q4 < 4; ++q4) {
             const u32x2 w = {H::pack(o[4 * q4] * inv, o[4 * q4 + 1] * inv), H::pack(o[4 * q4 + 2] * inv, o[4 * q4 + 3] * inv)};
-            if (32 * db + 8 * q4 + 4 * hh < p.Dq) *(u32x2*)(orow + 32 * db + 8 * q4) = w;
+            *(__attribute__((address_space(3))) u32x2*)(uintptr_t)(stage + (uint32_t)(j32 * RS16 + (32 * db + 8 * q4 + 4 * hh) * 2)) = w;
+          }
+        }
+        constexpr int CPRO = D * 2 / 16, RPIO = 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
+#pragma unroll
+        for (int it = 0; it < 32 / RPIO; ++it) {
+          const int r = it * RPIO + lane / CPRO, c = lane % CPRO;
+          const u32x4 v = *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)(stage + (uint32_t)(r * RS16 + c * 16));
+          const int slot_r = __shfl(my_slot, r);
+          if (slot_r >= 0) *(u32x4*)((char*)p.out + ((int64_t)slot_r * D) * 2 + c * 16) = v;
+        }
+      }
+    } else {
+      const int64_t pbase = (int64_t)chunk * p.T * p.Hq;
+      if (!staged) {
+        if (row_ok[rb]) {
+          float* prow = p.pre_o + (pbase + my_slot) * D + 4 * hh;
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const f32x16 o = o_acc[rb][db];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4)
+              *(f32x4*)(prow + 32 * db + 8 * q4) = (f32x4){o[4 * q4], o[4 * q4 + 1], o[4 * q4 + 2], o[4 * q4 + 3]};
           }
         }
       } else {
-        const int64_t pslot = ((int64_t)chunk * p.T + out_tok[rb]) * p.Hq + out_head[rb];
-        float* prow = p.pre_o + pslot * D + 4 * hh;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
           const f32x16 o = o_acc[rb][db];
 #pragma unroll
           for (int q4 = 0; q4 < 4; ++q4)
-            *(f32x4*)(prow + 32 * db + 8 * q4) = (f32x4){o[4 * q4], o[4 * q4 + 1], o[4 * q4 + 2], o[4 * q4 + 3]};
+            *(__attribute__((address_space(3))) f32x4*)(uintptr_t)(stage + (uint32_t)(j32 * RS32 + (32 * db + 8 * q4 + 4 * hh) * 4)) =
+                (f32x4){o[4 * q4], o[4 * q4 + 1], o[4 * q4 + 2], o[4 * q4 + 3]};
         }
-        if (hh == 0) {
-          p.pre_ml[pslot * 2 + 0] = m_ref[rb];
-          p.pre_ml[pslot * 2 + 1] = l_tot;
+        constexpr int CPRO = D * 4 / 16, RPIO = CPRO >= 64 ? 1 : 64 / CPRO;  // 16-byte chunks per row, rows per store instruction
+        constexpr int IPR = CPRO >= 64 ? CPRO / 64 : 1;                        // store instructions per row where a row is wider than a wave
+#pragma unroll
+        for (int it = 0; it < 32 / RPIO * IPR; ++it) {
+          const int r = IPR > 1 ? it / IPR : it * RPIO + lane / CPRO;
+          const int c = IPR > 1 ? (it % IPR) * 64 + lane : lane % CPRO;
+          const f32x4 v = *(const __attribute__((address_space(3))) f32x4*)(uintptr_t)(stage + (uint32_t)(r * RS32 + c * 16));
+          const int slot_r = __shfl(my_slot, r);
+          if (slot_r >= 0) *(f32x4*)((char*)p.pre_o + ((pbase + slot_r) * D) * 4 + c * 16) = v;
         }
+      }
+      if (row_ok[rb] && hh == 0) {
+        p.pre_ml[(pbase + my_slot) * 2 + 0] = m_ref[rb];
+        p.pre_ml[(pbase + my_slot) * 2 + 1] = l_tot;
       }
     }
   }
