@@ -34,7 +34,8 @@ def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=25,
+                    help="untimed calls ahead of the timed ones (the first twenty or so calls of a workload run a few percent slower than the later ones)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill", "fp8-prefill", "int8-prefill", "gemma-decode",
                              "decode-hkv4", "decode-hkv1", "decode-16seq", "decode-32seq",
                              "mla-decode-h128", "mla-decode-h16", "mla-prefill-h128"])
@@ -48,6 +49,8 @@ def parse_args():
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of a workload: the library's matrix-core feed probe (bf16 MFMA streams with operands from "
                          "registers or LDS, both tile shapes, 1 / 2 / 4 MFMAs per operand, one and two waves per SIMD), one line per setting")
+    ap.add_argument("--issue-probe", action="store_true",
+                    help="what one more instruction of a kind costs a lone wave per SIMD beside a stream of 32x32x16 MFMAs (rpa_issue_probe)")
     ap.add_argument("--cpu-sample-seqs", type=int, default=0, help="sequences in the CPU sample (0 = auto)")
     ap.add_argument("--decode-wgs", type=int, default=0)
     ap.add_argument("--prefill-chunks", type=int, default=0)
@@ -392,6 +395,47 @@ def mfma_probe():
                                       "frac_of_2500": round(tf / MFMA_BF16_PEAK_TFLOPS, 4), "clock_mhz": round(mhz)}), flush=True)
 
 
+def issue_probe():
+    """Cycles per MFMA of a lone wave per SIMD that issues, beside every 32x32x16 bf16 MFMA, six independent v_fma_f32 (a
+    full slot: MFMA 8 cycles of issue + 6 x 4) or none, and 0 / 1 / 2 / 4 instructions of one kind: rpa_issue_probe."""
+    import torch
+
+    from easydel_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    src = torch.ones(1 << 18, dtype=torch.float32, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    kinds = ["v_fma_f32", "v_exp_f32", "v_rcp_f32", "v_cvt_pk_bf16_f32", "v_max3_f32 (dependent chain)", "s_add_u32 (dependent chain)", "s_nop 0",
+             "ds_read_b128", "ds_read_b64_tr_b16", "global_load_lds_dwordx4 (m0 written each time)"]
+    for kind, name in enumerate(kinds):
+        rec = {"probe": "issue", "instruction": name}
+        for fill in (6, 0):
+            cyc = {}
+            for extra in (0, 1, 2, 4):
+                best = None
+                for rep in range(3):
+                    clocks.zero_()
+                    n = lib.rpa_issue_probe(stream.cuda_stream, kind, extra, fill, 1000, clocks.data_ptr(), sink.data_ptr(), src.data_ptr())
+                    if n == 0:
+                        raise RuntimeError(lib.rpa_last_error().decode())
+                    torch.cuda.synchronize()
+                    c = clocks.cpu().numpy()
+                    v = float(c[0]) / (cus * n)
+                    if rep > 0 and (best is None or v < best):
+                        best = v
+                        rec["clock_mhz"] = round(100.0 * float(c[0]) / float(c[1]))
+                cyc[extra] = best
+            key = "full_slot" if fill else "mfma_alone"
+            rec[f"cycles_per_mfma_{key}"] = {str(k): round(v, 1) for k, v in cyc.items()}
+            if fill:
+                rec["cycles_each_in_a_full_slot"] = round((cyc[4] - cyc[0]) / 4.0, 1)
+        print(json.dumps(rec), flush=True)
+
+
 _KEEP = []
 
 
@@ -595,6 +639,8 @@ def main():
         return read_probe_paged()
     if args.mfma_probe:
         return mfma_probe()
+    if args.issue_probe:
+        return issue_probe()
     if args.workload.startswith("mla-"):
         if args.mla_chunks:
             _lib.set_tunable("mla_chunks", args.mla_chunks)

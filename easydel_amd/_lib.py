@@ -61,6 +61,7 @@ PROBE_SIGNATURES = {
     "rpa_read_probe": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_vp]),
     "rpa_read_probe_paged": (_c_sz, [_c_vp, _c_vp, _c_sz, _c_int, _c_int, _c_int, _c_int, _c_vp]),
     "rpa_mfma_probe": (ctypes.c_double, [_c_vp, _c_int, _c_int, _c_int, _c_int, _c_int, _c_vp, _c_vp]),
+    "rpa_issue_probe": (ctypes.c_longlong, [_c_vp, _c_int, _c_int, _c_int, _c_int, _c_vp, _c_vp, _c_vp]),
 }
 
 

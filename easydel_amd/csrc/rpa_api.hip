@@ -21,6 +21,7 @@ int launch_calibration_copy(hipStream_t, void*, const void*, size_t);
 size_t launch_read_probe(hipStream_t, const void*, size_t, int, int, uint32_t*);
 size_t launch_read_probe_paged(hipStream_t, const void*, size_t, int, int, int, int, uint32_t*);
 double launch_mfma_probe(hipStream_t, int, int, int, int, int, unsigned long long*, float*);
+long long launch_issue_probe(hipStream_t, int, int, int, int, unsigned long long*, float*, const void*);
 #endif
 int launch_scatter_ragged_quant(hipStream_t, const void*, const void*, void*, float*, const int32_t*, const int32_t*,
                                 const int32_t*, const int32_t*, int, int, int, int, int, int, int, int, int, int, int);
@@ -245,6 +246,16 @@ double rpa_mfma_probe(rpa_stream_t stream, int shape, int source, int mfmas_per_
   if (flops == 0.0)
     fail(RPA_ERR_INVALID_ARGUMENT, "rpa_mfma_probe: shape 0 / 1, source 0..2, 1 / 2 / 4 MFMAs per operand, 1 or 2 waves per SIMD, iters > 0");
   return flops;
+}
+
+long long rpa_issue_probe(rpa_stream_t stream, int kind, int extra, int fill, int iters, void* clocks, void* sink, const void* src) {
+  if (!clocks || !sink || !src || ((uintptr_t)clocks & 7) || ((uintptr_t)sink & 3) || ((uintptr_t)src & 15)) {
+    fail(RPA_ERR_INVALID_ARGUMENT, "rpa_issue_probe: clocks must be two 8-byte device words, sink a 4-byte device word, src 1 MiB of 16-byte aligned device memory");
+    return 0;
+  }
+  const long long n = rpa::launch_issue_probe((hipStream_t)stream, kind, extra, fill, iters, (unsigned long long*)clocks, (float*)sink, src);
+  if (n == 0) fail(RPA_ERR_INVALID_ARGUMENT, "rpa_issue_probe: kind 0..9, extra 0 / 1 / 2 / 4, fill 0 or 6, iters > 0");
+  return n;
 }
 #endif  // RPA_PROBES
 

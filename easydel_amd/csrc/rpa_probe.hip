@@ -270,4 +270,111 @@ double launch_mfma_probe(hipStream_t stream, int shape, int source, int reuse, i
   return 0.0;
 }
 
+// Issue cost of one instruction kind beside a stream of 32x32x16 bf16 MFMAs on a lone wave per SIMD (how the 32x32 prefill
+// kernel runs): every MFMA is followed by FILL independent v_fma_f32 and NX instructions of kind KIND.  An MFMA holds the
+// matrix pipe for 32 cycles and the issue port for 8; what a slot's other instructions take beyond the remaining 24
+// shows as cycles per MFMA above 32.
+// KIND: 0 v_fma_f32, 1 v_exp_f32, 2 v_rcp_f32, 3 v_cvt_pk_bf16_f32, 4 v_max3_f32 (a dependent chain), 5 s_add_u32 (a
+// dependent chain), 6 s_nop 0, 7 ds_read_b128, 8 ds_read_b64_tr_b16, 9 global_load_lds_dwordx4 (1 KiB, m0 written each time).
+template <int KIND, int NX, int FILL>
+__global__ __launch_bounds__(256) void issue_probe_kernel(int iters, unsigned long long* clocks, float* sink, const char* src) {
+  __shared__ mp_u32x4 lds[2048];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < 2048; i += 256) lds[i] = (mp_u32x4){(uint32_t)i, 1u, 2u, 3u};
+  __syncthreads();
+  typedef MpAcc<1>::T acc_t;
+  acc_t acc[2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[a][j] = 0.f;
+  const mp_u32x4 A = {0x3f803f00u + lane, 0x3f003f80u, 0xbf803f80u, 0x3f80bf00u}, B = {0x3f803f80u, 0x3f003f00u + lane, 0xbf80bf80u, 0x3f803f00u};
+  float x[8], y[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    x[i] = lane * 0.001f + i;
+    y[i] = 0.5f + lane * 0.01f;
+  }
+  uint32_t sc = blockIdx.x, pk = 0;
+  float mx = 0.f;
+  mp_u32x4 rd[8];
+  mp_u32x2 rt[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    rd[i] = (mp_u32x4){0u, 0u, 0u, 0u};
+    rt[i] = (mp_u32x2){0u, 0u};
+  }
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) mp_u32x4*)lds;
+  const uint32_t la = lds0 + (uint32_t)lane * 16;
+  const uint32_t lb = lds0 + (uint32_t)((lane >> 4) * 512 + (lane & 15) * 8);
+  const uint32_t ldst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(1024 + wave * 64) * 16);  // the wave's 1 KiB landing area
+  const uint32_t voff = (uint32_t)lane * 16;
+  const uint64_t g = (uint64_t)(src + (size_t)((blockIdx.x * 4 + wave) & 255) * 4096);  // 1 KiB of a 1 MiB buffer per wave
+  const char* gbase = (const char*)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(g >> 32)) << 32) |
+                                    (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)g));
+  const unsigned long long t0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      acc[i % 2] = mp_mfma<1>(A, B, acc[i % 2]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int f = 0; f < FILL; ++f) {
+        const int q = (i * FILL + f) % 8;
+        x[q] = __builtin_fmaf(x[q], 1.0001f, 0.5f);
+        asm volatile("" : "+v"(x[q]));
+      }
+#pragma unroll
+      for (int f = 0; f < NX; ++f) {
+        const int q = (i * NX + f) % 8;
+        if constexpr (KIND == 0) asm volatile("v_fma_f32 %0, %0, %1, 0.5" : "+v"(y[q]) : "v"(x[7 - q]));
+        else if constexpr (KIND == 1) asm volatile("v_exp_f32 %0, %0" : "+v"(y[q]));
+        else if constexpr (KIND == 2) asm volatile("v_rcp_f32 %0, %0" : "+v"(y[q]));
+        else if constexpr (KIND == 3) asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(pk) : "v"(y[q]), "v"(y[(q + 1) % 8]));
+        else if constexpr (KIND == 4) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(mx) : "v"(y[q]), "v"(y[(q + 1) % 8]));
+        else if constexpr (KIND == 5) asm volatile("s_add_u32 %0, %0, 7" : "+s"(sc) : : "scc");
+        else if constexpr (KIND == 6) asm volatile("s_nop 0");
+        else if constexpr (KIND == 7) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(rd[q]) : "v"(la), "n"(1024 * (q % 8)));
+        else if constexpr (KIND == 8) asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(rt[q]) : "v"(lb), "n"(2048 * (q % 8)));
+        else asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(ldst), "v"(voff), "s"(gbase) : "memory");
+      }
+      if constexpr ((KIND == 7 || KIND == 8) && NX > 0) asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(NX >= 4 ? 4 : NX) : "memory");
+      if constexpr (KIND == 9 && NX > 0) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  const unsigned long long t1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  float r = (float)sc + __uint_as_float(pk) + mx;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r += x[i] + y[i] + __uint_as_float(rd[i][0] & 1u) + __uint_as_float(rt[i][0] & 1u);
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) r += acc[a][j];
+  if (r == 12345.678f) sink[0] = r + __uint_as_float(lds[1024 + lane][0]);
+  if (threadIdx.x == 0) {
+    atomicAdd(clocks, t1 - t0);
+    atomicAdd(clocks + 1, w1 - w0);
+  }
+}
+
+// Returns the MFMAs every wave issues (0: bad arguments).  clocks as for launch_mfma_probe; src: 1 MiB of device memory.
+long long launch_issue_probe(hipStream_t stream, int kind, int extra, int fill, int iters, unsigned long long* clocks, float* sink,
+                             const void* src) {
+  if (iters <= 0) return 0;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) return 0;
+#define RPA_IP(K, X, F)                                                                                              \
+  if (kind == K && extra == X && fill == F) {                                                                        \
+    hipLaunchKernelGGL((issue_probe_kernel<K, X, F>), dim3(cus), dim3(256), 0, stream, iters, clocks, sink, (const char*)src); \
+    return hipGetLastError() == hipSuccess ? 16ll * iters : 0;                                                       \
+  }
+#define RPA_IP4(K) RPA_IP(K, 0, 0) RPA_IP(K, 1, 0) RPA_IP(K, 2, 0) RPA_IP(K, 4, 0) RPA_IP(K, 0, 6) RPA_IP(K, 1, 6) RPA_IP(K, 2, 6) RPA_IP(K, 4, 6)
+  RPA_IP4(0) RPA_IP4(1) RPA_IP4(2) RPA_IP4(3) RPA_IP4(4) RPA_IP4(5) RPA_IP4(6) RPA_IP4(7) RPA_IP4(8) RPA_IP4(9)
+#undef RPA_IP4
+#undef RPA_IP
+  return 0;
+}
+
 }  // namespace rpa

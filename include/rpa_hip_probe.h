@@ -63,6 +63,20 @@ double rpa_mfma_probe(rpa_stream_t stream, int shape, int source, int mfmas_per_
                       void* clocks, void* sink);
 
 /*
+ * Measurement aid with no counterpart in the reference: what one more instruction costs a lone wavefront per SIMD that
+ * streams 32x32x16 bf16 MFMAs (how the 32x32 prefill kernel runs).  One workgroup of four wavefronts per CU; every
+ * wavefront issues 16 * iters MFMAs, each followed by `fill` (0 or 6) independent v_fma_f32 and `extra` (0, 1, 2 or 4)
+ * instructions of `kind`: 0 v_fma_f32, 1 v_exp_f32, 2 v_rcp_f32, 3 v_cvt_pk_bf16_f32, 4 v_max3_f32 (a dependent chain),
+ * 5 s_add_u32 (a dependent chain), 6 s_nop, 7 ds_read_b128, 8 ds_read_b64_tr_b16, 9 global_load_lds_dwordx4 (1 KiB per
+ * instruction, m0 written each time).  An MFMA holds the matrix pipe for 32 cycles and the issue port for 8: with
+ * fill = 6 the slot is full, and the cycles per MFMA above that say what an instruction of `kind` costs.  Returns the
+ * MFMAs per wavefront (0 on bad arguments).  `clocks` and `sink` as for rpa_mfma_probe: clocks[0] / (workgroups *
+ * MFMAs per wavefront) is the cycles per MFMA.  `src`: 1 MiB of initialised device memory, 16-byte aligned (read by
+ * kind 9 only).
+ */
+long long rpa_issue_probe(rpa_stream_t stream, int kind, int extra, int fill, int iters, void* clocks, void* sink, const void* src);
+
+/*
  * Knobs for tests and measurement.  They belong to the calling thread: a value set here is seen only by entry points
  * the same thread calls afterwards (each call reads them once, when it starts), so threads that never call this function
  * always run with the defaults.  Returns the previous value, -1 for an unknown name.

@@ -94,6 +94,9 @@ def test_host_only_entry_points():
     assert _lib.set_tunable("no_such_knob", 1) == -1
     assert lib.rpa_mfma_probe(None, 1, 1, 2, 1, 100, None, None) == 0.0 and b"rpa_mfma_probe" in lib.rpa_last_error()
     assert lib.rpa_mfma_probe(None, 1, 1, 3, 1, 100, a, a) == 0.0  # 1, 2 or 4 MFMAs per operand
+    assert lib.rpa_issue_probe(None, 1, 1, 6, 100, None, None, None) == 0 and b"rpa_issue_probe" in lib.rpa_last_error()
+    assert lib.rpa_issue_probe(None, 1, 3, 6, 100, a, a, a) == 0  # 0, 1, 2 or 4 instructions beside the MFMA
+    assert lib.rpa_issue_probe(None, 10, 1, 6, 100, a, a, a) == 0  # kinds 0..9
 
 
 def test_product_build_has_no_probes_and_no_stage_knob(tmp_path):
