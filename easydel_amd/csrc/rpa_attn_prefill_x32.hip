@@ -145,8 +145,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   constexpr int U0 = -2 / SPT;           // the first barrier (step -2)
   static_assert(2 * KN * HALF <= 160 * 1024 && FLYB >= 1 && DQ >= 1 && 2 * FLYB * NLH <= 48, "ring sizes");
   constexpr int NQ = NKK * RB;           // MFMA slots of the score phase
-  constexpr int NBIAS = CAP ? 0 : RB;    // MFMA slots that put the rows' reference into the scores (see below; not with a soft cap)
-  constexpr int NSUM = 2 * RB + NBIAS;   // MFMA slots between the two products: those, and the row sums (ones x P^T, per row block and 16-key half)
+  constexpr int NSUM = 2 * RB;           // MFMA slots of the row sums (ones x P^T, per row block and 16-key half)
   constexpr int NP = NVO * RB;           // MFMA slots of the PV phase
   constexpr int PD = 4;                  // operands read ahead
   constexpr int NPAIR = RB * 8;          // pairs of probabilities per lane and block
@@ -242,10 +241,6 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   int out_tok[RB], out_head[RB];
   u32x4 qf[RB][NKK];
   int wave_lo, wave_hi;          // keys every row of the wave sees: [max row_lo, min row_hi)
-  // The queries are scaled once, here, and rounded back to 16 bits: the scores then leave the MFMAs in the units the
-  // exponentials take (log2 units; with a soft cap: 2 log2(e) / cap times the scaled score, the argument of the cap's
-  // exponential), and no multiplication per score is left.  (The rounding moves a score by 2^-9 of its terms at most.)
-  const float q_mul = CAP ? (p.scale / p.softcap) * 2.8853900817779268f : p.scale_log2;
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int row = R0 + (wave * RB + rb) * 32 + j32;
@@ -355,25 +350,14 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   f32x16 o_acc[RB][DB];        // O^T: lane = row j32, register r = dim 8 (r / 4) + 4 hh + r % 4 of the 32-dim block
   f32x16 l_acc[RB];            // row sums, from the matrix cores: every register of lane j32 holds the sum of row j32
   float m_ref[RB], lmx[RB];
-  // Without a soft cap the scores carry their row's reference from the start: block b+2's S^T accumulators receive
-  // -m_ref through one more MFMA (the tile of ones against bias_b, whose first two k entries hold -m_ref in two 16-bit
-  // parts and whose others are zero), the plain steps add it with the vector ALU, and a probability is exp2 of what
-  // the softmax finds in the registers.  m_neg is what the scores carry: -m_ref exactly (0 while m_ref is -inf).
-  // With a soft cap the scores stay bare and m_neg = cap - m_ref enters behind the cap.
-  float m_neg[RB];
-  float thr[RB];               // what a block's row maximum (as the scores carry it) is compared with: slack above the reference
-  u32x4 bias_b[RB];            // B operand of the reference MFMA
+  float m_neg[RB];             // what is added to a scaled score ahead of the exponential: -m_ref (with a soft cap: cap - m_ref)
+  float thr[RB];               // (m_ref + slack) in units of the raw scores: what a block's maximum is compared with
   u32x4 ops[PD];               // operands read ahead of their MFMAs
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     m_ref[rb] = -INFINITY;
     thr[rb] = -INFINITY;
     m_neg[rb] = 0.f;
-    {
-      u32x4 z = {0u, 0u, 0u, 0u};
-      asm volatile("" : "+a"(z));
-      bias_b[rb] = z;
-    }
     {
       f32x16 z;
 #pragma unroll
@@ -391,17 +375,24 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       o_acc[rb][db] = z;
     }
   }
-  // With a soft cap the capped score in log2 units is cap_out tanh(x) = cap_out (1 - 2 / (exp2(y) + 1)) with y = 2 log2(e) x
-  // what the MFMAs deliver, so the probability is exp2(r cap_m2 + m_neg) with r = 1 / (exp2(y) + 1).
+  // Without a soft cap a probability is exp2(s sc_mul + m_neg).  With one, the capped score in log2 units is
+  // cap_out tanh(s cap_in) = cap_out (1 - 2 / (exp2(s cap_in2) + 1)), so the probability is exp2(r cap_m2 + m_neg) with
+  // r = 1 / (exp2(s cap_in2) + 1) and m_neg = cap_out - m_ref.  (The multiplication per score stays: queries scaled
+  // ahead of the MFMAs and rounded back to 16 bits would save it, and move a score by 2^-9 of its terms -- measured at
+  // four times the usual spread of scores: 3e-2 instead of 1.5e-2 max-abs against the oracle.)
+  const float sc_mul = p.scale_log2;
+  const float inv_sc = 1.f / sc_mul;
   const float cap_out = CAP ? p.softcap * 1.4426950408889634f : 0.f;
+  const float cap_in = CAP ? p.scale / p.softcap : 0.f;
+  const float cap_in2 = cap_in * 2.8853900817779268f;
   const float cap_m2 = -2.f * cap_out;
-  auto capped = [&](float y) -> float { return __builtin_fmaf(__builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(y) + 1.f), cap_m2, cap_out); };  // to log2 units
+  auto capped = [&](float s) -> float { return cap_out * fast_tanh(s * cap_in); };  // a raw score to log2 units
   auto prob = [&](float s, float mn) __attribute__((always_inline)) -> float {
     if constexpr (CAP) {
-      const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s) + 1.f);
+      const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s * cap_in2) + 1.f);
       return s == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(r, cap_m2, mn));  // a masked key is not the cap's lower end
     } else {
-      return __builtin_amdgcn_exp2f(s);
+      return __builtin_amdgcn_exp2f(__builtin_fmaf(s, sc_mul, mn));
     }
   };
   // The A operand of the row sums: ones, written to registers once, here.  (Left to the compiler it is rebuilt from
@@ -433,10 +424,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     return (u32x4){lo[0], lo[1], hi[0], hi[1]};
   };
 
-  // Raises the references of the rows whose new scores (maxima in lmx, as the scores carry them) exceed them by more than
-  // the slack; what has been accumulated, and the pending probabilities pend (relative to the old reference), are scaled
-  // to match, and without a soft cap the scores s_pend that await their softmax are moved to the new reference.
-  auto check = [&](u32x4 (&pend)[RB][2], f32x16 (&s_pend)[RB], bool has_pending) __attribute__((always_inline)) {
+  // Raises the references of the rows whose new scores (maxima in lmx, raw) exceed them by more than the slack; what
+  // has been accumulated, and the pending probabilities pend (relative to the old reference), are scaled to match.
+  auto check = [&](u32x4 (&pend)[RB][2], bool has_pending) __attribute__((always_inline)) {
     bool grow = false;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) grow |= lmx[rb] > thr[rb];
@@ -445,30 +435,18 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const float raw = xor32_max(lmx[rb]);
-        const float mx = raw == -INFINITY ? -INFINITY : (CAP ? capped(raw) : raw - m_neg[rb]);  // in log2 units, bare
-        float m_new = fmaxf(m_ref[rb], ceilf(mx));
-        if constexpr (CAP) {  // the MFMA output whose capped value is m_new + slack, if there is one
-          const float y = (m_new + kMaxSlack) / cap_out;
-          thr[rb] = (m_new == -INFINITY) ? -INFINITY : (y >= 0.999f ? INFINITY : __log2f((1.f + y) / (1.f - y)));
-          m_neg[rb] = (m_new == -INFINITY) ? 0.f : cap_out - m_new;
-        } else if (m_new != -INFINITY) {
-          // the reference as two 16-bit numbers: whole numbers below 2^16 exactly, so that alpha stays a power of two
-          const uint32_t w_hi = H::pack(-m_new, 0.f);
-          const float hi = W::lo_half(w_hi);
-          const uint32_t w = H::pack(hi, -m_new - hi);
-          const float mn = hi + W::hi_half(w);
-          m_new = -mn;
-          const float d = mn - m_neg[rb];  // what the scores that carry the old reference are moved by
-#pragma unroll
-          for (int r = 0; r < 16; ++r) s_pend[rb][r] += d;
-          m_neg[rb] = mn;
-          thr[rb] = kMaxSlack;
-          u32x4 bb = {hh == 0 ? w : 0u, 0u, 0u, 0u};
-          asm volatile("" : "+a"(bb));
-          bias_b[rb] = bb;
-        }
+        const float mx = CAP ? (raw == -INFINITY ? -INFINITY : capped(raw)) : raw * sc_mul;
+        const float m_new = fmaxf(m_ref[rb], ceilf(mx));
         float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref[rb] - m_new);  // a power of two, or 0
         m_ref[rb] = m_new;
+        if constexpr (CAP) {  // the raw score whose capped value is m_new + slack, if there is one
+          const float y = (m_new + kMaxSlack) / cap_out;
+          thr[rb] = (m_new == -INFINITY) ? -INFINITY : (y >= 0.999f ? INFINITY : 0.5f * __logf((1.f + y) / (1.f - y)) / cap_in);
+          m_neg[rb] = (m_new == -INFINITY) ? 0.f : cap_out - m_new;
+        } else {
+          thr[rb] = (m_new + kMaxSlack) * inv_sc;
+          m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
+        }
         asm volatile("s_nop 1" : "+v"(alpha));
         {
           f32x16 l = l_acc[rb];
@@ -532,13 +510,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           else ops[g % PD] = rv(nx - NKK);
         }
       } else if constexpr (PH == 1) {
-        const int e = k - NQ;
-        if (e < NBIAS) {
-          W::mfma_s(s_nxt[e], ones, bias_b[e]);  // S(b+2) of row block e receives -m_ref: the sum over k of 1 x bias_b
-        } else {
-          const int rb = (e - NBIAS) % RB, sh = (e - NBIAS) / RB;
-          W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
-        }
+        const int e = k - NQ, rb = e % RB, sh = e / RB;
+        W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
         // These slots carry no softmax and no operand read: the step's tile loads are requested from here on, where the
         // time the load unit takes to accept 1 KiB of addresses hides behind an MFMA.
         if (NDI <= NSUM && e < NDI) dma(e);
@@ -563,23 +536,28 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         const int srb = ip / 8, sr2 = ip % 8;
         const int jp = ip - 1, prb = jp / 8, pr2 = jp % 8;  // the pair before
         if constexpr (!CAP) {
-          // the scores carry the reference: the pair before is packed, then one exponential in each half of the pair's slots
+          // first the scaled differences of the pair, and the pair before packed (behind the two multiply-adds: they are
+          // the distance an exponential wants from its reader); half the pair's slots on, the exponentials
           if (st == 0) {
+            xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
+            xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc_mul, m_neg[srb]);
             if (ip > 0) p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
-            ea = __builtin_amdgcn_exp2f(s_cur[srb][2 * sr2]);
           } else if (st == SPP / 2) {
-            eb = __builtin_amdgcn_exp2f(s_cur[srb][2 * sr2 + 1]);
+            ea = __builtin_amdgcn_exp2f(xa);
+            eb = __builtin_amdgcn_exp2f(xb);
           }
         } else {
           // four stages, one slot each; the last exponentials and the packing of a pair ride on the first two slots of the next
           if (st == 0) {
+            xa = s_cur[srb][2 * sr2] * cap_in2;
+            xb = s_cur[srb][2 * sr2 + 1] * cap_in2;
             if (ip > 0) {
               fa = __builtin_amdgcn_exp2f(ea);
               fb = __builtin_amdgcn_exp2f(eb);
             }
           } else if (st == 1) {
-            xa = __builtin_amdgcn_exp2f(s_cur[srb][2 * sr2]);
-            xb = __builtin_amdgcn_exp2f(s_cur[srb][2 * sr2 + 1]);
+            xa = __builtin_amdgcn_exp2f(xa);
+            xb = __builtin_amdgcn_exp2f(xb);
             if (ip > 0) p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(fa, fb);
           } else if (st == 2) {
             xa += 1.f;
@@ -692,10 +670,6 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           if (!plain) {
             const int c = 8 * (r / 4) + (r % 4);
             sv = ((uint32_t)(c - lo_rel) < span) ? sv : -INFINITY;
-            if constexpr (CAP) s_nxt[rb][r] = sv;
-          }
-          if constexpr (!CAP) {  // what the pinned step's reference MFMA does
-            sv += m_neg[rb];
             s_nxt[rb][r] = sv;
           }
           mx = fmaxf(mx, sv);
@@ -719,14 +693,12 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     if (t < n_tiles) issue_half(false, t % KN, td[0]);
     if (t < U0 + VAH && t < n_tiles) issue_half(true, t % KN, td[0]);
   }
-  // The query rows, requested at the top: scaled, and from here on in the accumulation file.
+  // The query rows, requested at the top: from here on in the accumulation file.
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int kk = 0; kk < NKK; ++kk) {  // waited for here, behind the first tile requests and not inside the loop; kept in the accumulation file from here on
       u32x4 v = qf[rb][kk];
-#pragma unroll
-      for (int w = 0; w < 4; ++w) v[w] = W::scale_pair(v[w], q_mul);
       asm volatile("" : "+a"(v));
       qf[rb][kk] = v;
     }
@@ -745,7 +717,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     const bool do_qk = b + 2 < n_blocks, do_sm = b + 1 >= 0 && b + 1 < n_blocks, do_pv = b >= 0 && b < n_blocks;
     const bool next_k = b + 3 < n_blocks, first = b == -2;
     constexpr int PAR = decltype(par_tag)::value;
-    if (do_sm) check(pb[PAR ^ 1], sa[PAR], do_pv);
+    if (do_sm) check(pb[PAR ^ 1], do_pv);
     slow_step(par_tag, ring_off(b + 2), ring_off(b + 3), ring_off(max(b, 0)), do_qk, do_sm, do_pv, next_k, first, kv_lo + (b + 2) * BK);
   };
   // Pairs of steps (b, b + 1), b even, the pinned code may serve: b >= 0, the barriers whose requests may be in flight
@@ -814,7 +786,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       constexpr int PAR0 = decltype(par_tag)::value;
       // visible now: K tiles up to u + KNO, V tiles up to u; in flight stay the requests of the FLYB barriers before
       wait_loads_and_barrier<2 * FLYB * NLH>();
-      check(pb[PAR0 ^ 1], sa[PAR0], true);
+      check(pb[PAR0 ^ 1], true);
       // this barrier's requests, made from inside its steps: V(u + VAH), described DQ tiles ago, and K(u + KAH)
       const char* v_ptr = v_base + td[DQ - 1].off;
       next_tile(false);
@@ -829,7 +801,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         fast_step(std::integral_constant<int, PAR0>{},
                   [&](int nx) { return A[nx]; }, [&](int o) { return A[o] + PART; }, [&](int db) { return VA[db]; }, nothing,
                   dl0, voff_v, voff_v, dg0);
-        check(pb[PAR0], sa[PAR0 ^ 1], true);
+        check(pb[PAR0], true);
         fast_step(std::integral_constant<int, PAR0 ^ 1>{},
                   [&](int nx) { return A[nx] + PART; }, [&](int o) { return A[o]; }, [&](int db) { return VA[db] + PART; }, move_on,
                   dl1, voff_k, voff_k, dg1);

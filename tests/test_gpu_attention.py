@@ -327,6 +327,19 @@ def test_prefill_kernel_on_32x32_tiles(gpu, D, page_size, Hq, Hkv, cap, window):
     assert np.array_equal(again[rows], wide[rows]), "two runs of the same call must agree bit for bit"
 
 
+@pytest.mark.parametrize("D,page_size,Hq,Hkv,cap", [(128, 64, 32, 8, None), (256, 128, 16, 8, 50.0)])
+@pytest.mark.parametrize("spread", [4, 16])
+def test_prefill_holds_the_tolerance_on_peaked_scores(gpu, D, page_size, Hq, Hkv, cap, spread):
+    # Scores with `spread` times the usual spread (sharply peaked rows, as trained heads produce them): an error in a score is
+    # an error in the exponent of its weight, so whatever a kernel does to its queries ahead of the MFMAs shows here first.
+    # (Queries scaled by the softmax scale and rounded back to bf16 read 3e-2 at spread 4 and 1.3e-1 at 16.)
+    b = tl.make_batch(7 + D, [2100, 1500, 700], [640, 300, 700], Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, max_pages=-(-2100 // page_size))
+    kw = dict(softmax_scale=spread * D ** -0.5, logits_soft_cap=cap)
+    got = tl.run_gpu_attention(b, **kw)
+    mx, mean = tl.assert_close(got, tl.oracle_out(b, **kw), b, f"peaked scores D{D} spread {spread}")
+    print(f"peaked scores D{D} spread {spread}: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+
+
 def test_chunked_prefill_equals_rows_of_single_shot_prefill(gpu):
     # the same keys, queried as one 384-token prefill and as its last 128-token chunk
     b_full = tl.make_batch(53, [384], [384], Hq=32, Hkv=8, D=128, page_size=64)
