@@ -340,6 +340,15 @@ def test_prefill_holds_the_tolerance_on_peaked_scores(gpu, D, page_size, Hq, Hkv
     print(f"peaked scores D{D} spread {spread}: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
 
 
+@pytest.mark.parametrize("spread", [4, 16])
+def test_decode_holds_the_tolerance_on_peaked_scores(gpu, spread):
+    # the same for decode rows (the split-K decode kernel and the merge), with and without a soft cap
+    for D, page_size, Hq, Hkv, cap in ((128, 64, 32, 8, None), (256, 128, 16, 8, 50.0)):
+        b = tl.make_batch(11, [2100, 1500, 700, 4000, 33], [1, 1, 1, 1, 1], Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, max_pages=-(-4000 // page_size))
+        kw = dict(softmax_scale=spread * D ** -0.5, logits_soft_cap=cap)
+        tl.assert_close(tl.run_gpu_attention(b, **kw), tl.oracle_out(b, **kw), b, f"peaked scores, decode D{D} spread {spread}")
+
+
 def test_chunked_prefill_equals_rows_of_single_shot_prefill(gpu):
     # the same keys, queried as one 384-token prefill and as its last 128-token chunk
     b_full = tl.make_batch(53, [384], [384], Hq=32, Hkv=8, D=128, page_size=64)
