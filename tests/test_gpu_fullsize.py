@@ -183,6 +183,24 @@ def test_config5_gemma_long_context_first_sequence(gpu, windowed):
     print(f"C5 windowed={windowed}: worst max-abs {worst:.3e}", flush=True)
 
 
+def test_long_context_prefill_over_eight_rounds_of_row_tiles(gpu):
+    # 8 sequences of 2 048 prefill tokens at 10k-31k context, Llama-3-8B heads: 256 row tiles of the 32x32 kernel, eight
+    # rounds over the chip, every other of which the kernel walks backwards -- a slice of rows from every sequence
+    w = workloads.llama_long_prefill(seed=0)
+    tens = workloads.device_tensors(w, gpu, seed=0)
+    out = kernels.ragged_paged_attention(tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"],
+                                         tens["query_start_loc"], tens["num_seqs"], softmax_scale=w.softmax_scale, num_kv_heads=w.Hkv)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    worst = 0.0
+    for i in range(len(w.q_lens)):
+        r0 = (0, 2032, 992, 64, 1500, 2000, 448, 1216)[i % 8]
+        e = _oracle_on_rows(w, tens, i, r0, r0 + 16, out)
+        print(f"  long prefill: sequence {i} (ctx {int(w.context_lens[i])}) tokens [{r0}, {r0 + 16}): max-abs {e:.3e}", flush=True)
+        worst = max(worst, e)
+    print(f"long-context prefill: worst max-abs {worst:.3e}", flush=True)
+
+
 @pytest.mark.parametrize("Hq", [128, 16])
 def test_multi_latent_decode_at_benchmark_size(gpu, Hq):
     """256 sequences of 512..8192 tokens over latent pages (512 + 64, bf16), one new token each: the fused write is in
