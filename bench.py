@@ -58,6 +58,7 @@ def parse_args():
     ap.add_argument("--decode-dma", type=int, default=-1, help="LDS-direct decode kernel: -1 the library's choice, 0 never, 1 wherever built")
     ap.add_argument("--max-splits", type=int, default=0)
     ap.add_argument("--prefill-x32", type=int, default=-1, help="32x32-tile prefill kernel: -1 the library's choice, 0 never")
+    ap.add_argument("--prefill-wide", type=int, default=-1, help="bf16 copies of 8-bit pages for the 32x32-tile prefill kernel: -1 the library's choice, 0 never")
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
     ap.add_argument("--mla-uniform-context", type=int, default=0,
@@ -106,7 +107,7 @@ def build_workload(name, seed, sequential=False):
 
 KERNEL_SOURCES = {  # the files a kernel is compiled from: a counter run is only valid for the sources it was taken on
     "attn_decode_kernel": ("rpa_attn_decode.hip", "rpa_attn_decode_dma.h", "rpa_mfma.h", "rpa_common.h"),
-    "attn_prefill_kernel": ("rpa_attn_prefill_x32.hip", "rpa_attn_prefill_dma.hip", "rpa_attn_prefill_dma8.hip", "rpa_attn_prefill.hip", "rpa_mfma.h", "rpa_common.h"),
+    "attn_prefill_kernel": ("rpa_attn_prefill_x32.hip", "rpa_attn_prefill_dma.hip", "rpa_attn_prefill_dma8.hip", "rpa_attn_prefill.hip", "rpa_widen.hip", "rpa_mfma.h", "rpa_common.h"),
 }
 
 
@@ -659,6 +660,8 @@ def main():
         _lib.set_tunable("max_splits", args.max_splits)
     if args.prefill_x32 >= 0:
         _lib.set_tunable("prefill_x32", args.prefill_x32)
+    if args.prefill_wide >= 0:
+        _lib.set_tunable("prefill_wide", args.prefill_wide)
 
     result = measure(args, args.workload, True)
     if args.workload == "c2" and args.layout == "interleaved" and not args.no_extra_configs:

@@ -27,6 +27,7 @@ SOURCES = [
     "rpa_attn_prefill_dma.hip",
     "rpa_attn_prefill_dma8.hip",
     "rpa_attn_prefill_x32.hip",
+    "rpa_widen.hip",
     "rpa_attn_merge.hip",
     "rpa_mla.hip",
 ]

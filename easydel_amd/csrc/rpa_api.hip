@@ -44,6 +44,7 @@ struct Tunables {
   int force_generic = 0;
   int prefill_dma = 1;
   int prefill_x32 = 1;     // 1: the 32x32-tile prefill kernel serves the shapes it is built for
+  int prefill_wide = 1;    // 1: 8-bit pages reach that kernel through bf16 copies where the workspace has room and the batch's rows pay for them
   int decode_pace = 1;
   int decode_dma = -1;     // -1: where it measured faster (head size 256; int8 pages); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
   int mla_chunks = 0;      // 0 = sized from the shapes
@@ -194,6 +195,7 @@ int rpa_set_tunable(const char* name, int value) {
 #endif
   if (!strcmp(name, "prefill_dma")) return swap(g_tun.prefill_dma, value != 0);
   if (!strcmp(name, "prefill_x32")) return swap(g_tun.prefill_x32, value != 0);
+  if (!strcmp(name, "prefill_wide")) return swap(g_tun.prefill_wide, value != 0);
   if (!strcmp(name, "decode_pace")) return swap(g_tun.decode_pace, value != 0);
   if (!strcmp(name, "decode_dma")) return swap(g_tun.decode_dma, value < 0 ? -1 : value > 3 ? 3 : value);
   if (!strcmp(name, "mla_min_chunk")) return swap(g_tun.mla_min_chunk, value <= 0 ? 0 : ((value + 63) & ~63));
@@ -323,6 +325,23 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
                   "rpa_page_scatter_ragged_quantised launch");
 }
 
+// bf16 copies of 8-bit pages for the 32x32-tile prefill kernel (rpa_widen.hip): the pages the workspace is asked to
+// hold, from the static bounds -- a large-row sequence has more than dec_rows query rows per KV head, so there are at
+// most T group / (dec_rows + 1) of them, each with at most M pages -- capped at 4 GiB; 0 where the shapes rule the
+// copies out (other head sizes, pages that are not a multiple of 64 tokens, too few rows to pay for a copy).
+constexpr int64_t kWideMaxBytes = (int64_t)4 << 30;
+constexpr int kWideMinBatchRows = 1024;  // rows per KV head (T x group) up to which no batch is asked: the decision kernel's bar for one sequence
+static int64_t wide_page_bytes(int page_size, int Hkv, int D) { return (int64_t)page_size * 2 * Hkv * D * 2; }
+static int64_t wide_header_bytes(int S) { return (((int64_t)(2 + S) * 4) + 255) & ~(int64_t)255; }
+static int64_t wide_pages_wanted(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int kv_dtype, int dec_rows) {
+  if (kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8) return 0;
+  if (D != 128 || page_size % 64 != 0 || S > 65535) return 0;
+  const int64_t rows = (int64_t)T * (Hq / Hkv);
+  if (rows <= kWideMinBatchRows) return 0;
+  const int64_t seqs = std::min<int64_t>(S, rows / (dec_rows + 1));
+  return std::min<int64_t>(seqs * M, kWideMaxBytes / wide_page_bytes(page_size, Hkv, D));
+}
+
 size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int q_dtype,
                                      int kv_dtype) {
   (void)q_dtype;
@@ -333,7 +352,12 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
   int pre_keys, pre_chunks;
   prefill_split(T, S, M, page_size, Hq, Hkv, D, &pre_keys, &pre_chunks);
   const size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) : 0;
-  return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256;
+  size_t wide = 0;
+  if (g_tun.prefill_wide && g_tun.prefill_dma && g_tun.prefill_x32) {
+    const int64_t pages = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, D, kv_dtype, rpa::decode_row_limit(T, S, D, kv_dtype));
+    if (pages > 0) wide = (size_t)(wide_header_bytes(S) + pages * wide_page_bytes(page_size, Hkv, D) + 256);
+  }
+  return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256 + wide;
 }
 
 // Shared body of the attention entry points.  k_pages / v_pages and the strides describe where K and V of
@@ -464,7 +488,44 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     char* pre_base = base + pb + (size_t)splits * (po + pml);
     p.pre_o = (float*)pre_base;
     p.pre_ml = (float*)(pre_base + (size_t)pre_chunks * pre_po);
+    // 8-bit pages: what the workspace holds beyond the partial rows takes bf16 copies of the large-row sequences' pages,
+    // and the 32x32-tile kernel reads those where the decision kernel finds that they fit and pay (rpa_widen.hip).
+    rpa::AttnParams pw;
+    bool wide = false;
+    if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && !(p.softcap > 0.f) &&
+        p.D == 128 && p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
+      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows);
+      char* after = pre_base + pre;
+      char* hdr = (char*)(((uintptr_t)after + 255) & ~(uintptr_t)255);
+      char* pages0 = hdr + wide_header_bytes(S);
+      char* end = (char*)workspace + workspace_bytes;
+      const int64_t room = end > pages0 ? (int64_t)(end - pages0) / wide_page_bytes(page_size, Hkv, p.D) : 0;
+      const int64_t cap = std::min(want, room);
+      if (cap >= 1) {
+        p.wide = (const int32_t*)hdr;
+        p.wide_pages = pages0;
+        p.wide_cap = (int)cap;
+        p.wide_rows = 256;
+        p.wide_slots = device_cus();
+        p.src_P = P;
+        pw = p;
+        pw.k_pages = pages0;
+        pw.v_pages = pages0 + (size_t)p.D * 2;
+        pw.head_stride = (int64_t)2 * p.D * 2;
+        pw.token_stride = (int64_t)2 * Hkv * p.D * 2;
+        pw.page_stride = pw.token_stride * page_size;
+        pw.kv_dtype = RPA_BF16;
+        pw.P = (int)cap;
+        pw.pre_x32 = 1;
+        pw.pre_rows = p.wide_rows;
+        pw.pre_slots = p.wide_slots;
+        wide = rpa::prefill_x32_rows(pw) == p.wide_rows;
+        if (!wide) p.wide = nullptr;
+      }
+    }
     int err = 0;
+    if (wide) err = rpa::launch_widen_decide(s, p);
+    if (err) return hip_fail(err, "page-copy decision kernel launch");
     if (stages & 3) err = rpa::launch_attn_decode(s, p, stages & 3);
     if (err) return hip_fail(err, "decode kernel launch");
     // Rows too large for the decode kernel: MFMA prefill kernel where it applies, fp32 kernel otherwise.  No launch where
@@ -472,6 +533,12 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     const bool large_rows_possible = (int64_t)T * p.group > p.dec_rows;
     if ((stages & 4) && large_rows_possible) err = rpa::prefill_supported(p) ? rpa::launch_attn_prefill(s, p) : rpa::launch_attn_generic(s, p);
     if (err) return hip_fail(err, "prefill kernel launch");
+    if (wide && (stages & 4)) {  // (either this pair or the launch above finds work: the decision is the batch's)
+      err = rpa::launch_widen_pages(s, p);
+      if (err) return hip_fail(err, "page-copy kernel launch");
+      err = rpa::launch_attn_prefill_x32(s, pw);
+      if (err) return hip_fail(err, "prefill kernel launch (copied pages)");
+    }
   } else {
     int err = (stages & 4) ? rpa::launch_attn_generic(s, p) : 0;
     if (err) return hip_fail(err, "fp32 kernel launch");

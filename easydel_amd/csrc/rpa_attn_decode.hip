@@ -535,13 +535,14 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
   unsigned long long work = 0;  // keys the large-row kernel visits per KV head, over its row tiles (an estimate)
   int reach = 0;                // a bound on the keys one of its row tiles visits
   int span_min = 0x7fffffff, span_max = 0, n_tiles = 0;  // of a sequence's average row tile
+  const int pre_rows = pre_rows_of(p);
   for (int i = i0; i < i1; ++i) {
     const SeqPlan sp = seq_plan(p, i);
     sum += span_of(i, sp, toks);
     tsum += toks;
     if (sp.live && !sp.small_rows && sp.q_len > 0) {
-      const int tile_reach = p.window > 0 ? min(sp.ctx, p.window + p.pre_rows / p.group + 64) : sp.ctx;
-      const int tiles = (sp.q_len * p.group + p.pre_rows - 1) / p.pre_rows;
+      const int tile_reach = p.window > 0 ? min(sp.ctx, p.window + pre_rows / p.group + 64) : sp.ctx;
+      const int tiles = (sp.q_len * p.group + pre_rows - 1) / pre_rows;
       const int span = max(min(tile_reach, sp.ctx - sp.q_len / 2), 1);  // causal: half the new keys on average
       work += (unsigned long long)tiles * (unsigned)span;
       reach = max(reach, tile_reach);
@@ -599,7 +600,7 @@ __global__ __launch_bounds__(1024) void decode_plan_kernel(AttnParams p) {
     if (p.pre_max_chunks > 1) {
       chunk = p.pre_chunk;
       if (p.pre_auto) {
-        const int slots = max(p.pre_slots, 1);
+        const int slots = max(pre_slots_of(p), 1);
         chunk = (long long)((s_work * (unsigned)p.Hkv / (unsigned)slots / 4 + 63) & ~63ull);
         if (s_tiles > 0 && 4ll * s_span_max <= 5ll * s_span_min) {
           const long long units = (long long)s_tiles * p.Hkv;

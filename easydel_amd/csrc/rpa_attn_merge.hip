@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256, 8) void attn_merge_kernel(AttnParams p) {
       part_row = p.plan[kPlanHeader + p.S + 1 + i] + (t - sp.q0);
     } else if (p.mfma_path && p.pre_max_chunks > 1) {  // prefill row tile split over key chunks
       const int row = (t - sp.q0) * p.group + hq % p.group;
-      n_pieces = prefill_tile(p, sp, (row / p.pre_rows) * p.pre_rows).n_chunks;
+      n_pieces = prefill_tile(p, sp, (row / pre_rows_of(p)) * pre_rows_of(p)).n_chunks;
       part_row = t;
       part_o = p.pre_o;
       part_ml = p.pre_ml;
@@ -154,7 +154,7 @@ __global__ __launch_bounds__(256, 4) void attn_merge_wide_kernel(AttnParams p) {
 #pragma unroll
       for (int hh = 0; hh < HPW; ++hh) {  // neighbouring heads can lie in different row tiles
         const int row = (t - sp.q0) * p.group + (hq0 + hh) % p.group;
-        n_p[hh] = prefill_tile(p, sp, (row / p.pre_rows) * p.pre_rows).n_chunks;
+        n_p[hh] = prefill_tile(p, sp, (row / pre_rows_of(p)) * pre_rows_of(p)).n_chunks;
       }
       part_row = t;
       part_o = p.pre_o;

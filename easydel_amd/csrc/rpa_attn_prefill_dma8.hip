@@ -57,6 +57,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_dma8_kernel(AttnParam
   const int slot = (blockIdx.x / p.Hkv) % n_slots;
   const int chunk = blockIdx.x / (p.Hkv * n_slots);  // slowest: neighbouring blocks share a key chunk (L2 reuse)
   if (p.plan[2] == 0) return;  // the plan kernel saw no sequence with more than 16 rows per KV head
+  if (wide_mode(p)) return;    // this batch's large rows are served from bf16 copies of their pages, by the 32x32-tile kernel
   const int n_live = live_rows(p);
   if (n_live <= 0) return;
   // sequence i starts at slot floor(qsl[i]*G/ROWS) + i; find the last sequence starting at or before `slot`

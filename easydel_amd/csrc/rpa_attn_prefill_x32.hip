@@ -79,6 +79,9 @@ struct Wide16<RPA_BF16> {
   static __device__ __forceinline__ void mfma_o(f32x16& acc, const u32x4& a, const u32x4& b) {
     asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
   }
+  static __device__ __forceinline__ void mfma_o0(f32x16& acc, const u32x4& a, const u32x4& b) {  // starts from zero
+    asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&a"(acc) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ float lo_half(uint32_t w) { return __uint_as_float(w << 16); }
   static __device__ __forceinline__ float hi_half(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
   static __device__ __forceinline__ uint32_t scale_pair(uint32_t w, float a) {  // both halves times a
@@ -96,6 +99,9 @@ struct Wide16<RPA_F16> {
   }
   static __device__ __forceinline__ void mfma_o(f32x16& acc, const u32x4& a, const u32x4& b) {
     asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_o0(f32x16& acc, const u32x4& a, const u32x4& b) {
+    asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&a"(acc) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ float lo_half(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
   static __device__ __forceinline__ float hi_half(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
@@ -115,8 +121,15 @@ __device__ __forceinline__ int swz_key_v32(int tok) {
   else return 0;
 }
 
-template <int D, int NW, int RB, int HT, bool CAP>
+// KS: the pages are bf16 copies of scaled 8-bit pages (AttnParams::wide), bare codes.  A tile of 64 keys lies in one
+// page: its scores are scaled by the page's K scale on top of the softmax scale; its probabilities are multiplied by
+// the page's V scale (inside the exponent) before they are rounded for the PV product, and the row sums are taken per
+// tile and divided by that scale in float32 as they join the running sums -- numerator and denominator then hold
+// the same rounded weights, as with 16-bit pages.  (The scale rounded to 16 bits anywhere, in the values or in the
+// operand of the row sums, is 2^-9 of an output: rows of a few keys then miss 2e-2 on outputs near 4.)
+template <int D, int NW, int RB, int HT, bool CAP, bool KS = false>
 __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p) {
+  static_assert(!(KS && CAP), "per-page key scales are not combined with a soft cap");
   using H = Half16<HT>;
   using W = Wide16<HT>;
   constexpr int BK = 32;                 // keys per block (what a step computes)
@@ -173,6 +186,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   int slot = (blockIdx.x / p.Hkv) % n_slots;
   const int chunk = blockIdx.x / (p.Hkv * n_slots);
   if (p.plan[2] == 0) return;
+  if constexpr (KS) {
+    if (!wide_mode(p)) return;  // this batch stays with the kernel that reads the 8-bit pages
+  }
   const int n_live = live_rows(p);
   if (n_live <= 0) return;
   // Slot -> (sequence, row tile): through the plan's longest-first order where the plan kernel made one (the grid deals
@@ -244,8 +260,32 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // (held as the page's offset in the pool in units of 256 bytes: ids clipped and multiplied once per 64 columns here,
   //  not once per tile in scalar arithmetic; a page is a multiple of 64 rows of 16 bytes or more, the pool is below 2^40 bytes)
   const uint32_t page_units = (uint32_t)(p.page_stride >> 8);
-  auto page_offsets = [&](int col0) -> uint32_t { return (uint32_t)min(max(bt_row[min(col0 + lane, p.M - 1)], 0), p.P - 1) * page_units; };
+  const float sc_mul = p.scale_log2;
+  int wide_first = 0;
+  if constexpr (KS) wide_first = p.wide[2 + i];  // the sequence's copied pages follow one another
+  auto page_offsets = [&](int col0) -> uint32_t {
+    if constexpr (KS) return (uint32_t)min(max(wide_first + col0 + lane, 0), p.P - 1) * page_units;
+    else return (uint32_t)min(max(bt_row[min(col0 + lane, p.M - 1)], 0), p.P - 1) * page_units;
+  };
   uint32_t pages_vec = page_offsets(col_base);
+  // KS: beside them the score scale of each of the 64 columns (softmax scale x the K scale of the column's 8-bit page)
+  // and the logarithm of its V scale; a tile's pair is taken when the tile is requested and queued until its steps.
+  float sck_vec = sc_mul, lvs_vec = 0.f;
+  auto page_scales = [&](int col0) __attribute__((always_inline)) {
+    if (p.kv_scales != nullptr) {
+      const int id = min(max(bt_row[min(col0 + lane, p.M - 1)], 0), p.src_P - 1);
+      const float2 kv = *(const float2*)(p.kv_scales + (int64_t)id * p.C + 2 * h);
+      sck_vec = sc_mul * fmaxf(kv.x, 1e-30f);
+      lvs_vec = __builtin_amdgcn_logf(fmaxf(kv.y, 1e-30f));  // log2
+    }
+  };
+  if constexpr (KS) page_scales(col_base);
+  float kq[KAH + 1], lq[KAH + 1];  // after barrier u: kq[c], lq[c] belong to tile u + c
+#pragma unroll
+  for (int c = 0; c <= KAH; ++c) {
+    kq[c] = sc_mul;
+    lq[c] = 0.f;
+  }
   int cur_col = col_base, cur_off = kv_lo - col_base * p.page_size, cur_tb = kv_lo;
 
   // ---- per row-block lane state --------------------------------------------------------------------
@@ -315,13 +355,18 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     int64_t off;
     bool edge;
     int tb;
+    float sc, lv;  // KS: the tile's score scale and the logarithm of its V scale
   };
   TileDesc td[DQ];
 #pragma unroll
-  for (int j = 0; j < DQ; ++j) td[j] = TileDesc{0, false, 0};
+  for (int j = 0; j < DQ; ++j) td[j] = TileDesc{0, false, 0, 0.f, 0.f};
   // The next 64 columns are fetched when the cursor is within `margin` columns of the end of the held ones.
   auto refill_pages = [&](int margin) __attribute__((always_inline)) {
     if (cur_col - col_base >= 64 - margin) {
+      if constexpr (KS) {
+        page_scales(cur_col);
+        asm volatile("" : "+v"(sck_vec), "+v"(lvs_vec));
+      }
       col_base = cur_col;
       pages_vec = page_offsets(col_base);
       asm volatile("" : "+v"(pages_vec));  // waited for here, once in 64 columns, not at the look-up every tile shares
@@ -333,6 +378,10 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
     for (int j = DQ - 1; j > 0; --j) td[j] = td[j - 1];
     td[0].off = (int64_t)(page_off + (uint32_t)cur_off * tok_stride);
+    if constexpr (KS) {
+      td[0].sc = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(sck_vec), (cur_col - col_base) & 63));
+      td[0].lv = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(lvs_vec), (cur_col - col_base) & 63));
+    }
     td[0].edge = (cur_tb + TT > sp.ctx) || (cur_tb < vis_lo);
     td[0].tb = cur_tb;
     cur_tb += TT;
@@ -393,20 +442,45 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // r = 1 / (exp2(s cap_in2) + 1) and m_neg = cap_out - m_ref.  (The multiplication per score stays: queries scaled
   // ahead of the MFMAs and rounded back to 16 bits would save it, and move a score by 2^-9 of its terms -- measured at
   // four times the usual spread of scores: 3e-2 instead of 1.5e-2 max-abs against the oracle.)
-  const float sc_mul = p.scale_log2;
   const float inv_sc = 1.f / sc_mul;
   const float cap_out = CAP ? p.softcap * 1.4426950408889634f : 0.f;
   const float cap_in = CAP ? p.scale / p.softcap : 0.f;
   const float cap_in2 = cap_in * 2.8853900817779268f;
   const float cap_m2 = -2.f * cap_out;
   auto capped = [&](float s) -> float { return cap_out * fast_tanh(s * cap_in); };  // a raw score to log2 units
-  auto prob = [&](float s, float mn) __attribute__((always_inline)) -> float {
+  auto prob = [&](float s, float mn, float sc) __attribute__((always_inline)) -> float {
     if constexpr (CAP) {
       const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s * cap_in2) + 1.f);
       return s == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(r, cap_m2, mn));  // a masked key is not the cap's lower end
     } else {
-      return __builtin_amdgcn_exp2f(__builtin_fmaf(s, sc_mul, mn));
+      return __builtin_amdgcn_exp2f(__builtin_fmaf(s, sc, mn));
     }
+  };
+  // KS: the queues move on by a tile (at a barrier, ahead of its request), and take the pair of the tile just described.
+  auto queue_shift = [&]() __attribute__((always_inline)) {
+    if constexpr (KS) {
+#pragma unroll
+      for (int c = 0; c < KAH; ++c) {
+        kq[c] = kq[c + 1];
+        lq[c] = lq[c + 1];
+      }
+    }
+  };
+  auto queue_put = [&](int c) __attribute__((always_inline)) {
+    if constexpr (KS) {
+      kq[c] = td[0].sc;
+      lq[c] = td[0].lv;
+    }
+  };
+  // KS: l_acc holds the row sums of one tile, in units of 1 / inv_cur; l_run the sums of the tiles before.  At a tile's
+  // first step, ahead of its row-sum MFMAs (the first of which starts from zero), the tile before joins the running sums.
+  float l_run[RB], inv_cur = 0.f;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) l_run[rb] = 0.f;
+  auto fold_tile = [&](float lv_new) __attribute__((always_inline)) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) l_run[rb] = __builtin_fmaf(l_acc[rb][0], inv_cur, l_run[rb]);
+    inv_cur = __builtin_amdgcn_exp2f(-lv_new);
   };
   // The A operand of the row sums: ones, written to registers once, here.  (Left to the compiler it is rebuilt from
   // scalar registers right in front of the MFMA that reads it, and an MFMA issued through an assembly statement gets
@@ -439,16 +513,17 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 
   // Raises the references of the rows whose new scores (maxima in lmx, raw) exceed them by more than the slack; what
   // has been accumulated, and the pending probabilities pend (relative to the old reference), are scaled to match.
-  auto check = [&](u32x4 (&pend)[RB][2], bool has_pending) __attribute__((always_inline)) {
+  // sc: the scale of the scores the maxima were taken of (KS: thr is then in scaled units, the scores of two tiles having no common unit).
+  auto check = [&](u32x4 (&pend)[RB][2], bool has_pending, float sc) __attribute__((always_inline)) {
     bool grow = false;
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) grow |= lmx[rb] > thr[rb];
+    for (int rb = 0; rb < RB; ++rb) grow |= (KS ? lmx[rb] * sc : lmx[rb]) > thr[rb];
     if (__builtin_expect(__any(grow), 0)) {  // rare: what the register allocator has to park, it parks around this block
       mfma_settle_acc(*(f32x16 (*)[RB * DB])o_acc, l_acc);  // the accumulators may still be on their way
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const float raw = xor32_max(lmx[rb]);
-        const float mx = CAP ? (raw == -INFINITY ? -INFINITY : capped(raw)) : raw * sc_mul;
+        const float mx = CAP ? (raw == -INFINITY ? -INFINITY : capped(raw)) : raw * sc;
         const float m_new = fmaxf(m_ref[rb], ceilf(mx));
         float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref[rb] - m_new);  // a power of two, or 0
         m_ref[rb] = m_new;
@@ -457,7 +532,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           thr[rb] = (m_new == -INFINITY) ? -INFINITY : (y >= 0.999f ? INFINITY : 0.5f * __logf((1.f + y) / (1.f - y)) / cap_in);
           m_neg[rb] = (m_new == -INFINITY) ? 0.f : cap_out - m_new;
         } else {
-          thr[rb] = (m_new + kMaxSlack) * inv_sc;
+          thr[rb] = KS ? m_new + kMaxSlack : (m_new + kMaxSlack) * inv_sc;
           m_neg[rb] = (m_new == -INFINITY) ? 0.f : -m_new;
         }
         asm volatile("s_nop 1" : "+v"(alpha));
@@ -465,6 +540,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           f32x16 l = l_acc[rb];
           l[0] *= alpha;  // the register the epilogue reads; the others hold the same sum and are never read
           l_acc[rb] = l;
+          if constexpr (KS) l_run[rb] *= alpha;
         }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
@@ -488,8 +564,12 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // the K operands of block b+2; kn: of the first PD operands of block b+3 (read at the end); va: lane addresses of the V
   // operands of block b.  dl / dv0, dv1 / dg: LDS address, lane offsets and global base of the NG half tiles the step requests.
   auto fast_step = [&](auto par_tag, auto&& ka, auto&& kn, auto&& va, auto&& in_slot, const uint32_t (&dl)[NG],
-                       const uint32_t (&dv0)[NLH], const uint32_t (&dv1)[NLH], const char* const (&dg)[NG]) __attribute__((always_inline)) {
+                       const uint32_t (&dv0)[NLH], const uint32_t (&dv1)[NLH], const char* const (&dg)[NG], const float sc, const float lv, auto first_tag) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;
+    constexpr bool FIRST = decltype(first_tag)::value;  // KS: the step is the first of its tile
+    float mn[RB];  // what the exponent adds to a scaled score (KS: the logarithm of the tile's V scale on top)
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) mn[rb] = KS ? m_neg[rb] + lv : m_neg[rb];
     f32x16 (&s_cur)[RB] = sa[PAR];              // S(b+1), consumed by the softmax
     f32x16 (&s_nxt)[RB] = sa[PAR ^ 1];          // S(b+2), produced
     u32x4 (&p_cur)[RB][2] = pb[PAR ^ 1];        // P(b), consumed by the PV product
@@ -524,7 +604,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         }
       } else if constexpr (PH == 1) {
         const int e = k - NQ, rb = e % RB, sh = e / RB;
-        W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
+        if (KS && FIRST && sh == 0) W::mfma_o0(l_acc[rb], ones, p_cur[rb][sh]);
+        else W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
         // These slots carry no softmax and no operand read: the step's tile loads are requested from here on, where the
         // time the load unit takes to accept 1 KiB of addresses hides behind an MFMA.
         if (NDI <= NSUM && e < NDI) dma(e);
@@ -552,8 +633,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
           // first the scaled differences of the pair, and the pair before packed (behind the two multiply-adds: they are
           // the distance an exponential wants from its reader); half the pair's slots on, the exponentials
           if (st == 0) {
-            xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc_mul, m_neg[srb]);
-            xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc_mul, m_neg[srb]);
+            xa = __builtin_fmaf(s_cur[srb][2 * sr2], sc, mn[srb]);
+            xb = __builtin_fmaf(s_cur[srb][2 * sr2 + 1], sc, mn[srb]);
             if (ip > 0) p_nxt[prb][pr2 / 4][pr2 % 4] = H::pack(ea, eb);
           } else if (st == SPP / 2) {
             ea = __builtin_amdgcn_exp2f(xa);
@@ -578,8 +659,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
             xa = __builtin_amdgcn_rcpf(xa);
             xb = __builtin_amdgcn_rcpf(xb);
           } else {
-            ea = __builtin_fmaf(xa, cap_m2, m_neg[srb]);
-            eb = __builtin_fmaf(xb, cap_m2, m_neg[srb]);
+            ea = __builtin_fmaf(xa, cap_m2, mn[srb]);
+            eb = __builtin_fmaf(xb, cap_m2, mn[srb]);
           }
         }
         // (the last pair's stages have no reader inside the step: unpinned they gather behind its last MFMA)
@@ -616,7 +697,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // do_qk: block b+2 exists; do_sm: block b+1 exists; do_pv: block b >= 0; next_k: block b+3 exists (its first operands
   // are read at the end); first: the first operands of block b+2 have not been read ahead.  kb2: first key of block b+2.
   // koff / nkoff / voff: byte offsets (slot and part) of blocks b+2 / b+3 in the K ring and of block b in the V ring.
-  auto slow_step = [&](auto par_tag, uint32_t koff, uint32_t nkoff, uint32_t voff, bool do_qk, bool do_sm, bool do_pv, bool next_k, bool first, int kb2) __attribute__((always_inline)) {
+  auto slow_step = [&](auto par_tag, uint32_t koff, uint32_t nkoff, uint32_t voff, bool do_qk, bool do_sm, bool do_pv, bool next_k, bool first, int kb2, float sc, float lv, bool first_of_tile) __attribute__((always_inline)) {
     constexpr int PAR = decltype(par_tag)::value;
     f32x16 (&s_cur)[RB] = sa[PAR];
     f32x16 (&s_nxt)[RB] = sa[PAR ^ 1];
@@ -646,8 +727,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
       for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
         for (int r2 = 0; r2 < 8; ++r2) {
-          const float e0 = prob(s_cur[rb][2 * r2], m_neg[rb]);
-          const float e1 = prob(s_cur[rb][2 * r2 + 1], m_neg[rb]);
+          const float e0 = prob(s_cur[rb][2 * r2], KS ? m_neg[rb] + lv : m_neg[rb], sc);
+          const float e1 = prob(s_cur[rb][2 * r2 + 1], KS ? m_neg[rb] + lv : m_neg[rb], sc);
           p_nxt[rb][r2 / 4][r2 % 4] = H::pack(e0, e1);
         }
     }
@@ -658,7 +739,10 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
       for (int sh = 0; sh < 2; ++sh)
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);  // row sums of block b
+        for (int rb = 0; rb < RB; ++rb) {  // row sums of block b
+          if (KS && first_of_tile && sh == 0) W::mfma_o0(l_acc[rb], ones, p_cur[rb][sh]);
+          else W::mfma_o(l_acc[rb], ones, p_cur[rb][sh]);
+        }
 #pragma unroll
       for (int g = 0; g < NVO; ++g) {
         const int db = g / 2, s = g % 2;
@@ -703,6 +787,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
   for (int t = 0; t < U0 + KAH; ++t) {
     next_tile();
+    queue_put(t - U0 + 1);  // (the first barrier moves the queues on by one)
     if (t < n_tiles) issue_half(false, t % KN, td[0]);
     if (t < U0 + VAH && t < n_tiles) issue_half(true, t % KN, td[0]);
   }
@@ -722,7 +807,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     else wait_loads_and_barrier<0>();
     const int vt = u + VAH, kt = u + KAH;
     if (vt < n_tiles) issue_half(true, vt % KN, td[DQ - 1]);
+    queue_shift();
     next_tile();
+    queue_put(KAH);
     if (kt < n_tiles) issue_half(false, kt % KN, td[0]);
   };
   auto slow_step_at = [&](auto par_tag, int b) __attribute__((always_inline)) {
@@ -730,8 +817,19 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     const bool do_qk = b + 2 < n_blocks, do_sm = b + 1 >= 0 && b + 1 < n_blocks, do_pv = b >= 0 && b < n_blocks;
     const bool next_k = b + 3 < n_blocks, first = b == -2;
     constexpr int PAR = decltype(par_tag)::value;
-    if (do_sm) check(pb[PAR ^ 1], do_pv);
-    slow_step(par_tag, ring_off(b + 2), ring_off(b + 3), ring_off(max(b, 0)), do_qk, do_sm, do_pv, next_k, first, kv_lo + (b + 2) * BK);
+    // KS: block b + 1 lies in the barrier's tile if b is even and there are two steps per tile, else in the next; block b in the barrier's
+    constexpr int C1 = (SPT == 2 && PAR == 1) ? 0 : 1;
+    const float sc = kq[C1], lv = lq[C1];
+    const bool first_of_tile = SPT == 1 || PAR == 1;  // (b is even)
+    if constexpr (KS) {
+      if (first_of_tile) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(l_acc[rb]));  // the row sums may still be on their way
+        fold_tile(lq[0]);
+      }
+    }
+    if (do_sm) check(pb[PAR ^ 1], do_pv, sc);
+    slow_step(par_tag, ring_off(b + 2), ring_off(b + 3), ring_off(max(b, 0)), do_qk, do_sm, do_pv, next_k, first, kv_lo + (b + 2) * BK, sc, lv, first_of_tile);
   };
   // Pairs of steps (b, b + 1), b even, the pinned code may serve: b >= 0, the barriers whose requests may be in flight
   // were regular ones, blocks b+2 and b+3 exist and are unmasked for the whole wave ...
@@ -757,6 +855,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
   for (int u = 0; u < NLH; ++u) asm volatile("" : "+v"(voff_k[u]), "+v"(voff_v[u]));
   asm volatile("" : "+v"(pages_vec));
+  if constexpr (KS) asm volatile("" : "+v"(sck_vec), "+v"(lvs_vec));
   if (b < b_fast_hi) {
     // Ring offsets of the tiles u .. u + KN - 1, u the index of the next barrier (r[c]: tile u + c), turned once per barrier.
     uint32_t r[KN];
@@ -794,15 +893,21 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         if (k == V_UPD0 + db) VA[db] = pinned_add(r[1 % KN] - r[0], VA[db]);
     };
     auto nothing = [&](int) __attribute__((always_inline)) {};
+
     // one barrier and the SPT steps behind it; PAR0: the buffer the first of them hands its softmax
     auto fast_trip = [&](auto par_tag) __attribute__((always_inline)) {
       constexpr int PAR0 = decltype(par_tag)::value;
       // visible now: K tiles up to u + KNO, V tiles up to u; in flight stay the requests of the FLYB barriers before
       wait_loads_and_barrier<2 * FLYB * NLH>();
-      check(pb[PAR0 ^ 1], true);
+      queue_shift();
+      const float sc0 = kq[SPT == 2 ? 0 : 1], sc1 = kq[1];  // of blocks b + 1 and b + 2
+      const float lv0 = lq[SPT == 2 ? 0 : 1], lv1 = lq[1];
+      if constexpr (KS) fold_tile(lq[0]);  // (the row sums of the tile before were issued a whole PV phase ago)
+      check(pb[PAR0 ^ 1], true, sc0);
       // this barrier's requests, made from inside its steps: V(u + VAH), described DQ tiles ago, and K(u + KAH)
       const char* v_ptr = v_base + td[DQ - 1].off;
       next_tile(false);
+      queue_put(KAH);
       const char* k_ptr = k_base + td[0].off;
       const uint32_t v_lds = v_lds0 + r[VAH % KN];
       const uint32_t k_lds = k_lds0 + r[KAH % KN];
@@ -813,17 +918,17 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         const char* const dg1[1] = {k_ptr};
         fast_step(std::integral_constant<int, PAR0>{},
                   [&](int nx) { return A[nx]; }, [&](int o) { return A[o] + PART; }, [&](int db) { return VA[db]; }, nothing,
-                  dl0, voff_v, voff_v, dg0);
-        check(pb[PAR0], true);
+                  dl0, voff_v, voff_v, dg0, sc0, lv0, std::true_type{});
+        check(pb[PAR0], true, sc1);
         fast_step(std::integral_constant<int, PAR0 ^ 1>{},
                   [&](int nx) { return A[nx] + PART; }, [&](int o) { return A[o]; }, [&](int db) { return VA[db] + PART; }, move_on,
-                  dl1, voff_k, voff_k, dg1);
+                  dl1, voff_k, voff_k, dg1, sc1, lv1, std::false_type{});
       } else {
         const uint32_t dl0[2] = {v_lds, k_lds};
         const char* const dg0[2] = {v_ptr, k_ptr};
         fast_step(std::integral_constant<int, PAR0>{},
                   [&](int nx) { return A[nx % NKA] + (uint32_t)(256 * (nx / NKA)); }, [&](int o) { return A[o]; },
-                  [&](int db) { return VA[db % NVA] + (uint32_t)(256 * (db / NVA)); }, move_on, dl0, voff_v, voff_k, dg0);
+                  [&](int db) { return VA[db % NVA] + (uint32_t)(256 * (db / NVA)); }, move_on, dl0, voff_v, voff_k, dg0, sc0, lv0, std::true_type{});
       }
       const uint32_t r0 = r[0];
 #pragma unroll
@@ -860,7 +965,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   if (staged) wait_loads_and_barrier<0>();  // every wave is through with the rings, and no tile is still on its way into them
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    const float l_tot = l_acc[rb][0];
+    const float l_tot = KS ? __builtin_fmaf(l_acc[rb][0], inv_cur, l_run[rb]) : l_acc[rb][0];
     // where the lane's row goes: its index among the [T][Hq] rows of the output (or of a chunk's partial rows), -1: nowhere
     const int my_slot = row_ok[rb] ? out_tok[rb] * p.Hq + out_head[rb] : -1;
     if (single) {
@@ -939,14 +1044,14 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   }
 }
 
-template <int D, int NW, int RB, int HT, bool CAP>
+template <int D, int NW, int RB, int HT, bool CAP, bool KS = false>
 static int launch_x32(hipStream_t stream, const AttnParams& p) {
   constexpr int ROWS = NW * RB * 32;
   if (p.pre_rows != ROWS) return (int)hipErrorInvalidValue;  // the plan and merge kernels are told this row-tile height
   const int64_t slots = ((int64_t)p.T * p.group) / ROWS + p.S;  // upper bound on row tiles of the batch
   const int64_t blocks = slots * p.Hkv * p.pre_max_chunks;
   if (blocks > 0x7fffffff) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL((attn_prefill_x32_kernel<D, NW, RB, HT, CAP>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
+  hipLaunchKernelGGL((attn_prefill_x32_kernel<D, NW, RB, HT, CAP, KS>), dim3((unsigned)blocks), dim3(64 * NW), 0, stream, p);
   return (int)hipGetLastError();
 }
 
@@ -962,6 +1067,10 @@ int prefill_x32_rows(const AttnParams& p) {
 }
 
 int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p) {
+  if (p.wide != nullptr) {  // bf16 copies of 8-bit pages
+    if (p.D != 128 || p.kv_dtype != RPA_BF16 || p.softcap > 0.f) return (int)hipErrorInvalidValue;
+    return launch_x32<128, 4, 2, RPA_BF16, false, true>(stream, p);
+  }
   if (p.D == 256) return p.softcap > 0.f ? launch_x32<256, 4, 1, RPA_BF16, true>(stream, p) : launch_x32<256, 4, 1, RPA_BF16, false>(stream, p);
   if (p.kv_dtype == RPA_F16) return launch_x32<128, 4, 2, RPA_F16, false>(stream, p);
   return launch_x32<128, 4, 2, RPA_BF16, false>(stream, p);

@@ -74,7 +74,21 @@ struct AttnParams {
   int decode_which;  // launches of the decode stage: bit 0 plan kernel, bit 1 decode kernel
   int prefill_dma;   // 1: bf16 prefill tiles go global -> LDS directly where that kernel applies; 0: always through registers
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
+  // 8-bit pages whose large-row sequences may be served from bf16 copies of their pages (null: never).  Written by the
+  // decision kernel ahead of the plan: [0] = 1 if this batch is served that way, [1] = copied pages in use,
+  // [2 + i] = first copied page of sequence i (its pages follow in block-table order).
+  const int32_t* wide;
+  void* wide_pages;    // the copies: [wide_cap][page_size][2 Hkv][D] bf16, bare codes, K of head h at row 2h, V at 2h + 1
+  int wide_cap;        // pages the copies hold
+  int wide_rows;       // pre_rows of a batch served from the copies
+  int wide_slots;      // pre_slots likewise
+  int src_P;           // pages of the 8-bit pool, for the kernel that reads the copies (its P is wide_cap)
 };
+
+// Row-tile height and resident workgroups of the large-row kernel that serves this batch.
+__device__ __forceinline__ bool wide_mode(const AttnParams& p) { return p.wide != nullptr && p.wide[0] != 0; }
+__device__ __forceinline__ int pre_rows_of(const AttnParams& p) { return wide_mode(p) ? p.wide_rows : p.pre_rows; }
+__device__ __forceinline__ int pre_slots_of(const AttnParams& p) { return wide_mode(p) ? p.wide_slots : p.pre_slots; }
 
 __device__ __forceinline__ int live_rows(const AttnParams& p);
 
@@ -117,7 +131,7 @@ __device__ __forceinline__ float with_sink(const AttnParams& p, int hq, float m_
   return l + __builtin_amdgcn_exp2f(__builtin_fmaf(p.sinks[hq], 1.4426950408889634f, -m_log2));
 }
 
-// Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + pre_rows) of a sequence) must visit, kv_lo
+// Key range [kv_lo, kv_hi) a prefill row tile (rows [R0, R0 + pre_rows_of(p)) of a sequence) must visit, kv_lo
 // rounded down to 64, and the split-K chunks the prefill kernel cuts it into: the range over the chunk length the
 // plan kernel chose (plan[4]), rounded to the nearest count the partial buffers hold, all chunks of one length (a
 // multiple of 64; the last one holds what is left), so that the workgroups of a sequence finish together.
@@ -127,7 +141,7 @@ struct PrefillTile {
 __device__ __forceinline__ PrefillTile prefill_tile(const AttnParams& p, const SeqPlan& sp, int R0) {
   PrefillTile t;
   const int rows_total = sp.q_len * p.group;
-  const int last_row = min(R0 + p.pre_rows, rows_total) - 1;
+  const int last_row = min(R0 + pre_rows_of(p), rows_total) - 1;
   const int base_pos = sp.ctx - sp.q_len;
   t.kv_hi = min(sp.ctx, base_pos + last_row / p.group + 1);
   t.vis_lo = (p.window > 0) ? max(base_pos + R0 / p.group - p.window + 1, 0) : 0;
@@ -285,5 +299,7 @@ int launch_attn_prefill_dma8(hipStream_t stream, const AttnParams& p);  // 8-bit
 int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p);   // 16-bit pages, 32x32x16 tiles, one workgroup per CU
 int prefill_x32_rows(const AttnParams& p);  // its row-tile height at the call's shape, 0 where it does not apply
 bool prefill_dma8_supported(const AttnParams& p);
+int launch_widen_decide(hipStream_t stream, const AttnParams& p);  // 8-bit pages: whether this batch's large rows are served from bf16 copies ...
+int launch_widen_pages(hipStream_t stream, const AttnParams& p);   // ... and the copies
 
 }  // namespace rpa

@@ -1,0 +1,105 @@
+"""GPU parity of the prefill path that serves scaled 8-bit pages through bf16 copies: the decision kernel finds that a
+batch's large-row sequences fit the workspace and have rows enough to pay for the copies, their pages are widened once
+(bare codes, exact in bf16) and the 32x32-tile kernel reads the copies, scaling each tile's scores by its page's K
+scale and its probabilities by the page's V scale.  Checked against the oracle, and against the kernel that reads the 8-bit pages (``prefill_wide`` 0)."""
+
+import numpy as np
+import pytest
+import torch
+
+import rpa_testlib as tl
+from easydel_amd import _lib, kernels
+from rpa_testlib import FP8, INT8
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(b, what, **kw):
+    """Output with the copies allowed, output with them switched off, both checked against the oracle."""
+    want = tl.oracle_out(b, **kw)
+    got = tl.run_gpu_attention(b, **kw)
+    mx, mean = tl.assert_close(got, want, b, what, one_ulp_above_4=True)
+    print(f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}", flush=True)
+    prev = _lib.set_tunable("prefill_wide", 0)
+    try:
+        plain = tl.run_gpu_attention(b, **kw)
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
+    tl.assert_close(plain, want, b, what + " (8-bit kernel)", one_ulp_above_4=True)
+    return got, plain
+
+
+@pytest.mark.parametrize("kv_dtype", [FP8, INT8])
+@pytest.mark.parametrize("page_size,Hq,Hkv", [(64, 32, 8), (128, 40, 8), (64, 8, 1)])
+def test_long_prefill_over_scaled_8bit_pages_reads_the_copies(gpu, kv_dtype, page_size, Hq, Hkv):
+    """Two long prefill chunks, a short one (large rows too: it is copied with them), decode sequences and an empty row;
+    contexts that end inside a page, whose slots past the end hold NaN codes in the fp8 pool."""
+    b = tl.make_batch(900 + page_size + Hq, [5000, 1, 700, 9300, 333, 40], [700, 1, 1, 1100, 1, 40], Hq=Hq, Hkv=Hkv, D=128,
+                      page_size=page_size, kv_dtype=kv_dtype, pad_rows=2, pad_tokens=5)
+    if kv_dtype == FP8:
+        for i, c in enumerate(b.context_lens[:b.n]):
+            if c % page_size:
+                b.kv_raw[b.block_tables[i, c // page_size], c % page_size:] = 0x7F
+    got, plain = _both(b, f"copied pages kv{kv_dtype} pg{page_size} Hq{Hq}/{Hkv}")
+    rows = tl.valid_rows(b)
+    assert np.abs(got - plain)[rows].max() <= 2 * tl.TOL_BF16_MAX
+    assert (got[rows] != plain[rows]).any(), "the two kernels round differently: identical outputs mean the copies were not used"
+
+
+def test_key_chunks_over_the_copies(gpu):
+    """One prompt chunk behind a long context: its row tiles are cut into key chunks and merged."""
+    prev = _lib.set_tunable("prefill_chunks", 8)
+    try:
+        b = tl.make_batch(911, [30000], [600], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
+        got, plain = _both(b, "copied pages, row tiles split over key chunks")
+    finally:
+        _lib.set_tunable("prefill_chunks", prev)
+    b = tl.make_batch(912, [30000, 2000], [600, 300], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8)
+    got, plain = _both(b, "copied pages, chunk length chosen on the device")
+    assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
+
+
+def test_fp8_pages_without_scales_are_copied_exactly(gpu):
+    b = tl.make_batch(913, [4000, 2500], [1200, 400], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8, scaled=False)
+    _both(b, "copied pages, cast-only fp8")
+
+
+def test_batches_whose_rows_do_not_pay_stay_on_the_8bit_kernel(gpu):
+    """Many short prompt chunks behind long contexts: copying every page would cost more than it saves; the decision
+    kernel says no and the result is the 8-bit kernel's, bit for bit.  Likewise under a window or a soft cap, which
+    the copies do not serve."""
+    b = tl.make_batch(914, [6000] * 8 + [50], [40] * 8 + [1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
+    got, plain = _both(b, "short chunks behind long contexts")
+    assert np.array_equal(got, plain)
+    b = tl.make_batch(915, [5000, 3000], [700, 600], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8)
+    for kw in (dict(sliding_window=1000), dict(logits_soft_cap=30.0)):
+        got, plain = _both(b, f"copies not offered with {sorted(kw)}", **kw)
+        assert np.array_equal(got, plain)
+
+
+def test_a_workspace_without_room_for_the_copies_falls_back(gpu, monkeypatch):
+    """The copies live in what the workspace holds beyond the partial rows: sized without them, the call runs the 8-bit
+    kernel (bit-identical to ``prefill_wide`` 0); with room for some pages but not all, likewise."""
+    b = tl.make_batch(916, [5000, 700, 9300], [700, 1, 1100], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
+    prev = _lib.set_tunable("prefill_wide", 0)
+    try:
+        plain = tl.run_gpu_attention(b)
+        d = tl.device_batch(b)
+        lib = _lib.load()
+        T, S, M = d["query"].shape[0], b.S, b.M
+        small = int(lib.rpa_attention_workspace_bytes(T, S, M, b.page_size, b.Hq, b.Hkv, b.D, tl.BF16, INT8))
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
+    full = int(_lib.load().rpa_attention_workspace_bytes(T, S, M, b.page_size, b.Hq, b.Hkv, b.D, tl.BF16, INT8))
+    page16 = b.page_size * 2 * b.Hkv * b.D * 2
+    assert full >= small + (79 + 11 + 146) * page16, "the sizing call asks for room for the copies"
+    for nbytes in (small, small + 100 * page16):
+        kernels._workspaces.clear()
+        monkeypatch.setattr(kernels, "_workspace", lambda device, n, nb=nbytes: torch.empty(nb, dtype=torch.uint8, device=device))
+        got = tl.run_gpu_attention(b)
+        assert np.array_equal(got, plain), nbytes
+    monkeypatch.undo()
+    kernels._workspaces.clear()
+    got = tl.run_gpu_attention(b)
+    assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
+    tl.assert_close(got, tl.oracle_out(b), b, "full workspace", one_ulp_above_4=True)
