@@ -59,6 +59,8 @@ def parse_args():
     ap.add_argument("--max-splits", type=int, default=0)
     ap.add_argument("--prefill-x32", type=int, default=-1, help="32x32-tile prefill kernel: -1 the library's choice, 0 never")
     ap.add_argument("--prefill-wide", type=int, default=-1, help="bf16 copies of 8-bit pages for the 32x32-tile prefill kernel: -1 the library's choice, 0 never")
+    ap.add_argument("--chunk-seqs", type=int, default=0, help="fp8-prefill / int8-prefill: this many prompt chunks (1..16) instead of 4 ...")
+    ap.add_argument("--chunk-len", type=int, default=0, help="... of this many tokens instead of 2 048")
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
     ap.add_argument("--mla-uniform-context", type=int, default=0,
@@ -83,7 +85,7 @@ DECODE_SHAPES = {"decode-hkv4": dict(Hq=28, Hkv=4), "decode-hkv1": dict(Hq=8, Hk
                  "decode-32seq": dict(n_seqs=32)}
 
 
-def build_workload(name, seed, sequential=False):
+def build_workload(name, seed, sequential=False, chunks=(0, 0)):
     import bench_workloads as workloads
 
     if name == "c2":
@@ -95,6 +97,8 @@ def build_workload(name, seed, sequential=False):
     if name == "c4-int8":
         return workloads.config4_quantised_decode(seed, "int8")
     if name in ("fp8-prefill", "int8-prefill"):  # tuning shape for the 8-bit prefill kernel
+        if chunks[0] > 0 and chunks[1] > 0:  # (6 000 pages hold 16 chunks of up to 16 384 tokens of context)
+            return workloads.quantised_long_prefill(seed, name.split("-")[0], n_seqs=chunks[0], q_len=chunks[1], num_pages=6000 if chunks[0] > 4 else 2000)
         return workloads.quantised_long_prefill(seed, name.split("-")[0])
     if name == "gemma-decode":  # tuning shape: decode at head size 256, where the LDS-direct decode kernel is the default
         return workloads.gemma_decode(seed)
@@ -449,7 +453,7 @@ def measure(args, workload, with_cpu):
     from easydel_amd import _lib, kernels
 
     dev = torch.device("cuda:0")
-    w = build_workload(workload, args.seed, args.sequential_pages)
+    w = build_workload(workload, args.seed, args.sequential_pages, (args.chunk_seqs, args.chunk_len))
     tens = workloads.device_tensors(w, dev, seed=args.seed)
     quant = w.kv_dtype in ("fp8", "int8")
     out = torch.empty_like(tens["query"])

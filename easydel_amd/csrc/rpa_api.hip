@@ -44,7 +44,9 @@ struct Tunables {
   int force_generic = 0;
   int prefill_dma = 1;
   int prefill_x32 = 1;     // 1: the 32x32-tile prefill kernel serves the shapes it is built for
-  int prefill_wide = 1;    // 1: 8-bit pages reach that kernel through bf16 copies where the workspace has room and the batch's rows pay for them
+  int prefill_wide = 1;    // 8-bit pages reach that kernel through bf16 copies where the workspace has room and the batch's rows pay for
+                           // them: 0 never, 1 at the default bar (kWideMinRows rows per copied page, a workgroup per CU), n > 1 at
+                           // a bar of n rows and none on the workgroups
   int decode_pace = 1;
   int decode_dma = -1;     // -1: where it measured faster (head size 256; int8 pages); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
   int mla_chunks = 0;      // 0 = sized from the shapes
@@ -195,7 +197,7 @@ int rpa_set_tunable(const char* name, int value) {
 #endif
   if (!strcmp(name, "prefill_dma")) return swap(g_tun.prefill_dma, value != 0);
   if (!strcmp(name, "prefill_x32")) return swap(g_tun.prefill_x32, value != 0);
-  if (!strcmp(name, "prefill_wide")) return swap(g_tun.prefill_wide, value != 0);
+  if (!strcmp(name, "prefill_wide")) return swap(g_tun.prefill_wide, value < 0 ? 0 : value);
   if (!strcmp(name, "decode_pace")) return swap(g_tun.decode_pace, value != 0);
   if (!strcmp(name, "decode_dma")) return swap(g_tun.decode_dma, value < 0 ? -1 : value > 3 ? 3 : value);
   if (!strcmp(name, "mla_min_chunk")) return swap(g_tun.mla_min_chunk, value <= 0 ? 0 : ((value + 63) & ~63));
@@ -330,14 +332,15 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
 // most T group / (dec_rows + 1) of them, each with at most M pages -- capped at 4 GiB; 0 where the shapes rule the
 // copies out (other head sizes, pages that are not a multiple of 64 tokens, too few rows to pay for a copy).
 constexpr int64_t kWideMaxBytes = (int64_t)4 << 30;
-constexpr int kWideMinBatchRows = 1024;  // rows per KV head (T x group) up to which no batch is asked: the decision kernel's bar for one sequence
+constexpr int kWideMinRows = 1024;  // the decision kernel's default bar: query rows per KV head and copied page, on the batch's average
+static int wide_min_rows(int tunable) { return tunable > 1 ? tunable : kWideMinRows; }
 static int64_t wide_page_bytes(int page_size, int Hkv, int D) { return (int64_t)page_size * 2 * Hkv * D * 2; }
 static int64_t wide_header_bytes(int S) { return (((int64_t)(2 + S) * 4) + 255) & ~(int64_t)255; }
-static int64_t wide_pages_wanted(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int kv_dtype, int dec_rows) {
+static int64_t wide_pages_wanted(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int kv_dtype, int dec_rows, int min_rows) {
   if (kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8) return 0;
   if (D != 128 || page_size % 64 != 0 || S > 65535) return 0;
   const int64_t rows = (int64_t)T * (Hq / Hkv);
-  if (rows <= kWideMinBatchRows) return 0;
+  if (rows <= min_rows) return 0;  // no batch of so few rows (T x group) holds a sequence that reaches the bar
   const int64_t seqs = std::min<int64_t>(S, rows / (dec_rows + 1));
   return std::min<int64_t>(seqs * M, kWideMaxBytes / wide_page_bytes(page_size, Hkv, D));
 }
@@ -354,7 +357,7 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
   const size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) : 0;
   size_t wide = 0;
   if (g_tun.prefill_wide && g_tun.prefill_dma && g_tun.prefill_x32) {
-    const int64_t pages = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, D, kv_dtype, rpa::decode_row_limit(T, S, D, kv_dtype));
+    const int64_t pages = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, D, kv_dtype, rpa::decode_row_limit(T, S, D, kv_dtype), wide_min_rows(g_tun.prefill_wide));
     if (pages > 0) wide = (size_t)(wide_header_bytes(S) + pages * wide_page_bytes(page_size, Hkv, D) + 256);
   }
   return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256 + wide;
@@ -494,7 +497,9 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     bool wide = false;
     if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && !(p.softcap > 0.f) &&
         p.D == 128 && p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
-      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows);
+      p.wide_min_rows = wide_min_rows(tun.prefill_wide);
+      p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : device_cus();
+      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows, p.wide_min_rows);
       char* after = pre_base + pre;
       char* hdr = (char*)(((uintptr_t)after + 255) & ~(uintptr_t)255);
       char* pages0 = hdr + wide_header_bytes(S);

@@ -21,9 +21,10 @@
 
 namespace rpa {
 
-// Fewest query rows per KV head (tokens x group) per copied page, on the batch's average, from which the copies pay:
-// a page costs 3 bytes per element to copy, and saves about a quarter of the matrix time of every row tile that reads it.
-constexpr int kWideMinRows = 1024;
+// (AttnParams::wide_min_rows: the fewest query rows per KV head (tokens x group) per copied page, on the batch's average,
+// from which the copies pay -- a page costs 3 bytes per element to copy, and saves about a quarter of the matrix time
+// of every row tile that reads it.  AttnParams::wide_min_wgs: the fewest workgroups of the 32x32-tile kernel, whose row
+// tiles are twice as tall as the 8-bit kernel's and one to a CU: a batch of few row tiles fills the chip better there.)
 
 // wide[0] = 1 and wide[2 + i] = first copied page of sequence i if the large-row sequences' pages fit wide_cap and
 // their rows are worth it; else wide[0] = 0.  One workgroup of 256 threads.
@@ -31,14 +32,17 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
   __shared__ int s_scan[256];
   __shared__ int s_carry;
   __shared__ unsigned long long s_work;
+  __shared__ int s_tiles;
   const int tid = threadIdx.x;
   if (tid == 0) {
     s_carry = 0;
     s_work = 0ull;
+    s_tiles = 0;
   }
   __syncthreads();
   const int n_live = live_rows(p);
   unsigned long long work = 0;
+  int tiles = 0;
   bool fits = true;
   for (int i0 = 0; i0 < p.S; i0 += 256) {  // (uniform trip count)
     const int i = i0 + tid;
@@ -48,6 +52,7 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
       if (sp.live && !sp.small_rows) {
         need = (sp.ctx + p.page_size - 1) / p.page_size;
         work += (unsigned long long)need * (unsigned)(sp.q_len * p.group);
+        tiles += (sp.q_len * p.group + p.wide_rows - 1) / p.wide_rows;
       }
     }
     s_scan[tid] = need;
@@ -67,10 +72,12 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
     __syncthreads();
   }
   if (work) atomicAdd(&s_work, work);
+  if (tiles) atomicAdd(&s_tiles, tiles);
   const int all_fit = __syncthreads_and(fits ? 1 : 0);
   if (tid == 0) {
     const int total = s_carry;
-    const bool pays = total > 0 && s_work >= (unsigned long long)kWideMinRows * (unsigned)total;
+    const bool pays = total > 0 && s_work >= (unsigned long long)p.wide_min_rows * (unsigned)total &&
+                      (long long)s_tiles * p.Hkv >= p.wide_min_wgs;
     wide[0] = (all_fit && pays) ? 1 : 0;
     wide[1] = total;
   }
