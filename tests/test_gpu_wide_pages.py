@@ -123,3 +123,72 @@ def test_a_workspace_without_room_for_the_copies_falls_back(gpu, monkeypatch):
         _lib.set_tunable("prefill_wide", prev)
     assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
     tl.assert_close(got, tl.oracle_out(b), b, "full workspace", one_ulp_above_4=True)
+
+
+@pytest.mark.parametrize("kv_dtype", [FP8, INT8])
+def test_separate_key_and_value_pools_are_copied_alike(gpu, kv_dtype):
+    """The same through ``unified_attention``: the copy kernel reads K and V rows through the pools' own strides."""
+    b = tl.make_batch(919, [3000, 200, 1800], [800, 1, 500], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=kv_dtype, pad_rows=1)
+    want = tl.oracle_out(b)
+    prev = _lib.set_tunable("prefill_wide", 2)
+    try:
+        got = tl.run_gpu_unified_attention(b)
+        same = tl.run_gpu_attention(b)
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
+    tl.assert_close(got, want, b, "separate pools, copied pages", one_ulp_above_4=True)
+    assert np.array_equal(got, same), "the pool layout changes no bit"
+    prev = _lib.set_tunable("prefill_wide", 0)
+    try:
+        plain = tl.run_gpu_unified_attention(b)
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
+    assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
+
+
+@pytest.mark.parametrize("kv_dtype", [FP8, INT8])
+def test_fused_quantised_v3_operation_over_long_chunks(gpu, kv_dtype):
+    """Registry -> v3 operation on a view with scales, two serving steps with long prompt chunks: the step's K/V rows are
+    written quantised first, the copies are made from the pages as written (the rows of this step among them)."""
+    from easydel_amd.caching import RaggedPagesCacheConfig, RaggedPagesCacheView, RaggedPagesMetadata
+    from easydel_amd.operations import OperationMetadata, OperationRegistry
+    from rpa_testlib import BF16, orc
+
+    torch_kv = {FP8: torch.float8_e4m3fn, INT8: torch.int8}[kv_dtype]
+    rng = np.random.default_rng(21)
+    Hq, Hkv, D, pg, S, M = 32, 8, 128, 64, 4, 40
+    P = S * M + 1
+    cfg = RaggedPagesCacheConfig.create(torch_kv, num_hidden_layers=1, num_kv_heads=Hkv, max_model_length=M * pg,
+                                        kv_head_dim_size=D, page_size=pg, num_pages=P)
+    view = RaggedPagesCacheView.init(cfg, device=gpu, scaled=True)
+    bt = rng.permutation(np.arange(1, P)).astype(np.int32)[:S * M].reshape(S, M)
+    op = OperationRegistry.create("ragged_page_attention_v3", OperationMetadata())
+    codes = np.zeros((P, pg, 2 * Hkv, D), np.uint8)
+    scales = np.ones((P, 2 * Hkv), np.float32)
+    ctx = np.zeros(S, np.int32)
+    prev = _lib.set_tunable("prefill_wide", 2)
+    try:
+        for q_lens in ([1500, 600, 1, 33], [1, 700, 1, 400]):
+            q_lens = np.array(q_lens, np.int32)
+            ctx = (ctx + q_lens).astype(np.int32)
+            qsl = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+            T = int(qsl[-1])
+            q_raw, k_raw, v_raw = (orc.f32_to_bf16_bits(rng.standard_normal((T, h, D), dtype=np.float32)) for h in (Hq, Hkv, Hkv))
+            dist = orc.request_distribution_ref(q_lens, ctx)
+            meta = RaggedPagesMetadata(pages_tables=torch.from_numpy(bt).to(gpu), context_lens=torch.from_numpy(ctx).to(gpu),
+                                       query_start_loc=torch.from_numpy(qsl).to(gpu), num_seqs=torch.tensor([S], dtype=torch.int32, device=gpu),
+                                       request_distribution=torch.from_numpy(dist).to(gpu), page_size=pg)
+            out = op(tl.to_torch(q_raw, BF16, gpu), tl.to_torch(k_raw, BF16, gpu), tl.to_torch(v_raw, BF16, gpu), view, meta)
+            torch.cuda.synchronize()
+            codes, scales = orc.page_scatter_ragged_quantised_ref(orc.bf16_bits_to_f32(k_raw), orc.bf16_bits_to_f32(v_raw), codes, scales,
+                                                                  ctx, bt, qsl, [S], kv_dtype=kv_dtype)
+            assert np.array_equal(view.kv_pages.view(torch.uint8).cpu().numpy().reshape(codes.shape), codes)
+            assert np.array_equal(view.kv_scales.cpu().numpy(), scales)
+            kv_val = orc.decode_codes(codes, kv_dtype).astype(np.float64) * scales[:, None, :, None]
+            want = orc.ragged_paged_attention_ref(orc.bf16_bits_to_f32(q_raw).astype(np.float64), kv_val, ctx, bt, qsl, [S])
+            got = tl.from_torch(out.attention_outputs, BF16)
+            err = np.abs(got - want)
+            print(f"  v3 operation over {q_lens.tolist()}: max-abs {err.max():.3e} mean-abs {err.mean():.3e}", flush=True)
+            assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
