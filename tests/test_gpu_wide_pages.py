@@ -3,6 +3,8 @@ batch's large-row sequences fit the workspace and have rows enough to pay for th
 (bare codes, exact in bf16) and the 32x32-tile kernel reads the copies, scaling each tile's scores by its page's K
 scale and its probabilities by the page's V scale.  Checked against the oracle, and against the kernel that reads the 8-bit pages (``prefill_wide`` 0)."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -192,3 +194,52 @@ def test_fused_quantised_v3_operation_over_long_chunks(gpu, kv_dtype):
             assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN
     finally:
         _lib.set_tunable("prefill_wide", prev)
+
+
+_SEEDS = int(os.environ.get("RPA_RANDOM_SEEDS", "12"))
+_FIRST_SEED = int(os.environ.get("RPA_RANDOM_FIRST_SEED", "0"))
+
+
+@pytest.mark.parametrize("seed", range(_FIRST_SEED, _FIRST_SEED + _SEEDS))
+def test_random_batches_over_the_copies(gpu, seed):
+    """Seeded random ragged batches (12 by default, ``RPA_RANDOM_SEEDS`` widens the sweep) with the copies forced: every
+    seed draws its heads, page size, page format, a mix of decode rows, short and long chunks, whole prompts and empty
+    rows, and optionally sinks and a softmax scale."""
+    rng = np.random.default_rng(7000 + seed)
+    page_size, Hq, Hkv = [(64, 32, 8), (128, 40, 8), (64, 16, 1), (64, 8, 8), (192, 12, 4), (64, 24, 2)][seed % 6]
+    kv_dtype, scaled = [(FP8, True), (INT8, True), (FP8, False)][int(rng.integers(0, 3))]
+    n = int(rng.integers(1, 9))
+    kinds = rng.integers(0, 6, size=n)  # 0 decode, 1 a few tokens, 2 short chunk, 3 long chunk, 4 whole prompt, 5 no tokens
+    ctx, q_lens = [], []
+    for k in kinds:
+        if k == 0:
+            c = int(rng.integers(1, 3000)); q = 1
+        elif k == 1:
+            c = int(rng.integers(2, 2500)); q = int(rng.integers(2, min(c, 12) + 1))
+        elif k == 2:
+            c = int(rng.integers(50, 5000)); q = int(rng.integers(13, min(c, 200) + 1))
+        elif k == 3:
+            c = int(rng.integers(300, 6000)); q = int(rng.integers(200, min(c, 1200) + 1))
+        elif k == 4:
+            c = int(rng.integers(1, 1500)); q = c
+        else:
+            c = int(rng.integers(0, 500)); q = 0
+        ctx.append(c); q_lens.append(q)
+    if sum(q_lens) == 0:
+        q_lens[0], ctx[0] = 1, max(ctx[0], 1)
+    kw = {}
+    if rng.random() < 0.3:
+        kw["softmax_aux"] = rng.uniform(-3.0, 7.0, size=Hq).astype(np.float32)
+    if rng.random() < 0.3:
+        kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * 128 ** -0.5
+    b = tl.make_batch(7100 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=128, page_size=page_size, kv_dtype=kv_dtype, scaled=scaled,
+                      pad_rows=int(rng.integers(0, 3)), pad_tokens=int(rng.integers(0, 6)), shared_prefix_pages=int(rng.integers(0, 3)))
+    what = f"seed {seed}: pg{page_size} {Hq}/{Hkv} kv{kv_dtype}{'' if scaled else ' bare'} ctx {ctx} q {q_lens} {sorted(kw)}"
+    print(what, flush=True)
+    prev = _lib.set_tunable("prefill_wide", 2)
+    try:
+        got = tl.run_gpu_attention(b, **kw)
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
+    tl.assert_close(got, tl.oracle_out(b, **kw), b, what, one_ulp_above_4=True)
+    assert np.all(got[int(b.query_start_loc[b.n]):] == 0.0), "padded token rows must be written as zeros"
