@@ -671,8 +671,7 @@ def main():
     if args.workload == "c2" and args.layout == "interleaved" and not args.no_extra_configs:
         # the other benchmark configurations, each with its step time and its dominant kernel against its roofline
         # (no host leg for them); the headline fields above stay those of the decode configuration
-        extra = {}
-        for name in ("c3", "c4-fp8", "c4-int8", "c5-global", "c5-window"):
+        def record(name):
             r = measure(args, name, False)
             roof = r["roofline"]
             rec = {"workload": r["config"]["workload"], "ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"], "dtype": r["dtype"],
@@ -682,8 +681,12 @@ def main():
             for key in ("algorithmic_bytes_per_launch", "algorithmic_flops_per_launch"):
                 if key in roof:
                     rec[key.replace("_per_launch", "")] = roof[key]
-            extra[name] = rec
-        result["configs"] = extra
+            return rec
+
+        result["configs"] = {name: record(name) for name in ("c3", "c4-fp8", "c4-int8", "c5-global", "c5-window")}
+        # two shapes that are none of the benchmark's, in the same form: the prefill kernel on a batch that fills the chip,
+        # and prompt chunks over scaled fp8 pages (the prefill stage there: decision, page copy, the kernel on the copies)
+        result["tuning_shapes"] = {name: record(name) for name in ("llama-prefill", "fp8-prefill")}
     print(json.dumps(result))
 
 
