@@ -201,6 +201,50 @@ def test_long_context_prefill_over_eight_rounds_of_row_tiles(gpu):
     print(f"long-context prefill: worst max-abs {worst:.3e}", flush=True)
 
 
+@pytest.mark.parametrize("kv", ["fp8", "int8"])
+def test_quantised_prefill_full_size_reads_the_copies(gpu, kv):
+    # 4 x 2 048 prompt tokens behind 8k-16k tokens of scaled 8-bit pages, 40 query heads over 8 KV heads: by the library's
+    # own rule the chunks' pages are copied to bf16 once and the 32x32-tile kernel reads the copies; a slice of rows
+    # of every sequence against the oracle on the dequantised pages
+    from easydel_amd import _lib
+
+    w = workloads.quantised_long_prefill(seed=0, kv_dtype=kv)
+    tens = workloads.device_tensors(w, gpu, seed=0)
+    att = lambda: kernels.ragged_paged_attention(  # noqa: E731
+        tens["query"], tens["kv_pages"], tens["context_lens"], tens["block_tables"], tens["query_start_loc"], tens["num_seqs"],
+        softmax_scale=w.softmax_scale, kv_scales=tens["kv_scales"], num_kv_heads=w.Hkv)
+    out = att()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    prev = _lib.set_tunable("prefill_wide", 0)
+    try:
+        plain = att()
+        torch.cuda.synchronize()
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
+    assert not torch.equal(out, plain), "identical bits: the copies were not used"
+    assert (out.float() - plain.float()).abs().max().item() <= 2 * tl.TOL_BF16_MAX
+    G = w.Hq // w.Hkv
+    bf = lambda t: orc.bf16_bits_to_f32(t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)  # noqa: E731
+    worst = 0.0
+    for i in range(len(w.q_lens)):
+        r0 = (0, 2032, 1000, 517)[i % 4]
+        r1 = r0 + 16
+        ctx_rows = int(w.context_lens[i]) - int(w.q_lens[i]) + r1
+        n_pages = -(-ctx_rows // w.page_size)
+        ids = torch.from_numpy(w.block_tables[i, :n_pages].astype(np.int64)).to(gpu)
+        q0 = int(w.query_start_loc[i])
+        q, got = bf(tens["query"][q0 + r0:q0 + r1]), bf(out[q0 + r0:q0 + r1])
+        for h in range(w.Hkv):
+            vals = (tens["kv_pages"][ids][:, :, 2 * h:2 * h + 2].float() * tens["kv_scales"][ids][:, None, 2 * h:2 * h + 2, None]).double().cpu().numpy()
+            want = orc.ragged_paged_attention_ref(q[:, h * G:(h + 1) * G], vals, [ctx_rows], np.arange(n_pages)[None], [0, r1 - r0], [1],
+                                                  softmax_scale=w.softmax_scale, num_kv_heads=1)
+            err = np.abs(got[:, h * G:(h + 1) * G] - want)
+            assert err.max() <= tl.TOL_BF16_MAX and err.mean() <= tl.TOL_BF16_MEAN, (i, h, err.max(), err.mean())
+            worst = max(worst, err.max())
+    print(f"{kv} prefill through the copies: worst max-abs {worst:.3e}", flush=True)
+
+
 @pytest.mark.parametrize("Hq", [128, 16])
 def test_multi_latent_decode_at_benchmark_size(gpu, Hq):
     """256 sequences of 512..8192 tokens over latent pages (512 + 64, bf16), one new token each: the fused write is in
