@@ -45,8 +45,8 @@ struct Tunables {
   int prefill_dma = 1;
   int prefill_x32 = 1;     // 1: the 32x32-tile prefill kernel serves the shapes it is built for
   int prefill_wide = 1;    // 8-bit pages reach that kernel through bf16 copies where the workspace has room and the batch's rows pay for
-                           // them: 0 never, 1 at the default bar (kWideMinRows rows per copied page, a workgroup per CU), n > 1 at
-                           // a bar of n rows and none on the workgroups
+                           // them: 0 never, 1 at the default bars (kWideMinRows rows per copied page, kWideMinRowsFull in a batch
+                           // of two workgroups per CU), n > 1 at a bar of n rows
   int decode_pace = 1;
   int decode_dma = -1;     // -1: where it measured faster (head size 256; int8 pages); 0: never; 1: wherever it applies; 2: same, one tile ahead; 3: same, K with V
   int mla_chunks = 0;      // 0 = sized from the shapes
@@ -332,8 +332,10 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
 // most T group / (dec_rows + 1) of them, each with at most M pages -- capped at 4 GiB; 0 where the shapes rule the
 // copies out (other head sizes, pages that are not a multiple of 64 tokens, too few rows to pay for a copy).
 constexpr int64_t kWideMaxBytes = (int64_t)4 << 30;
-constexpr int kWideMinRows = 1024;  // the decision kernel's default bar: query rows per KV head and copied page, on the batch's average
-static int wide_min_rows(int tunable) { return tunable > 1 ? tunable : kWideMinRows; }
+// the decision kernel's default bars, in query rows per KV head and copied page on the batch's average: any batch, and a
+// batch of two workgroups of the 32x32-tile kernel per CU or more
+constexpr int kWideMinRows = 1792, kWideMinRowsFull = 1024;
+static int wide_min_rows(int tunable) { return tunable > 1 ? tunable : kWideMinRowsFull; }  // the lower of the two
 static int64_t wide_page_bytes(int page_size, int Hkv, int D) { return (int64_t)page_size * 2 * Hkv * D * 2; }
 static int64_t wide_header_bytes(int S) { return (((int64_t)(2 + S) * 4) + 255) & ~(int64_t)255; }
 static int64_t wide_pages_wanted(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int kv_dtype, int dec_rows, int min_rows) {
@@ -497,9 +499,10 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     bool wide = false;
     if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && !(p.softcap > 0.f) &&
         p.D == 128 && p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
-      p.wide_min_rows = wide_min_rows(tun.prefill_wide);
-      p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : device_cus();
-      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows, p.wide_min_rows);
+      p.wide_min_rows = tun.prefill_wide > 1 ? tun.prefill_wide : kWideMinRows;
+      p.wide_min_rows_full = wide_min_rows(tun.prefill_wide);
+      p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : 2 * device_cus();
+      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows, p.wide_min_rows_full);
       char* after = pre_base + pre;
       char* hdr = (char*)(((uintptr_t)after + 255) & ~(uintptr_t)255);
       char* pages0 = hdr + wide_header_bytes(S);

@@ -83,8 +83,9 @@ struct AttnParams {
   int wide_rows;       // pre_rows of a batch served from the copies
   int wide_slots;      // pre_slots likewise
   int src_P;           // pages of the 8-bit pool, for the kernel that reads the copies (its P is wide_cap)
-  int wide_min_rows;   // fewest query rows per KV head and copied page, on the batch's average, for the copies to be made
-  int wide_min_wgs;    // fewest workgroups (row tiles of wide_rows x KV heads) of the kernel that reads them
+  int wide_min_rows;   // fewest query rows per KV head and copied page, on the batch's average, for the copies to be made ...
+  int wide_min_rows_full;  // ... and the lower bar of a batch that gives the kernel that reads them wide_min_wgs
+  int wide_min_wgs;        // workgroups (row tiles of wide_rows x KV heads) or more
 };
 
 // Row-tile height and resident workgroups of the large-row kernel that serves this batch.

@@ -23,8 +23,9 @@ namespace rpa {
 
 // (AttnParams::wide_min_rows: the fewest query rows per KV head (tokens x group) per copied page, on the batch's average,
 // from which the copies pay -- a page costs 3 bytes per element to copy, and saves about a quarter of the matrix time
-// of every row tile that reads it.  AttnParams::wide_min_wgs: the fewest workgroups of the 32x32-tile kernel, whose row
-// tiles are twice as tall as the 8-bit kernel's and one to a CU: a batch of few row tiles fills the chip better there.)
+// of every row tile that reads it.  Measured at 5 query heads per KV head: chunks of 384 tokens and more win in batches
+// of one to sixteen chunks, chunks of 256 tokens only where the batch gives the 32x32-tile kernel, whose row tiles are
+// twice as tall as the 8-bit kernel's and one to a CU, two workgroups per CU: wide_min_rows_full, wide_min_wgs.)
 
 // wide[0] = 1 and wide[2 + i] = first copied page of sequence i if the large-row sequences' pages fit wide_cap and
 // their rows are worth it; else wide[0] = 0.  One workgroup of 256 threads.
@@ -76,8 +77,9 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
   const int all_fit = __syncthreads_and(fits ? 1 : 0);
   if (tid == 0) {
     const int total = s_carry;
-    const bool pays = total > 0 && s_work >= (unsigned long long)p.wide_min_rows * (unsigned)total &&
-                      (long long)s_tiles * p.Hkv >= p.wide_min_wgs;
+    const bool pays = total > 0 && (s_work >= (unsigned long long)p.wide_min_rows * (unsigned)total ||
+                                    (s_work >= (unsigned long long)p.wide_min_rows_full * (unsigned)total &&
+                                     (long long)s_tiles * p.Hkv >= p.wide_min_wgs));
     wide[0] = (all_fit && pays) ? 1 : 0;
     wide[1] = total;
   }

@@ -102,10 +102,10 @@ long long rpa_issue_probe(rpa_stream_t stream, int kind, int extra, int fill, in
  *   "prefill_wide"   1 (default): scaled or bare 8-bit pages of head size 128 (pages of a multiple of 64 tokens, no window, no
  *                    soft cap) reach that kernel through bf16 copies of the large-row sequences' pages, made once per
  *                    call in what the workspace holds beyond the partial rows, where a decision kernel finds that the
- *                    pages fit and that the batch has 1 024 query rows per KV head and copied page or more on average and a
- *                    workgroup of that kernel per CU or more (256 rows x KV heads); n > 1: the same with a bar of n
- *                    rows and none on the workgroups (tests, measurements); 0: never (set it before sizing the
- *                    workspace: the sizing call then asks for no room for copies)
+ *                    pages fit and that the batch has 1 792 query rows per KV head and copied page or more on average, or
+ *                    1 024 and two workgroups of that kernel per CU (256 rows x KV heads); n > 1: a single bar of n
+ *                    rows (tests, measurements); 0: never (set it before sizing the workspace: the sizing call then
+ *                    asks for no room for copies)
  *   "mla_chunks"     most key chunks one row tile of the multi-latent kernel is split into (1..16, 0 = sized from
  *                    the shapes, and batches of few row tiles cut by a chunk length chosen on the device from their
  *                    own lengths); set it before sizing the workspace

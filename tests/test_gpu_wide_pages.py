@@ -18,8 +18,8 @@ pytestmark = pytest.mark.gpu
 
 def _both(b, what, bar=2, **kw):
     """Output with the copies allowed, output with them switched off, both checked against the oracle.  ``bar`` is the
-    ``prefill_wide`` knob: 1 the library's rule (1 024 rows per KV head and copied page, a workgroup per CU), n > 1 a bar
-    of n rows and none on the workgroups -- the batches here are sized for the oracle, not for 256 CUs."""
+    ``prefill_wide`` knob: 1 the library's rule (1 792 rows per KV head and copied page, or 1 024 in a batch of two
+    workgroups per CU), n > 1 a single bar of n rows."""
     want = tl.oracle_out(b, **kw)
     prev = _lib.set_tunable("prefill_wide", bar)
     try:
@@ -72,8 +72,8 @@ def test_fp8_pages_without_scales_are_copied_exactly(gpu):
     _both(b, "copied pages, cast-only fp8")
 
 
-def test_the_librarys_rule_takes_a_batch_that_fills_the_chip(gpu):
-    """At the default setting: 37 row tiles of 256 rows x 8 KV heads, 4 000 rows per copied page."""
+def test_the_librarys_rule_takes_long_chunks(gpu):
+    """At the default setting: 4 000 rows per KV head and copied page on average."""
     b = tl.make_batch(917, [4000, 6000, 30], [900, 1300, 1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
     got, plain = _both(b, "copied pages by the library's rule", bar=1)
     assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
@@ -81,13 +81,14 @@ def test_the_librarys_rule_takes_a_batch_that_fills_the_chip(gpu):
 
 def test_batches_whose_rows_do_not_pay_stay_on_the_8bit_kernel(gpu):
     """Many short prompt chunks behind long contexts: copying every page would cost more than it saves; the decision
-    kernel says no and the result is the 8-bit kernel's, bit for bit -- by the rows per page at a bar of 1 024 rows, by
-    the number of workgroups at the library's rule.  Likewise under a window or a soft cap, which the copies do not serve."""
+    kernel says no and the result is the 8-bit kernel's, bit for bit -- at a bar of 1 024 rows, and at the library's
+    rule for a chunk of 1 200 rows that is far from filling the chip.  Likewise under a window or a soft cap, which the
+    copies do not serve."""
     b = tl.make_batch(914, [6000] * 8 + [50], [40] * 8 + [1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
     got, plain = _both(b, "short chunks behind long contexts", bar=1024)
     assert np.array_equal(got, plain)
-    b = tl.make_batch(918, [3000, 50], [500, 1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8)
-    got, plain = _both(b, "one chunk of eight row tiles", bar=1)
+    b = tl.make_batch(918, [3000, 50], [300, 1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8)
+    got, plain = _both(b, "one chunk of 1 200 rows", bar=1)
     assert np.array_equal(got, plain)
     b = tl.make_batch(915, [5000, 3000], [700, 600], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8)
     for kw in (dict(sliding_window=1000), dict(logits_soft_cap=30.0)):
