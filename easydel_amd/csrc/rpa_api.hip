@@ -340,7 +340,7 @@ static int64_t wide_page_bytes(int page_size, int Hkv, int D) { return (int64_t)
 static int64_t wide_header_bytes(int S) { return (((int64_t)(2 + S) * 4) + 255) & ~(int64_t)255; }
 static int64_t wide_pages_wanted(int T, int S, int M, int page_size, int Hq, int Hkv, int D, int kv_dtype, int dec_rows, int min_rows) {
   if (kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8) return 0;
-  if (D != 128 || page_size % 64 != 0 || S > 65535) return 0;
+  if ((D != 128 && D != 256) || page_size % 64 != 0 || S > 65535) return 0;
   const int64_t rows = (int64_t)T * (Hq / Hkv);
   if (rows <= min_rows) return 0;  // no batch of so few rows (T x group) holds a sequence that reaches the bar
   const int64_t seqs = std::min<int64_t>(S, rows / (dec_rows + 1));
@@ -498,7 +498,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     rpa::AttnParams pw;
     bool wide = false;
     if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && !(p.softcap > 0.f) &&
-        p.D == 128 && p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
+        (p.D == 128 || p.D == 256) && p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
       p.wide_min_rows = tun.prefill_wide > 1 ? tun.prefill_wide : kWideMinRows;
       p.wide_min_rows_full = wide_min_rows(tun.prefill_wide);
       p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : 2 * device_cus();
@@ -513,7 +513,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
         p.wide = (const int32_t*)hdr;
         p.wide_pages = pages0;
         p.wide_cap = (int)cap;
-        p.wide_rows = 256;
+        p.wide_rows = p.D == 128 ? 256 : 128;  // the 32x32-tile kernel's row tiles at this head size
         p.wide_slots = device_cus();
         p.src_P = P;
         pw = p;

@@ -822,7 +822,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
     const float sc = kq[C1], lv = lq[C1];
     const bool first_of_tile = SPT == 1 || PAR == 1;  // (b is even)
     if constexpr (KS) {
-      if (first_of_tile) {
+      if (first_of_tile && do_pv) {  // (a step past the last block issues no row sums: the last tile's stay for the epilogue)
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) asm volatile("s_nop 15\n\ts_nop 15" : "+a"(l_acc[rb]));  // the row sums may still be on their way
         fold_tile(lq[0]);
@@ -1068,8 +1068,8 @@ int prefill_x32_rows(const AttnParams& p) {
 
 int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p) {
   if (p.wide != nullptr) {  // bf16 copies of 8-bit pages
-    if (p.D != 128 || p.kv_dtype != RPA_BF16 || p.softcap > 0.f) return (int)hipErrorInvalidValue;
-    return launch_x32<128, 4, 2, RPA_BF16, false, true>(stream, p);
+    if ((p.D != 128 && p.D != 256) || p.kv_dtype != RPA_BF16 || p.softcap > 0.f) return (int)hipErrorInvalidValue;
+    return p.D == 256 ? launch_x32<256, 4, 1, RPA_BF16, false, true>(stream, p) : launch_x32<128, 4, 2, RPA_BF16, false, true>(stream, p);
   }
   if (p.D == 256) return p.softcap > 0.f ? launch_x32<256, 4, 1, RPA_BF16, true>(stream, p) : launch_x32<256, 4, 1, RPA_BF16, false>(stream, p);
   if (p.kv_dtype == RPA_F16) return launch_x32<128, 4, 2, RPA_F16, false>(stream, p);

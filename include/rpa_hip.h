@@ -126,7 +126,7 @@ int rpa_page_scatter_ragged_quantised(rpa_stream_t stream, const void* key, cons
  * as the kernels would like; an attention call accepts any workspace that holds two partial
  * slots (it reports RPA_ERR_WORKSPACE below that), lays the buffer out from the bytes it is
  * given and splits less when they are fewer, so the two calls cannot disagree.  For 8-bit
- * pages of head size 128 the figure also holds room for bf16 copies of the pages of prompt
+ * pages of head size 128 or 256 the figure also holds room for bf16 copies of the pages of prompt
  * chunks (two bytes per element of at most T * group / (rows per decode sequence + 1)
  * sequences of M pages, at most 4 GiB): with them a long chunk runs on the faster 16-bit
  * prefill kernel; a workspace without that room gives the same results from the 8-bit kernel.

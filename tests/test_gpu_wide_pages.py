@@ -38,17 +38,17 @@ def _both(b, what, bar=2, **kw):
 
 
 @pytest.mark.parametrize("kv_dtype", [FP8, INT8])
-@pytest.mark.parametrize("page_size,Hq,Hkv", [(64, 32, 8), (128, 40, 8), (64, 8, 1)])
-def test_long_prefill_over_scaled_8bit_pages_reads_the_copies(gpu, kv_dtype, page_size, Hq, Hkv):
+@pytest.mark.parametrize("page_size,Hq,Hkv,D", [(64, 32, 8, 128), (128, 40, 8, 128), (64, 8, 1, 128), (64, 16, 8, 256), (128, 8, 2, 256)])
+def test_long_prefill_over_scaled_8bit_pages_reads_the_copies(gpu, kv_dtype, page_size, Hq, Hkv, D):
     """Two long prefill chunks, a short one (large rows too: it is copied with them), decode sequences and an empty row;
     contexts that end inside a page, whose slots past the end hold NaN codes in the fp8 pool."""
-    b = tl.make_batch(900 + page_size + Hq, [5000, 1, 700, 9300, 333, 40], [700, 1, 1, 1100, 1, 40], Hq=Hq, Hkv=Hkv, D=128,
+    b = tl.make_batch(900 + page_size + Hq, [5000, 1, 700, 9300, 333, 40], [700, 1, 1, 1100, 1, 40], Hq=Hq, Hkv=Hkv, D=D,
                       page_size=page_size, kv_dtype=kv_dtype, pad_rows=2, pad_tokens=5)
     if kv_dtype == FP8:
         for i, c in enumerate(b.context_lens[:b.n]):
             if c % page_size:
                 b.kv_raw[b.block_tables[i, c // page_size], c % page_size:] = 0x7F
-    got, plain = _both(b, f"copied pages kv{kv_dtype} pg{page_size} Hq{Hq}/{Hkv}")
+    got, plain = _both(b, f"copied pages kv{kv_dtype} D{D} pg{page_size} Hq{Hq}/{Hkv}")
     rows = tl.valid_rows(b)
     assert np.abs(got - plain)[rows].max() <= 2 * tl.TOL_BF16_MAX
     assert (got[rows] != plain[rows]).any(), "the two kernels round differently: identical outputs mean the copies were not used"
@@ -207,7 +207,8 @@ def test_random_batches_over_the_copies(gpu, seed):
     seed draws its heads, page size, page format, a mix of decode rows, short and long chunks, whole prompts and empty
     rows, and optionally sinks and a softmax scale."""
     rng = np.random.default_rng(7000 + seed)
-    page_size, Hq, Hkv = [(64, 32, 8), (128, 40, 8), (64, 16, 1), (64, 8, 8), (192, 12, 4), (64, 24, 2)][seed % 6]
+    page_size, Hq, Hkv, D = [(64, 32, 8, 128), (128, 40, 8, 128), (64, 16, 1, 128), (64, 16, 8, 256), (64, 8, 8, 128), (192, 12, 4, 128),
+                             (64, 24, 2, 128), (128, 8, 2, 256)][seed % 8]
     kv_dtype, scaled = [(FP8, True), (INT8, True), (FP8, False)][int(rng.integers(0, 3))]
     n = int(rng.integers(1, 9))
     kinds = rng.integers(0, 6, size=n)  # 0 decode, 1 a few tokens, 2 short chunk, 3 long chunk, 4 whole prompt, 5 no tokens
@@ -232,10 +233,10 @@ def test_random_batches_over_the_copies(gpu, seed):
     if rng.random() < 0.3:
         kw["softmax_aux"] = rng.uniform(-3.0, 7.0, size=Hq).astype(np.float32)
     if rng.random() < 0.3:
-        kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * 128 ** -0.5
-    b = tl.make_batch(7100 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=128, page_size=page_size, kv_dtype=kv_dtype, scaled=scaled,
+        kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * D ** -0.5
+    b = tl.make_batch(7100 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype, scaled=scaled,
                       pad_rows=int(rng.integers(0, 3)), pad_tokens=int(rng.integers(0, 6)), shared_prefix_pages=int(rng.integers(0, 3)))
-    what = f"seed {seed}: pg{page_size} {Hq}/{Hkv} kv{kv_dtype}{'' if scaled else ' bare'} ctx {ctx} q {q_lens} {sorted(kw)}"
+    what = f"seed {seed}: D{D} pg{page_size} {Hq}/{Hkv} kv{kv_dtype}{'' if scaled else ' bare'} ctx {ctx} q {q_lens} {sorted(kw)}"
     print(what, flush=True)
     prev = _lib.set_tunable("prefill_wide", 2)
     try:
