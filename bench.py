@@ -36,7 +36,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=25,
                     help="untimed calls ahead of the timed ones (the first twenty or so calls of a workload run a few percent slower than the later ones)")
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill", "fp8-prefill", "int8-prefill", "int8-prefill-d256", "gemma-decode",
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4-fp8", "c4-int8", "c5-global", "c5-window", "llama-prefill", "fp8-prefill", "int8-prefill", "int8-prefill-d256", "int8-prefill-d256-cap", "gemma-decode",
                              "decode-hkv4", "decode-hkv1", "decode-16seq", "decode-32seq",
                              "mla-decode-h128", "mla-decode-h16", "mla-prefill-h128"])
     ap.add_argument("--layout", default="interleaved", choices=["interleaved", "unified"],
@@ -96,9 +96,9 @@ def build_workload(name, seed, sequential=False, chunks=(0, 0)):
         return workloads.config4_quantised_decode(seed, "fp8")
     if name == "c4-int8":
         return workloads.config4_quantised_decode(seed, "int8")
-    if name == "int8-prefill-d256":
+    if name in ("int8-prefill-d256", "int8-prefill-d256-cap"):
         kw = dict(n_seqs=chunks[0], q_len=chunks[1], num_pages=6000 if chunks[0] > 4 else 2000) if chunks[0] > 0 and chunks[1] > 0 else {}
-        return workloads.quantised_long_prefill(seed, "int8", head_dim=256, **kw)
+        return workloads.quantised_long_prefill(seed, "int8", head_dim=256, soft_cap=50.0 if name.endswith("-cap") else None, **kw)
     if name in ("fp8-prefill", "int8-prefill"):  # tuning shape for the 8-bit prefill kernel
         if chunks[0] > 0 and chunks[1] > 0:  # (6 000 pages hold 16 chunks of up to 16 384 tokens of context)
             return workloads.quantised_long_prefill(seed, name.split("-")[0], n_seqs=chunks[0], q_len=chunks[1], num_pages=6000 if chunks[0] > 4 else 2000)

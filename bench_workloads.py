@@ -206,18 +206,19 @@ def gemma_decode(seed: int = 0, n_seqs: int = 256, num_pages: int = 12_000) -> W
 
 
 def quantised_long_prefill(seed: int = 0, kv_dtype: str = "fp8", n_seqs: int = 4, q_len: int = 2048, num_pages: int = 2000,
-                           head_dim: int = 128) -> Workload:
+                           head_dim: int = 128, soft_cap: float | None = None) -> Workload:
     """Not one of the five benchmark shapes: chunked prefill over scaled 8-bit pages at the heads of the quantised decode
     configuration (40 query heads, 8 KV heads, head size 128, 64-token pages): ``n_seqs`` chunks of ``q_len`` tokens
     appended to 8192..16384 tokens of context.  Used to measure the 8-bit prefill kernel.  ``head_dim`` 256: the same at
-    16 query heads over 8 KV heads of 256 (a Gemma-shaped global-attention layer without soft cap)."""
+    16 query heads over 8 KV heads of 256 (a Gemma-shaped global-attention layer), with ``soft_cap`` or without."""
     rng = np.random.default_rng(seed)
     prior = rng.integers(8192 - q_len, 16385 - q_len, size=n_seqs)
     ctx = (prior + q_len).astype(np.int32)
     if head_dim == 256:
-        return Workload(f"Gemma-shaped (head size 256, no soft cap) {kv_dtype}-KV chunked prefill (tuning shape)", Hq=16, Hkv=8, D=256,
-                        page_size=64, num_pages=num_pages, max_pages_per_seq=256, context_lens=ctx, q_lens=np.full(n_seqs, q_len, dtype=np.int32),
-                        block_tables=_tables(rng, ctx, 64, num_pages, 256), kv_dtype=kv_dtype, softmax_scale=256.0 ** -0.5)
+        return Workload(f"Gemma-shaped (head size 256, {'soft cap %g' % soft_cap if soft_cap else 'no soft cap'}) {kv_dtype}-KV chunked prefill (tuning shape)",
+                        Hq=16, Hkv=8, D=256, page_size=64, num_pages=num_pages, max_pages_per_seq=256, context_lens=ctx,
+                        q_lens=np.full(n_seqs, q_len, dtype=np.int32), block_tables=_tables(rng, ctx, 64, num_pages, 256), kv_dtype=kv_dtype,
+                        softmax_scale=256.0 ** -0.5, logits_soft_cap=soft_cap)
     return Workload(f"Qwen2.5-32B-shaped {kv_dtype}-KV chunked prefill (tuning shape)", Hq=40, Hkv=8, D=128, page_size=64,
                     num_pages=num_pages, max_pages_per_seq=256, context_lens=ctx, q_lens=np.full(n_seqs, q_len, dtype=np.int32),
                     block_tables=_tables(rng, ctx, 64, num_pages, 256), kv_dtype=kv_dtype, softmax_scale=128.0 ** -0.5)

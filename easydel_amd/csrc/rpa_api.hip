@@ -497,8 +497,8 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     // and the 32x32-tile kernel reads those where the decision kernel finds that they fit and pay (rpa_widen.hip).
     rpa::AttnParams pw;
     bool wide = false;
-    if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && !(p.softcap > 0.f) &&
-        (p.D == 128 || p.D == 256) && p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
+    if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && (p.D == 256 || (p.D == 128 && !(p.softcap > 0.f))) &&
+        p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
       p.wide_min_rows = tun.prefill_wide > 1 ? tun.prefill_wide : kWideMinRows;
       p.wide_min_rows_full = wide_min_rows(tun.prefill_wide);
       p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : 2 * device_cus();

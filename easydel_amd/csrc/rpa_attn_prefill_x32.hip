@@ -129,7 +129,6 @@ __device__ __forceinline__ int swz_key_v32(int tok) {
 // operand of the row sums, is 2^-9 of an output: rows of a few keys then miss 2e-2 on outputs near 4.)
 template <int D, int NW, int RB, int HT, bool CAP, bool KS = false>
 __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p) {
-  static_assert(!(KS && CAP), "per-page key scales are not combined with a soft cap");
   using H = Half16<HT>;
   using W = Wide16<HT>;
   constexpr int BK = 32;                 // keys per block (what a step computes)
@@ -261,6 +260,9 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   //  not once per tile in scalar arithmetic; a page is a multiple of 64 rows of 16 bytes or more, the pool is below 2^40 bytes)
   const uint32_t page_units = (uint32_t)(p.page_stride >> 8);
   const float sc_mul = p.scale_log2;
+  // what a raw score is multiplied by first: the softmax scale in log2 units, or with a soft cap 2 log2(e) scale / cap
+  // (the argument of the exponential the hyperbolic tangent is made of); KS: times the K scale of the score's page
+  const float sc_unit = CAP ? (p.scale / p.softcap) * 2.8853900817779268f : sc_mul;
   int wide_first = 0;
   if constexpr (KS) wide_first = p.wide[2 + i];  // the sequence's copied pages follow one another
   auto page_offsets = [&](int col0) -> uint32_t {
@@ -270,12 +272,12 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   uint32_t pages_vec = page_offsets(col_base);
   // KS: beside them the score scale of each of the 64 columns (softmax scale x the K scale of the column's 8-bit page)
   // and the logarithm of its V scale; a tile's pair is taken when the tile is requested and queued until its steps.
-  float sck_vec = sc_mul, lvs_vec = 0.f;
+  float sck_vec = sc_unit, lvs_vec = 0.f;
   auto page_scales = [&](int col0) __attribute__((always_inline)) {
     if (p.kv_scales != nullptr) {
       const int id = min(max(bt_row[min(col0 + lane, p.M - 1)], 0), p.src_P - 1);
       const float2 kv = *(const float2*)(p.kv_scales + (int64_t)id * p.C + 2 * h);
-      sck_vec = sc_mul * fmaxf(kv.x, 1e-30f);
+      sck_vec = sc_unit * fmaxf(kv.x, 1e-30f);
       lvs_vec = __builtin_amdgcn_logf(fmaxf(kv.y, 1e-30f));  // log2
     }
   };
@@ -283,7 +285,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   float kq[KAH + 1], lq[KAH + 1];  // after barrier u: kq[c], lq[c] belong to tile u + c
 #pragma unroll
   for (int c = 0; c <= KAH; ++c) {
-    kq[c] = sc_mul;
+    kq[c] = sc_unit;
     lq[c] = 0.f;
   }
   int cur_col = col_base, cur_off = kv_lo - col_base * p.page_size, cur_tb = kv_lo;
@@ -447,10 +449,11 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   const float cap_in = CAP ? p.scale / p.softcap : 0.f;
   const float cap_in2 = cap_in * 2.8853900817779268f;
   const float cap_m2 = -2.f * cap_out;
-  auto capped = [&](float s) -> float { return cap_out * fast_tanh(s * cap_in); };  // a raw score to log2 units
+  // a raw score to log2 units (sc: what fast_step multiplies it by, cap_in2 or with KS cap_in2 x the page's K scale)
+  auto capped = [&](float s, float sc) -> float { return cap_out * fast_tanh(KS ? s * sc * 0.34657359027997264f : s * cap_in); };
   auto prob = [&](float s, float mn, float sc) __attribute__((always_inline)) -> float {
     if constexpr (CAP) {
-      const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s * cap_in2) + 1.f);
+      const float r = __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(s * (KS ? sc : cap_in2)) + 1.f);
       return s == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(__builtin_fmaf(r, cap_m2, mn));  // a masked key is not the cap's lower end
     } else {
       return __builtin_amdgcn_exp2f(__builtin_fmaf(s, sc, mn));
@@ -523,13 +526,14 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         const float raw = xor32_max(lmx[rb]);
-        const float mx = CAP ? (raw == -INFINITY ? -INFINITY : capped(raw)) : raw * sc;
+        const float mx = CAP ? (raw == -INFINITY ? -INFINITY : capped(raw, sc)) : raw * sc;
         const float m_new = fmaxf(m_ref[rb], ceilf(mx));
         float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref[rb] - m_new);  // a power of two, or 0
         m_ref[rb] = m_new;
         if constexpr (CAP) {  // the raw score whose capped value is m_new + slack, if there is one
           const float y = (m_new + kMaxSlack) / cap_out;
-          thr[rb] = (m_new == -INFINITY) ? -INFINITY : (y >= 0.999f ? INFINITY : 0.5f * __logf((1.f + y) / (1.f - y)) / cap_in);
+          const float ath = 0.5f * __logf((1.f + y) / (1.f - y));  // (KS: thr in units of raw score x sc)
+          thr[rb] = (m_new == -INFINITY) ? -INFINITY : (y >= 0.999f ? INFINITY : (KS ? ath * 2.8853900817779268f : ath / cap_in));
           m_neg[rb] = (m_new == -INFINITY) ? 0.f : cap_out - m_new;
         } else {
           thr[rb] = KS ? m_new + kMaxSlack : (m_new + kMaxSlack) * inv_sc;
@@ -643,8 +647,8 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
         } else {
           // four stages, one slot each; the last exponentials and the packing of a pair ride on the first two slots of the next
           if (st == 0) {
-            xa = s_cur[srb][2 * sr2] * cap_in2;
-            xb = s_cur[srb][2 * sr2 + 1] * cap_in2;
+            xa = s_cur[srb][2 * sr2] * (KS ? sc : cap_in2);
+            xb = s_cur[srb][2 * sr2 + 1] * (KS ? sc : cap_in2);
             if (ip > 0) {
               fa = __builtin_amdgcn_exp2f(ea);
               fb = __builtin_amdgcn_exp2f(eb);
@@ -1068,8 +1072,9 @@ int prefill_x32_rows(const AttnParams& p) {
 
 int launch_attn_prefill_x32(hipStream_t stream, const AttnParams& p) {
   if (p.wide != nullptr) {  // bf16 copies of 8-bit pages
-    if ((p.D != 128 && p.D != 256) || p.kv_dtype != RPA_BF16 || p.softcap > 0.f) return (int)hipErrorInvalidValue;
-    return p.D == 256 ? launch_x32<256, 4, 1, RPA_BF16, false, true>(stream, p) : launch_x32<128, 4, 2, RPA_BF16, false, true>(stream, p);
+    if ((p.D != 128 && p.D != 256) || p.kv_dtype != RPA_BF16 || (p.softcap > 0.f && p.D != 256)) return (int)hipErrorInvalidValue;
+    if (p.D == 256) return p.softcap > 0.f ? launch_x32<256, 4, 1, RPA_BF16, true, true>(stream, p) : launch_x32<256, 4, 1, RPA_BF16, false, true>(stream, p);
+    return launch_x32<128, 4, 2, RPA_BF16, false, true>(stream, p);
   }
   if (p.D == 256) return p.softcap > 0.f ? launch_x32<256, 4, 1, RPA_BF16, true>(stream, p) : launch_x32<256, 4, 1, RPA_BF16, false>(stream, p);
   if (p.kv_dtype == RPA_F16) return launch_x32<128, 4, 2, RPA_F16, false>(stream, p);

@@ -54,6 +54,16 @@ def test_long_prefill_over_scaled_8bit_pages_reads_the_copies(gpu, kv_dtype, pag
     assert (got[rows] != plain[rows]).any(), "the two kernels round differently: identical outputs mean the copies were not used"
 
 
+@pytest.mark.parametrize("kv_dtype", [FP8, INT8])
+def test_soft_cap_at_head_size_256_over_the_copies(gpu, kv_dtype):
+    """The soft cap's hyperbolic tangent takes the score scaled by the page's K scale (head size 256 only: at 128 the
+    32x32-tile kernel has no soft cap)."""
+    b = tl.make_batch(920, [4000, 333, 7000, 50], [600, 1, 900, 50], Hq=16, Hkv=8, D=256, page_size=128, kv_dtype=kv_dtype, pad_rows=1)
+    for cap in (50.0, 8.0):
+        got, plain = _both(b, f"copied pages kv{kv_dtype} D256, soft cap {cap}", logits_soft_cap=cap)
+        assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
+
+
 def test_key_chunks_over_the_copies(gpu):
     """One prompt chunk behind a long context: its row tiles are cut into key chunks and merged."""
     prev = _lib.set_tunable("prefill_chunks", 8)
@@ -82,8 +92,8 @@ def test_the_librarys_rule_takes_long_chunks(gpu):
 def test_batches_whose_rows_do_not_pay_stay_on_the_8bit_kernel(gpu):
     """Many short prompt chunks behind long contexts: copying every page would cost more than it saves; the decision
     kernel says no and the result is the 8-bit kernel's, bit for bit -- at a bar of 1 024 rows, and at the library's
-    rule for a chunk of 1 200 rows that is far from filling the chip.  Likewise under a window or a soft cap, which the
-    copies do not serve."""
+    rule for a chunk of 1 200 rows that is far from filling the chip.  Likewise under a window, or a soft cap at head
+    size 128, which the copies do not serve."""
     b = tl.make_batch(914, [6000] * 8 + [50], [40] * 8 + [1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
     got, plain = _both(b, "short chunks behind long contexts", bar=1024)
     assert np.array_equal(got, plain)
@@ -234,6 +244,8 @@ def test_random_batches_over_the_copies(gpu, seed):
         kw["softmax_aux"] = rng.uniform(-3.0, 7.0, size=Hq).astype(np.float32)
     if rng.random() < 0.3:
         kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * D ** -0.5
+    if D == 256 and rng.random() < 0.5:
+        kw["logits_soft_cap"] = float(rng.uniform(5.0, 60.0))
     b = tl.make_batch(7100 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype, scaled=scaled,
                       pad_rows=int(rng.integers(0, 3)), pad_tokens=int(rng.integers(0, 6)), shared_prefix_pages=int(rng.integers(0, 3)))
     what = f"seed {seed}: D{D} pg{page_size} {Hq}/{Hkv} kv{kv_dtype}{'' if scaled else ' bare'} ctx {ctx} q {q_lens} {sorted(kw)}"
