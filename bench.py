@@ -61,6 +61,7 @@ def parse_args():
     ap.add_argument("--prefill-wide", type=int, default=-1, help="bf16 copies of 8-bit pages for the 32x32-tile prefill kernel: -1 the library's choice, 0 never")
     ap.add_argument("--chunk-seqs", type=int, default=0, help="fp8-prefill / int8-prefill: this many prompt chunks (1..16) instead of 4 ...")
     ap.add_argument("--chunk-len", type=int, default=0, help="... of this many tokens instead of 2 048")
+    ap.add_argument("--chunk-window", type=int, default=0, help="the 8-bit prefill shapes under a sliding window of this many tokens")
     ap.add_argument("--mla-chunks", type=int, default=0)
     ap.add_argument("--mla-min-chunk", type=int, default=0)
     ap.add_argument("--mla-uniform-context", type=int, default=0,
@@ -457,6 +458,10 @@ def measure(args, workload, with_cpu):
 
     dev = torch.device("cuda:0")
     w = build_workload(workload, args.seed, args.sequential_pages, (args.chunk_seqs, args.chunk_len))
+    if args.chunk_window > 0 and workload in ("fp8-prefill", "int8-prefill", "int8-prefill-d256", "int8-prefill-d256-cap"):
+        import dataclasses
+
+        w = dataclasses.replace(w, sliding_window=args.chunk_window)
     tens = workloads.device_tensors(w, dev, seed=args.seed)
     quant = w.kv_dtype in ("fp8", "int8")
     out = torch.empty_like(tens["query"])

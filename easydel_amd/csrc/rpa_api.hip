@@ -497,11 +497,12 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
     // and the 32x32-tile kernel reads those where the decision kernel finds that they fit and pay (rpa_widen.hip).
     rpa::AttnParams pw;
     bool wide = false;
-    if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && p.window == 0 && (p.D == 256 || (p.D == 128 && !(p.softcap > 0.f))) &&
+    if (tun.prefill_wide && tun.prefill_dma && tun.prefill_x32 && (p.D == 256 || (p.D == 128 && !(p.softcap > 0.f))) &&
         p.kv_pad_bytes == 0 && rpa::prefill_dma8_supported(p)) {
       p.wide_min_rows = tun.prefill_wide > 1 ? tun.prefill_wide : kWideMinRows;
       p.wide_min_rows_full = wide_min_rows(tun.prefill_wide);
       p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : 2 * device_cus();
+      p.wide_min_window = tun.prefill_wide > 1 ? 0 : 2048;
       const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows, p.wide_min_rows_full);
       char* after = pre_base + pre;
       char* hdr = (char*)(((uintptr_t)after + 255) & ~(uintptr_t)255);

@@ -264,7 +264,7 @@ __global__ __launch_bounds__(64 * NW) void attn_prefill_x32_kernel(AttnParams p)
   // (the argument of the exponential the hyperbolic tangent is made of); KS: times the K scale of the score's page
   const float sc_unit = CAP ? (p.scale / p.softcap) * 2.8853900817779268f : sc_mul;
   int wide_first = 0;
-  if constexpr (KS) wide_first = p.wide[2 + i];  // the sequence's copied pages follow one another
+  if constexpr (KS) wide_first = p.wide[2 + i];  // the sequence's copied pages follow one another: column c is page wide_first + c
   auto page_offsets = [&](int col0) -> uint32_t {
     if constexpr (KS) return (uint32_t)min(max(wide_first + col0 + lane, 0), p.P - 1) * page_units;
     else return (uint32_t)min(max(bt_row[min(col0 + lane, p.M - 1)], 0), p.P - 1) * page_units;

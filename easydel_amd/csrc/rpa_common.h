@@ -76,7 +76,8 @@ struct AttnParams {
   int mfma_path;     // 1: bf16 queries served by the MFMA kernels; 0: fp32 VALU kernel serves every row
   // 8-bit pages whose large-row sequences may be served from bf16 copies of their pages (null: never).  Written by the
   // decision kernel ahead of the plan: [0] = 1 if this batch is served that way, [1] = copied pages in use,
-  // [2 + i] = first copied page of sequence i (its pages follow in block-table order).
+  // [2 + i] = the copied page of block-table column 0 of sequence i, were it copied (the visible columns follow in
+  // block-table order; under a sliding window the first ones are not copied and this is below zero).
   const int32_t* wide;
   void* wide_pages;    // the copies: [wide_cap][page_size][2 Hkv][D] bf16, bare codes, K of head h at row 2h, V at 2h + 1
   int wide_cap;        // pages the copies hold
@@ -86,6 +87,7 @@ struct AttnParams {
   int wide_min_rows;   // fewest query rows per KV head and copied page, on the batch's average, for the copies to be made ...
   int wide_min_rows_full;  // ... and the lower bar of a batch that gives the kernel that reads them wide_min_wgs
   int wide_min_wgs;        // workgroups (row tiles of wide_rows x KV heads) or more
+  int wide_min_window;     // under a sliding window: the shortest window, and wide_min_wgs workgroups, for the copies to be made
 };
 
 // Row-tile height and resident workgroups of the large-row kernel that serves this batch.

@@ -27,8 +27,10 @@ namespace rpa {
 // of one to sixteen chunks, chunks of 256 tokens only where the batch gives the 32x32-tile kernel, whose row tiles are
 // twice as tall as the 8-bit kernel's and one to a CU, two workgroups per CU: wide_min_rows_full, wide_min_wgs.)
 
-// wide[0] = 1 and wide[2 + i] = first copied page of sequence i if the large-row sequences' pages fit wide_cap and
-// their rows are worth it; else wide[0] = 0.  One workgroup of 256 threads.
+// wide[0] = 1 and wide[2 + i] = where block-table column 0 of sequence i would lie among the copied pages (its first
+// copied page less its first visible column: below zero under a sliding window, whose earlier pages are not copied) if
+// the large-row sequences' visible pages fit wide_cap and their rows are worth it; else wide[0] = 0.  One workgroup of
+// 256 threads.
 __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t* wide) {
   __shared__ int s_scan[256];
   __shared__ int s_carry;
@@ -47,12 +49,14 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
   bool fits = true;
   for (int i0 = 0; i0 < p.S; i0 += 256) {  // (uniform trip count)
     const int i = i0 + tid;
-    int need = 0;
+    int need = 0, col_lo = 0;
     if (i < n_live) {
       const SeqPlan sp = seq_plan(p, i);
       if (sp.live && !sp.small_rows) {
-        need = (sp.ctx + p.page_size - 1) / p.page_size;
-        work += (unsigned long long)need * (unsigned)(sp.q_len * p.group);
+        col_lo = sp.lo / p.page_size;  // (sp.lo: the first key any row of the sequence sees, rounded down to 64)
+        need = (sp.ctx + p.page_size - 1) / p.page_size - col_lo;
+        const int readers = p.window > 0 ? min(sp.q_len, p.window + p.page_size) : sp.q_len;  // tokens that see a page, at most
+        work += (unsigned long long)need * (unsigned)(readers * p.group);
         tiles += (sp.q_len * p.group + p.wide_rows - 1) / p.wide_rows;
       }
     }
@@ -66,7 +70,7 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
     }
     const int carry = s_carry;
     const long long first = (long long)carry + s_scan[tid] - need;
-    if (i < p.S) wide[2 + i] = first + need <= p.wide_cap ? (int)first : 0;
+    if (i < p.S) wide[2 + i] = first + need <= p.wide_cap ? (int)first - col_lo : 0;
     if (first + need > p.wide_cap) fits = false;
     __syncthreads();
     if (tid == 255) s_carry = (int)min((long long)carry + s_scan[255], (long long)0x3fffffff);
@@ -77,15 +81,18 @@ __global__ __launch_bounds__(256) void widen_decide_kernel(AttnParams p, int32_t
   const int all_fit = __syncthreads_and(fits ? 1 : 0);
   if (tid == 0) {
     const int total = s_carry;
-    const bool pays = total > 0 && (s_work >= (unsigned long long)p.wide_min_rows * (unsigned)total ||
-                                    (s_work >= (unsigned long long)p.wide_min_rows_full * (unsigned)total &&
-                                     (long long)s_tiles * p.Hkv >= p.wide_min_wgs));
+    const bool rows_high = s_work >= (unsigned long long)p.wide_min_rows * (unsigned)total;
+    const bool rows_low = s_work >= (unsigned long long)p.wide_min_rows_full * (unsigned)total;
+    const bool full = (long long)s_tiles * p.Hkv >= p.wide_min_wgs;
+    // (under a window a row tile's key range is short, and the 32x32-tile kernel's start and end weigh more: measured, the
+    //  copies win at a window of 4 096 on a full chip, and lose by 4-6 % at a window of 1 024 or on 320 workgroups)
+    const bool pays = total > 0 && (p.window > 0 ? rows_high && full && p.window >= p.wide_min_window : rows_high || (rows_low && full));
     wide[0] = (all_fit && pays) ? 1 : 0;
     wide[1] = total;
   }
 }
 
-// Pages j = blockIdx.x, blockIdx.x + gridDim.x, ... of sequence blockIdx.y: 16 codes per thread and turn.
+// Visible pages j = first visible + blockIdx.x, + gridDim.x, ... of sequence blockIdx.y: 16 codes per thread and turn.
 template <int KVT>
 __global__ __launch_bounds__(256) void widen_pages_kernel(AttnParams p) {
   if (!wide_mode(p)) return;
@@ -98,8 +105,8 @@ __global__ __launch_bounds__(256) void widen_pages_kernel(AttnParams p) {
   const int CH = p.D / 16;              // 16-code pieces of a head's row
   const int per_tok = 2 * p.Hkv * CH;   // pieces of a token: K and V of every head
   const int64_t dst_tok = (int64_t)2 * p.Hkv * p.D * 2, dst_page = dst_tok * p.page_size;
-  for (int j = blockIdx.x; j < n_pages; j += gridDim.x) {
-    if (first + j >= p.wide_cap) return;  // (the decision kernel has made sure of this)
+  for (int j = sp.lo / p.page_size + blockIdx.x; j < n_pages; j += gridDim.x) {
+    if (first + j < 0 || first + j >= p.wide_cap) return;  // (the decision kernel has made sure of this)
     const int page = min(max(p.block_tables[(int64_t)i * p.M + j], 0), p.P - 1);
     const int n_tok = min(p.page_size, sp.ctx - j * p.page_size);  // rows past the context are never read
     char* dst = (char*)p.wide_pages + (int64_t)(first + j) * dst_page;

@@ -99,8 +99,9 @@ long long rpa_issue_probe(rpa_stream_t stream, int kind, int extra, int fill, in
  *   "prefill_x32"    1 (default): pages of a multiple of 64 tokens take the prefill kernel built on 32x32x16 tiles, one
  *                    workgroup per CU, at head size 128 (bf16 / float16 pages, no soft cap: 256-row workgroups) and at
  *                    head size 256 (bf16 pages, with or without soft cap: 128-row workgroups); 0: never
- *   "prefill_wide"   1 (default): scaled or bare 8-bit pages of head size 128 or 256 (pages of a multiple of 64 tokens, no window, a
- *                    soft cap at head size 256 only) reach that kernel through bf16 copies of the large-row sequences' pages, made once per
+ *   "prefill_wide"   1 (default): scaled or bare 8-bit pages of head size 128 or 256 (pages of a multiple of 64 tokens, a soft cap at
+ *                    head size 256 only; under a sliding window only from 2 048 tokens of window and two workgroups
+ *                    per CU on) reach that kernel through bf16 copies of the large-row sequences' pages, made once per
  *                    call in what the workspace holds beyond the partial rows, where a decision kernel finds that the
  *                    pages fit and that the batch has 1 792 query rows per KV head and copied page or more on average, or
  *                    1 024 and two workgroups of that kernel per CU (256 rows x KV heads); n > 1: a single bar of n

@@ -92,8 +92,8 @@ def test_the_librarys_rule_takes_long_chunks(gpu):
 def test_batches_whose_rows_do_not_pay_stay_on_the_8bit_kernel(gpu):
     """Many short prompt chunks behind long contexts: copying every page would cost more than it saves; the decision
     kernel says no and the result is the 8-bit kernel's, bit for bit -- at a bar of 1 024 rows, and at the library's
-    rule for a chunk of 1 200 rows that is far from filling the chip.  Likewise under a window, or a soft cap at head
-    size 128, which the copies do not serve."""
+    rule for a chunk of 1 200 rows that is far from filling the chip.  Likewise under a soft cap at head size 128, which
+    the copies do not serve."""
     b = tl.make_batch(914, [6000] * 8 + [50], [40] * 8 + [1], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
     got, plain = _both(b, "short chunks behind long contexts", bar=1024)
     assert np.array_equal(got, plain)
@@ -101,9 +101,23 @@ def test_batches_whose_rows_do_not_pay_stay_on_the_8bit_kernel(gpu):
     got, plain = _both(b, "one chunk of 1 200 rows", bar=1)
     assert np.array_equal(got, plain)
     b = tl.make_batch(915, [5000, 3000], [700, 600], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=FP8)
-    for kw in (dict(sliding_window=1000), dict(logits_soft_cap=30.0)):
-        got, plain = _both(b, f"copies not offered with {sorted(kw)}", **kw)
-        assert np.array_equal(got, plain)
+    got, plain = _both(b, "copies not offered with a soft cap at head size 128", logits_soft_cap=30.0)
+    assert np.array_equal(got, plain)
+
+
+@pytest.mark.parametrize("kv_dtype", [FP8, INT8])
+@pytest.mark.parametrize("D,page_size,Hq,Hkv,window,cap", [(128, 64, 32, 8, 777, None), (128, 128, 40, 8, 3000, None), (256, 64, 16, 8, 1500, 50.0),
+                                                            (128, 64, 8, 1, 64, None)])
+def test_sliding_window_over_the_copies(gpu, kv_dtype, D, page_size, Hq, Hkv, window, cap):
+    """Under a window only the pages some row of the chunk can see are copied: the first copied page of a sequence is the
+    page of its first visible key, wherever that falls inside a page."""
+    b = tl.make_batch(930 + window, [5000, 1, 9300, 700, 40], [700, 1, 1100, 300, 40], Hq=Hq, Hkv=Hkv, D=D, page_size=page_size,
+                      kv_dtype=kv_dtype, pad_rows=1, pad_tokens=2)
+    kw = dict(sliding_window=window)
+    if cap:
+        kw["logits_soft_cap"] = cap
+    got, plain = _both(b, f"copied pages kv{kv_dtype} D{D} pg{page_size} window {window} cap {cap}", **kw)
+    assert (got[tl.valid_rows(b)] != plain[tl.valid_rows(b)]).any()
 
 
 def test_a_workspace_without_room_for_the_copies_falls_back(gpu, monkeypatch):
@@ -246,6 +260,8 @@ def test_random_batches_over_the_copies(gpu, seed):
         kw["softmax_scale"] = float(rng.uniform(0.5, 1.5)) * D ** -0.5
     if D == 256 and rng.random() < 0.5:
         kw["logits_soft_cap"] = float(rng.uniform(5.0, 60.0))
+    if rng.random() < 0.35:
+        kw["sliding_window"] = int(rng.integers(1, 3000))
     b = tl.make_batch(7100 + seed, ctx, q_lens, Hq=Hq, Hkv=Hkv, D=D, page_size=page_size, kv_dtype=kv_dtype, scaled=scaled,
                       pad_rows=int(rng.integers(0, 3)), pad_tokens=int(rng.integers(0, 6)), shared_prefix_pages=int(rng.integers(0, 3)))
     what = f"seed {seed}: D{D} pg{page_size} {Hq}/{Hkv} kv{kv_dtype}{'' if scaled else ' bare'} ctx {ctx} q {q_lens} {sorted(kw)}"
