@@ -46,6 +46,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-configs", action="store_true",
                     help="default workload only: do not measure the other benchmark configurations afterwards")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="also time the step recorded once in a HIP graph and replayed (ms_per_step_hip_graph)")
     ap.add_argument("--mfma-probe", action="store_true",
                     help="instead of a workload: the library's matrix-core feed probe (bf16 MFMA streams with operands from "
                          "registers or LDS, both tile shapes, 1 / 2 / 4 MFMAs per operand, one and two waves per SIMD), one line per setting")
@@ -521,6 +523,29 @@ def measure(args, workload, with_cpu):
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # the same step recorded once in a HIP graph and replayed: what a serving loop that captures its decode step pays
+    # (the library's launches are plain kernels on the caller's stream; its workspace was sized by the calls above)
+    graph_ms = None
+    if args.hip_graph:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        del graph
+
     # kernels in isolation: one call that only runs the plan kernel, then calls that launch only the decode
     # kernel (it reuses the plan left in the workspace) or only the prefill kernel, bracketed by events on the
     # launch stream
@@ -585,6 +610,7 @@ def measure(args, workload, with_cpu):
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_hip_graph": graph_ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
