@@ -342,7 +342,9 @@ static int64_t wide_pages_wanted(int T, int S, int M, int page_size, int Hq, int
   if (kv_dtype != RPA_FP8_E4M3 && kv_dtype != RPA_INT8) return 0;
   if ((D != 128 && D != 256) || page_size % 64 != 0 || S > 65535) return 0;
   const int64_t rows = (int64_t)T * (Hq / Hkv);
-  if (rows <= min_rows) return 0;  // no batch of so few rows (T x group) holds a sequence that reaches the bar
+  // No batch of fewer rows (T x group) in all is served from copies: the upper bar is an average, so some sequence
+  // reaches it; the lower bar counts only with two workgroups of 128 or 256 rows per CU, many times as many rows.
+  if (rows < min_rows) return 0;
   const int64_t seqs = std::min<int64_t>(S, rows / (dec_rows + 1));
   return std::min<int64_t>(seqs * M, kWideMaxBytes / wide_page_bytes(page_size, Hkv, D));
 }
@@ -359,7 +361,8 @@ size_t rpa_attention_workspace_bytes(int T, int S, int M, int page_size, int Hq,
   const size_t pre = pre_chunks > 1 ? (size_t)pre_chunks * (part_o_bytes(T, Hq, D) + part_ml_bytes(T, Hq)) : 0;
   size_t wide = 0;
   if (g_tun.prefill_wide && g_tun.prefill_dma && g_tun.prefill_x32) {
-    const int64_t pages = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, D, kv_dtype, rpa::decode_row_limit(T, S, D, kv_dtype), wide_min_rows(g_tun.prefill_wide));
+    const int64_t pages = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, D, kv_dtype, rpa::decode_row_limit(T, S, D, kv_dtype),
+                                            g_tun.prefill_wide > 1 ? g_tun.prefill_wide : kWideMinRows);
     if (pages > 0) wide = (size_t)(wide_header_bytes(S) + pages * wide_page_bytes(page_size, Hkv, D) + 256);
   }
   return (size_t)splits * (part_o_bytes(td, Hq, D) + part_ml_bytes(td, Hq)) + pre + plan_bytes(S) + 256 + wide;
@@ -503,7 +506,7 @@ static int attention_impl(const char* who, rpa_stream_t stream, const void* q, c
       p.wide_min_rows_full = wide_min_rows(tun.prefill_wide);
       p.wide_min_wgs = tun.prefill_wide > 1 ? 0 : 2 * device_cus();
       p.wide_min_window = tun.prefill_wide > 1 ? 0 : 2048;
-      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows, p.wide_min_rows_full);
+      const int64_t want = wide_pages_wanted(T, S, M, page_size, Hq, Hkv, p.D, kv_dtype, p.dec_rows, p.wide_min_rows);
       char* after = pre_base + pre;
       char* hdr = (char*)(((uintptr_t)after + 255) & ~(uintptr_t)255);
       char* pages0 = hdr + wide_header_bytes(S);

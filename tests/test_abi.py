@@ -99,6 +99,36 @@ def test_host_only_entry_points():
     assert lib.rpa_issue_probe(None, 10, 1, 6, 100, a, a, a) == 0  # kinds 0..9
 
 
+def test_workspace_sizing_asks_for_page_copies_only_where_a_call_could_use_them():
+    """8-bit pages: the sizing call adds room for bf16 copies of prompt chunks' pages -- for the sequences that can have
+    large rows, M pages each -- and nothing for a pure-decode bucket, 16-bit pages, head sizes the kernel on the copies
+    does not serve, pages that are not a multiple of 64 tokens, or with the copies switched off."""
+    lib = _lib.load()
+    f = lib.rpa_attention_workspace_bytes  # (T, S, M, page_size, Hq, Hkv, D, q_dtype, kv_dtype)
+    BF16, FP8, INT8 = 1, 2, 3
+
+    def room(*shape):  # what the copies add: the figure with them less the figure with them switched off
+        with_copies = f(*shape)
+        prev = _lib.set_tunable("prefill_wide", 0)
+        try:
+            return with_copies - f(*shape)
+        finally:
+            _lib.set_tunable("prefill_wide", prev)
+
+    page16 = 64 * 2 * 8 * 128 * 2
+    for kv in (FP8, INT8):
+        assert 4 * 256 * page16 <= room(8192, 4, 256, 64, 40, 8, 128, BF16, kv) < 4 * 256 * page16 + (1 << 16)  # 4 sequences x 256 pages
+        assert room(256, 256, 128, 64, 40, 8, 128, BF16, kv) == 0   # 1 280 rows per KV head in all: a pure-decode bucket
+        assert room(8192, 4, 256, 32, 40, 8, 128, BF16, kv) == 0   # 32-token pages
+        assert room(8192, 4, 256, 64, 8, 8, 64, BF16, kv) == 0     # head size 64
+        assert room(8192, 4, 256, 64, 16, 8, 256, BF16, kv) >= 4 * 256 * 2 * page16  # head size 256
+    assert room(8192, 4, 256, 64, 40, 8, 128, BF16, BF16) == 0
+    # many sequences, few tokens: not all of them can have large rows (more than 16 or 32 rows per KV head each)
+    assert 0 < room(2048, 512, 16, 64, 32, 8, 128, BF16, INT8) <= (2048 * 4 // 17) * 16 * page16 + (1 << 16) < 512 * 16 * page16
+    # capped at 4 GiB
+    assert room(65536, 512, 4096, 64, 32, 8, 128, BF16, INT8) <= (4 << 30) + (1 << 16)
+
+
 def test_product_build_has_no_probes_and_no_stage_knob(tmp_path):
     """The API source compiled without -DRPA_PROBES (what `python -m easydel_amd.build --product` links) neither defines
     the measurement entry points nor knows the knobs that change what a call computes with."""
