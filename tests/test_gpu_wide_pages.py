@@ -273,3 +273,45 @@ def test_random_batches_over_the_copies(gpu, seed):
         _lib.set_tunable("prefill_wide", prev)
     tl.assert_close(got, tl.oracle_out(b, **kw), b, what, one_ulp_above_4=True)
     assert np.all(got[int(b.query_start_loc[b.n]):] == 0.0), "padded token rows must be written as zeros"
+
+
+def test_a_call_over_the_copies_replays_from_a_hip_graph(gpu):
+    """The decision, the copy and the kernel on the copies are plain launches on the caller's stream: recorded once in a
+    graph, every replay gives the eager result, also with the program's own work and synchronisations in between, and
+    metadata changed in place (a shorter context) is picked up by the next replay."""
+    b = tl.make_batch(950, [4000, 300, 2500], [900, 1, 600], Hq=32, Hkv=8, D=128, page_size=64, kv_dtype=INT8)
+    d = tl.device_batch(b)
+    out = torch.empty_like(d["query"])
+
+    def call():
+        kernels.ragged_paged_attention(d["query"], d["kv_pages"], d["context_lens"], d["block_tables"], d["query_start_loc"], d["num_seqs"],
+                                       kv_scales=d["kv_scales"], num_kv_heads=b.Hkv, out=out)
+
+    prev = _lib.set_tunable("prefill_wide", 2)
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            call()  # warm-up on the capture stream: sizes the cached workspace outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        eager = out.clone()
+        tl.assert_close(tl.from_torch(eager, tl.BF16), tl.oracle_out(b), b, "eager call over the copies", one_ulp_above_4=True)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            call()
+        for rep in range(4):
+            out.zero_()
+            d["query"].mul_(1.0)  # eager work between replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), f"replay {rep} differs from the eager result"
+        d["context_lens"][0] = 3500  # the first chunk now ends 500 tokens earlier: fewer pages to copy, other rows to mask
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        b.context_lens[0] = 3500
+        tl.assert_close(tl.from_torch(out, tl.BF16), tl.oracle_out(b), b, "graph replay with new metadata", one_ulp_above_4=True)
+    finally:
+        _lib.set_tunable("prefill_wide", prev)
