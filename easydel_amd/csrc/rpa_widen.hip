@@ -12,7 +12,9 @@
 //
 // Two kernels: the decision (one workgroup, ahead of the plan kernel, which cuts row tiles at the height of whichever
 // kernel serves the batch) and the copy (behind the plan kernel's launch, which may write the step's new rows into the
-// pages).  The decision is all or nothing per batch: the plan and merge kernels work with one row-tile height.
+// pages).  The decision is all or nothing per batch: the plan and merge kernels work with one row-tile height, and a
+// batch split between the two large-row kernels, one launched behind the other, leaves the chip half empty twice
+// (measured slower than either kernel alone on chunks of mixed lengths).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
